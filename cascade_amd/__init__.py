@@ -1,0 +1,9 @@
+"""cascade_amd: MI355X (gfx950) per-partition suffix sort by prefix doubling, behind a C ABI.
+
+The compute lives in libcascade_hip.so (hand-written HIP, include/cascade_hip.h); this package is the thin
+host-side mirror of the reference's builder interface for that one path.
+"""
+from . import _native, workloads
+from .gpu_saca import GPU_SACA, PartitionSorter, pack_keys, sort_partition
+
+__all__ = ["GPU_SACA", "PartitionSorter", "pack_keys", "sort_partition", "workloads", "_native"]

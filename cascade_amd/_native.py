@@ -1,0 +1,85 @@
+"""ctypes bindings of the C ABI declared in include/cascade_hip.h.
+
+There is no CPU fallback: if the HIP library has not been built, loading fails with an error that says so.
+"""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+HIP_LIB_PATH = os.path.join(HERE, "libcascade_hip.so")
+
+CSA_MAX_GENERATIONS = 64
+CSA_MAX_PART_SZ = 2147483647
+CSA_MAX_INDEX = 1 << 40
+CSA_OK, CSA_ERR_ARG, CSA_ERR_TOO_LARGE, CSA_ERR_HIP, CSA_ERR_INTERNAL = 0, -1, -2, -3, -4
+CSA_FLAG_KERNEL_TIMING = 1
+
+# every symbol include/cascade_hip.h declares
+EXPORTS = (
+    "csa_bytes_per_suffix", "csa_create", "csa_destroy", "csa_sort_partition_u16_dev", "csa_sort_partition_u16",
+    "csa_pack_keys_u16_dev", "csa_radix_sort_pairs_dev", "csa_verify_sa40_dev", "csa_last_error",
+)
+
+
+class CsaStats(C.Structure):
+    _fields_ = [
+        ("n", C.c_uint64),
+        ("key_words", C.c_int32),
+        ("generations", C.c_int32),
+        ("active", C.c_uint64 * CSA_MAX_GENERATIONS),
+        ("groups", C.c_uint64 * CSA_MAX_GENERATIONS),
+        ("passes", C.c_int32 * CSA_MAX_GENERATIONS),
+        ("ms", C.c_float * CSA_MAX_GENERATIONS),
+        ("ms_output", C.c_float),
+        ("ms_total", C.c_float),
+        ("radix_launches", C.c_uint64),
+        ("radix_pairs", C.c_uint64),
+        ("radix_ms", C.c_double),
+    ]
+
+
+class CascadeError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__(f"cascade_hip status {status}: {message}")
+        self.status = status
+
+
+_lib = None
+
+
+def load():
+    """Loads libcascade_hip.so and declares its prototypes. Raises if the library is missing."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(HIP_LIB_PATH):
+        raise ImportError(
+            f"{HIP_LIB_PATH} is missing: build it with `python -m cascade_amd.build` "
+            "(there is no CPU fallback for the partition sort)")
+    lib = C.CDLL(HIP_LIB_PATH)
+    vp, u64, u32, i32 = C.c_void_p, C.c_uint64, C.c_uint32, C.c_int
+    lib.csa_bytes_per_suffix.restype = u64
+    lib.csa_bytes_per_suffix.argtypes = [i32]
+    lib.csa_create.restype = i32
+    lib.csa_create.argtypes = [u64, i32, C.POINTER(vp)]
+    lib.csa_destroy.restype = None
+    lib.csa_destroy.argtypes = [vp]
+    lib.csa_sort_partition_u16_dev.restype = i32
+    lib.csa_sort_partition_u16_dev.argtypes = [vp, vp, u64, u64, vp, vp, u32, C.POINTER(CsaStats)]
+    lib.csa_sort_partition_u16.restype = i32
+    lib.csa_sort_partition_u16.argtypes = [vp, u64, i32, vp, C.POINTER(CsaStats)]
+    lib.csa_pack_keys_u16_dev.restype = i32
+    lib.csa_pack_keys_u16_dev.argtypes = [vp, u64, i32, vp, vp]
+    lib.csa_radix_sort_pairs_dev.restype = i32
+    lib.csa_radix_sort_pairs_dev.argtypes = [vp, vp, vp, u64, i32, i32, vp]
+    lib.csa_verify_sa40_dev.restype = i32
+    lib.csa_verify_sa40_dev.argtypes = [vp, vp, u64, u64, vp, vp, C.POINTER(i32)]
+    lib.csa_last_error.restype = C.c_char_p
+    lib.csa_last_error.argtypes = []
+    _lib = lib
+    return lib
+
+
+def check(status):
+    if status != CSA_OK:
+        raise CascadeError(status, load().csa_last_error().decode())

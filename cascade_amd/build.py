@@ -1,0 +1,49 @@
+"""Compiles the native libraries of this package in-tree.
+
+  libcascade_hip.so        hand-written HIP for gfx950 behind the C ABI of include/cascade_hip.h
+  libcascade_workloads.so  host-only generator of the synthetic benchmark partitions
+
+Run as `python -m cascade_amd.build`. hipcc cross-compiles for gfx950 without a GPU.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+HIP_LIB = os.path.join(HERE, "libcascade_hip.so")
+WORKLOADS_LIB = os.path.join(HERE, "libcascade_workloads.so")
+
+HIPCC_FLAGS = [
+    "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared", "-Wall",
+    # packed FP32 instructions stay off (nothing here is floating point, the flag is policy for this target)
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def _run(cmd):
+    print("+", " ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+
+
+def build_hip(extra_flags=()):
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    _run([hipcc, *HIPCC_FLAGS, *extra_flags, "-o", HIP_LIB, os.path.join(CSRC, "cascade_hip.hip")])
+    return HIP_LIB
+
+
+def build_workloads():
+    cc = os.environ.get("CC", "gcc")
+    _run([cc, "-std=c11", "-O2", "-fopenmp", "-fPIC", "-shared", "-Wall", "-Wextra", "-o", WORKLOADS_LIB,
+          os.path.join(CSRC, "workloads.c"), "-lm"])
+    return WORKLOADS_LIB
+
+
+def build_all():
+    build_hip()
+    build_workloads()
+
+
+if __name__ == "__main__":
+    build_all()
+    sys.exit(0)

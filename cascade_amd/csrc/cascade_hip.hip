@@ -1,0 +1,676 @@
+// Host side of the library: the handle, the radix-sort driver, the generation loop and the C ABI
+// declared in include/cascade_hip.h. gfx950 only.
+#include "../../include/cascade_hip.h"
+
+#include "device_utils.hpp"
+#include "doubling.hpp"
+#include "radix_sort.hpp"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+using namespace csa;
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                                  \
+    do {                                                                                               \
+        hipError_t e_ = (expr);                                                                        \
+        if (e_ != hipSuccess)                                                                          \
+            return fail(CSA_ERR_HIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), __FILE__, __LINE__); \
+    } while (0)
+
+constexpr int SORT_BLOCK = 512;
+constexpr int SORT_ITEMS = 16;
+constexpr int SORT_TILE = SORT_BLOCK * SORT_ITEMS;
+constexpr int RANK_BLOCK = 256;
+constexpr int RANK_ITEMS = 8;
+constexpr int RANK_TILE = RANK_BLOCK * RANK_ITEMS;
+constexpr u32 TICKET_POOL = 4096;
+constexpr int EVENT_POOL = 2 * CSA_MAX_GENERATIONS * MAX_PASSES * 2;
+
+int bit_length(u64 v)
+{
+    int b = 0;
+    while (v) {
+        ++b;
+        v >>= 1;
+    }
+    return b;
+}
+
+} // namespace
+
+struct csa_handle {
+    int device = 0;
+    u64 cap = 0;
+    int key_words = 1;
+    u64* key[2] = {nullptr, nullptr};
+    u32* idx[3] = {nullptr, nullptr, nullptr};
+    u32* gid = nullptr;
+    u32* rank = nullptr;
+    u32* gprim[2] = {nullptr, nullptr};
+    u64* lookback = nullptr;
+    u64 lookback_words = 0;
+    u32* ghist = nullptr;      // [MAX_PASSES][256]
+    u32* digit_base = nullptr; // [MAX_PASSES][256]
+    u32* tickets = nullptr;    // [TICKET_POOL]
+    u32 ticket_next = 0;
+    u32* counts = nullptr; // [2] survivors, groups; [2] error flag; [3] verifier flag
+    u32* h_pinned = nullptr; // host mirror: [0..3] counts/err, [16 ..) histogram
+    u32 epoch = 0;
+    std::vector<hipEvent_t> events;
+    hipEvent_t ev_gen[CSA_MAX_GENERATIONS + 2] = {};
+    bool ev_gen_ready = false;
+};
+
+namespace {
+
+struct Launch {
+    csa_handle* h;
+    hipStream_t stream;
+    u32 flags;
+    csa_stats* stats;
+    std::vector<std::pair<int, u64>> timed; // (first event index, pairs) of each timed radix launch
+    int events_used = 0;
+};
+
+int next_ticket(Launch& L, u32** out)
+{
+    csa_handle* h = L.h;
+    if (h->ticket_next == TICKET_POOL) {
+        HIP_TRY(hipMemsetAsync(h->tickets, 0, TICKET_POOL * sizeof(u32), L.stream));
+        h->ticket_next = 0;
+    }
+    *out = h->tickets + h->ticket_next++;
+    return CSA_OK;
+}
+
+u32 next_epoch(csa_handle* h)
+{
+    h->epoch++;
+    if (h->epoch >= (1u << 30)) { // never in practice; stale words would need a clear before reuse
+        (void)hipMemset(h->lookback, 0, h->lookback_words * sizeof(u64));
+        h->epoch = 1;
+    }
+    return h->epoch;
+}
+
+template <int SRC>
+void launch_hist(const HistArgs& a, hipStream_t s)
+{
+    u64 blocks = ((u64)a.n + 256 * 16 - 1) / (256 * 16);
+    if (blocks > 4096)
+        blocks = 4096;
+    if (blocks == 0)
+        blocks = 1;
+    hipLaunchKernelGGL((radix_hist_kernel<SRC>), dim3((u32)blocks), dim3(256), 0, s, a);
+}
+
+template <int SRC>
+void launch_onesweep(const OnesweepArgs& a, hipStream_t s)
+{
+    const u32 tiles = (u32)(((u64)a.n + SORT_TILE - 1) / SORT_TILE);
+    hipLaunchKernelGGL((onesweep_kernel<SORT_BLOCK, SORT_ITEMS, SRC>), dim3(tiles), dim3(SORT_BLOCK), 0, s, a);
+}
+
+// Sorts n pairs by the digits of `plan`. The first pass that runs takes its input as `src` says
+// (pairs kin/vin, or the text); passes alternate between the (kin, vin) and (kout, vout) sets, the
+// very first one writing to (kout, vout). *result_in_out = 1 if the sorted pairs ended in (kout, vout).
+// Passes whose digit is the same for every pair are skipped (they would be the identity).
+int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 word, u64* kin, u32* vin, u64* kout,
+               u32* vout, u32 n, const PassPlan& plan, int* result_in_out, int* passes_run)
+{
+    csa_handle* h = L.h;
+    hipStream_t s = L.stream;
+    *result_in_out = 0;
+    *passes_run = 0;
+    if (n == 0)
+        return CSA_OK;
+    HIP_TRY(hipMemsetAsync(h->ghist, 0, MAX_PASSES * RADIX_BINS * sizeof(u32), s));
+    HistArgs ha;
+    ha.keys = kin;
+    ha.vals = vin;
+    ha.text = text;
+    ha.n = n;
+    ha.text_n = text_n;
+    ha.word = word;
+    ha.plan = plan;
+    ha.ghist = h->ghist;
+    if (src == SRC_PAIRS)
+        launch_hist<SRC_PAIRS>(ha, s);
+    else if (src == SRC_TEXT)
+        launch_hist<SRC_TEXT>(ha, s);
+    else
+        launch_hist<SRC_TEXT_IDX>(ha, s);
+    hipLaunchKernelGGL(radix_scan_hist_kernel, dim3(1), dim3(256), 0, s, h->ghist, h->digit_base, plan.num_passes);
+    HIP_TRY(hipGetLastError());
+    u32* h_hist = h->h_pinned + 16;
+    HIP_TRY(hipMemcpyAsync(h_hist, h->ghist, plan.num_passes * RADIX_BINS * sizeof(u32), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    bool run[MAX_PASSES];
+    int n_run = 0;
+    for (int p = 0; p < plan.num_passes; ++p) {
+        bool trivial = false;
+        for (int d = 0; d < RADIX_BINS; ++d)
+            if (h_hist[p * RADIX_BINS + d] == n)
+                trivial = true;
+        run[p] = !trivial;
+        n_run += run[p] ? 1 : 0;
+    }
+    if (n_run == 0 && src != SRC_PAIRS && plan.num_passes > 0) { // the pairs must still be materialised once
+        run[plan.num_passes - 1] = true;
+        n_run = 1;
+    }
+    bool first = true;
+    int where = 0; // 0: current data in (kin, vin) (or the text); 1: in (kout, vout)
+    for (int p = 0; p < plan.num_passes; ++p) {
+        if (!run[p])
+            continue;
+        OnesweepArgs a;
+        a.keys_in = where == 0 ? kin : kout;
+        a.vals_in = where == 0 ? vin : vout;
+        a.keys_out = where == 0 ? kout : kin;
+        a.vals_out = where == 0 ? vout : vin;
+        a.text = text;
+        a.n = n;
+        a.text_n = text_n;
+        a.tail = tail;
+        a.word = word;
+        a.shift = plan.shift[p];
+        a.bits = plan.bits[p];
+        a.digit_base = h->digit_base + p * RADIX_BINS;
+        a.lookback = h->lookback;
+        a.epoch = next_epoch(h);
+        a.err = h->counts + 2;
+        int rc = next_ticket(L, &a.ticket);
+        if (rc)
+            return rc;
+        const bool timed = (L.flags & CSA_FLAG_KERNEL_TIMING) && L.events_used + 2 <= (int)h->events.size();
+        if (timed)
+            HIP_TRY(hipEventRecord(h->events[L.events_used], s));
+        const int use_src = first ? src : SRC_PAIRS;
+        if (use_src == SRC_PAIRS)
+            launch_onesweep<SRC_PAIRS>(a, s);
+        else if (use_src == SRC_TEXT)
+            launch_onesweep<SRC_TEXT>(a, s);
+        else
+            launch_onesweep<SRC_TEXT_IDX>(a, s);
+        if (timed) {
+            HIP_TRY(hipEventRecord(h->events[L.events_used + 1], s));
+            L.timed.push_back({L.events_used, (u64)n});
+            L.events_used += 2;
+        }
+        first = false;
+        where ^= 1;
+        (*passes_run)++;
+    }
+    HIP_TRY(hipGetLastError());
+    *result_in_out = where;
+    return CSA_OK;
+}
+
+PassPlan make_plan(int begin_bit, int end_bit)
+{
+    PassPlan p;
+    p.num_passes = 0;
+    for (int s = begin_bit; s < end_bit && p.num_passes < MAX_PASSES; s += RADIX_BITS) {
+        p.shift[p.num_passes] = s;
+        p.bits[p.num_passes] = end_bit - s < RADIX_BITS ? end_bit - s : RADIX_BITS;
+        p.num_passes++;
+    }
+    return p;
+}
+
+int ensure_events(csa_handle* h, bool kernel_timing)
+{
+    if (!h->ev_gen_ready) {
+        for (auto& e : h->ev_gen)
+            HIP_TRY(hipEventCreate(&e));
+        h->ev_gen_ready = true;
+    }
+    if (kernel_timing && h->events.empty()) {
+        h->events.resize(EVENT_POOL);
+        for (auto& e : h->events)
+            HIP_TRY(hipEventCreate(&e));
+    }
+    return CSA_OK;
+}
+
+int read_counts(Launch& L, u32* survivors, u32* groups)
+{
+    csa_handle* h = L.h;
+    HIP_TRY(hipMemcpyAsync(h->h_pinned, h->counts, 4 * sizeof(u32), hipMemcpyDeviceToHost, L.stream));
+    HIP_TRY(hipStreamSynchronize(L.stream));
+    if (h->h_pinned[2])
+        return fail(CSA_ERR_INTERNAL, "a look-back wait ran into its spin limit");
+    *survivors = h->h_pinned[0];
+    *groups = h->h_pinned[1];
+    return CSA_OK;
+}
+
+int launch_rerank(Launch& L, RerankArgs& a)
+{
+    csa_handle* h = L.h;
+    a.lookback = h->lookback;
+    a.epoch = next_epoch(h);
+    a.err = h->counts + 2;
+    a.counts = h->counts;
+    int rc = next_ticket(L, &a.ticket);
+    if (rc)
+        return rc;
+    const u32 tiles = (u32)(((u64)a.m + RANK_TILE - 1) / RANK_TILE);
+    hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS>), dim3(tiles), dim3(RANK_BLOCK), 0, L.stream, a);
+    HIP_TRY(hipGetLastError());
+    return CSA_OK;
+}
+
+int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_sa40)
+{
+    csa_handle* h = L.h;
+    hipStream_t s = L.stream;
+    csa_stats* st = L.stats;
+    const u32 n = (u32)n64;
+    const u32 ell = 4u * (u32)h->key_words;
+    const u32 tail = n < ell ? n : ell;
+
+    HIP_TRY(hipMemsetAsync(h->counts, 0, 4 * sizeof(u32), s));
+    HIP_TRY(hipEventRecord(h->ev_gen[0], s));
+
+    // ---- generation 0: sort every suffix by its K-gram key, ties of tail suffixes broken by length ----
+    int passes = 0, p1 = 0, in_out = 0;
+    const PassPlan full = make_plan(0, 64);
+    u64* K[2] = {h->key[0], h->key[1]};
+    u32* V[2] = {h->idx[0], h->idx[1]};
+    int cur; // the (K, V) set that holds the sorted pairs
+    int rc;
+    if (h->key_words == 1) {
+        rc = radix_sort(L, SRC_TEXT, d_text, n, tail, 0, K[0], V[0], K[1], V[1], n, full, &in_out, &passes);
+        if (rc)
+            return rc;
+        cur = in_out ? 1 : 0;
+    } else {
+        // 128-bit key: sort by the least significant word first, then stably by the most significant
+        // word, which is rebuilt from the text through the suffix indices of the first sort
+        rc = radix_sort(L, SRC_TEXT, d_text, n, tail, 1, K[0], V[0], K[1], V[1], n, full, &in_out, &p1);
+        if (rc)
+            return rc;
+        const int r1 = in_out ? 1 : 0;
+        rc = radix_sort(L, SRC_TEXT_IDX, d_text, n, tail, 0, K[r1], V[r1], K[r1 ^ 1], V[r1 ^ 1], n, full, &in_out,
+                        &passes);
+        if (rc)
+            return rc;
+        cur = in_out ? (r1 ^ 1) : r1;
+        passes += p1;
+    }
+    u64* k_sorted = K[cur];
+    u32* sa32 = V[cur];      // from here on the suffix array under construction
+    u32* act_a = V[cur ^ 1]; // the two index arrays left for the active lists
+    u32* act_b = h->idx[2];
+    u64* key_a = K[cur ^ 1]; // key array that travels with act_a
+    u64* key_b = k_sorted;   // free once generation 0 has been ranked; travels with act_b
+
+    RerankArgs ra;
+    memset(&ra, 0, sizeof(ra));
+    ra.keys = k_sorted;
+    ra.sufs = sa32;
+    ra.m = n;
+    ra.gen0 = 1;
+    ra.key_words = h->key_words;
+    ra.sec_bits = 0;
+    ra.n = n;
+    ra.ell = ell;
+    ra.text = d_text;
+    ra.gprim_in = nullptr;
+    ra.rank = h->rank;
+    ra.sa32 = sa32;
+    ra.sufs_out = act_a;
+    ra.gids_out = h->gid;
+    ra.gprim_out = h->gprim[0];
+    rc = launch_rerank(L, ra);
+    if (rc)
+        return rc;
+    u32 m = 0, groups = 0;
+    rc = read_counts(L, &m, &groups);
+    if (rc)
+        return rc;
+    st->passes[0] = passes;
+    st->active[0] = n;
+    st->groups[0] = 0;
+    HIP_TRY(hipEventRecord(h->ev_gen[1], s));
+
+    // ---- generations t >= 1 (reference loop: src/GPU_SACA.cu:1999-2103) ----
+    int gen = 1;
+    int gp = 0; // gprim[gp] holds the first ranks of the current groups
+    const int sec_bits = bit_length(n > 1 ? n - 1 : 1);
+    u64 h_ctx = ell;
+    while (m > 0) {
+        if (gen >= CSA_MAX_GENERATIONS)
+            return fail(CSA_ERR_INTERNAL, "generation cap reached with %u suffixes still active", m);
+        st->active[gen] = m;
+        st->groups[gen] = groups;
+        const u32 hh = (u32)h_ctx;
+        hipLaunchKernelGGL(gather_keys_kernel, dim3((m + 255) / 256), dim3(256), 0, s, act_a, h->gid, h->rank, m, n, hh,
+                           sec_bits, key_a);
+        const int gid_bits = bit_length(groups > 1 ? groups - 1 : 0);
+        const PassPlan plan = make_plan(0, sec_bits + gid_bits);
+        rc = radix_sort(L, SRC_PAIRS, nullptr, n, 0, 0, key_a, act_a, key_b, act_b, m, plan, &in_out, &passes);
+        if (rc)
+            return rc;
+        memset(&ra, 0, sizeof(ra));
+        ra.keys = in_out ? key_b : key_a;
+        ra.sufs = in_out ? act_b : act_a;
+        ra.m = m;
+        ra.gen0 = 0;
+        ra.key_words = h->key_words;
+        ra.sec_bits = sec_bits;
+        ra.n = n;
+        ra.ell = ell;
+        ra.text = d_text;
+        ra.gprim_in = h->gprim[gp];
+        ra.rank = h->rank;
+        ra.sa32 = sa32;
+        ra.sufs_out = in_out ? act_a : act_b;
+        ra.gids_out = h->gid;
+        ra.gprim_out = h->gprim[gp ^ 1];
+        rc = launch_rerank(L, ra);
+        if (rc)
+            return rc;
+        if (in_out == 0) { // survivors went to act_b: it becomes the current list
+            std::swap(act_a, act_b);
+            std::swap(key_a, key_b);
+        }
+        gp ^= 1;
+        rc = read_counts(L, &m, &groups);
+        if (rc)
+            return rc;
+        st->passes[gen] = passes;
+        HIP_TRY(hipEventRecord(h->ev_gen[gen + 1], s));
+        gen++;
+        h_ctx *= 2;
+    }
+    st->generations = gen;
+
+    // ---- output: 5-byte little-endian entries in rank order ----
+    const int aligned4 = ((uintptr_t)d_sa40 & 3u) == 0;
+    const u64 quads = ((u64)n + 3) / 4;
+    hipLaunchKernelGGL(emit_sa40_kernel, dim3((u32)((quads + 255) / 256)), dim3(256), 0, s, sa32, n, index_base, d_sa40,
+                       aligned4);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipEventRecord(h->ev_gen[gen + 1], s));
+    HIP_TRY(hipStreamSynchronize(s));
+
+    for (int g = 0; g < gen; ++g)
+        HIP_TRY(hipEventElapsedTime(&st->ms[g], h->ev_gen[g], h->ev_gen[g + 1]));
+    HIP_TRY(hipEventElapsedTime(&st->ms_output, h->ev_gen[gen], h->ev_gen[gen + 1]));
+    HIP_TRY(hipEventElapsedTime(&st->ms_total, h->ev_gen[0], h->ev_gen[gen + 1]));
+    for (auto& tl : L.timed) {
+        float ms = 0;
+        HIP_TRY(hipEventElapsedTime(&ms, h->events[tl.first], h->events[tl.first + 1]));
+        st->radix_ms += ms;
+        st->radix_pairs += tl.second;
+        st->radix_launches++;
+    }
+    return CSA_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+const char* csa_last_error(void) { return g_err; }
+
+uint64_t csa_bytes_per_suffix(int key_words)
+{
+    (void)key_words;
+    // two key arrays (8 B), three index arrays (4 B), group ids, ranks, two half-size group tables
+    return 2 * 8 + 3 * 4 + 4 + 4 + 4;
+}
+
+int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
+{
+    if (!out)
+        return fail(CSA_ERR_ARG, "csa_create: out is null");
+    *out = nullptr;
+    if (key_words != 1 && key_words != 2)
+        return fail(CSA_ERR_ARG, "csa_create: key_words must be 1 or 2, got %d", key_words);
+    if (max_part_sz > CSA_MAX_PART_SZ)
+        return fail(CSA_ERR_TOO_LARGE, "csa_create: %llu suffixes exceed the partition limit %llu",
+                    (unsigned long long)max_part_sz, (unsigned long long)CSA_MAX_PART_SZ);
+    csa_handle* h = new csa_handle();
+    h->cap = max_part_sz ? max_part_sz : 1;
+    h->key_words = key_words;
+    const u64 cap = h->cap;
+    const u64 sort_tiles = (cap + SORT_TILE - 1) / SORT_TILE;
+    const u64 rank_tiles = (cap + RANK_TILE - 1) / RANK_TILE;
+    h->lookback_words = sort_tiles * RADIX_BINS;
+    if (rank_tiles * 4 > h->lookback_words)
+        h->lookback_words = rank_tiles * 4;
+    hipError_t e = hipGetDevice(&h->device);
+    auto alloc = [&](void** p, u64 bytes) {
+        if (e == hipSuccess)
+            e = hipMalloc(p, bytes ? bytes : 4);
+    };
+    alloc((void**)&h->key[0], cap * 8);
+    alloc((void**)&h->key[1], cap * 8);
+    for (int i = 0; i < 3; ++i)
+        alloc((void**)&h->idx[i], cap * 4);
+    alloc((void**)&h->gid, cap * 4);
+    alloc((void**)&h->rank, cap * 4);
+    alloc((void**)&h->gprim[0], (cap / 2 + 1) * 4);
+    alloc((void**)&h->gprim[1], (cap / 2 + 1) * 4);
+    alloc((void**)&h->lookback, h->lookback_words * 8);
+    alloc((void**)&h->ghist, MAX_PASSES * RADIX_BINS * 4);
+    alloc((void**)&h->digit_base, MAX_PASSES * RADIX_BINS * 4);
+    alloc((void**)&h->tickets, TICKET_POOL * 4);
+    alloc((void**)&h->counts, 16 * 4);
+    if (e == hipSuccess)
+        e = hipHostMalloc((void**)&h->h_pinned, (16 + MAX_PASSES * RADIX_BINS) * 4, hipHostMallocDefault);
+    if (e == hipSuccess)
+        e = hipMemset(h->lookback, 0, h->lookback_words * 8);
+    if (e == hipSuccess)
+        e = hipMemset(h->tickets, 0, TICKET_POOL * 4);
+    if (e == hipSuccess)
+        e = hipMemset(h->counts, 0, 16 * 4);
+    if (e == hipSuccess)
+        e = hipDeviceSynchronize();
+    if (e != hipSuccess) {
+        const int rc = fail(CSA_ERR_HIP, "csa_create: %s while allocating for %llu suffixes", hipGetErrorString(e),
+                            (unsigned long long)cap);
+        csa_destroy(h);
+        return rc;
+    }
+    *out = h;
+    return CSA_OK;
+}
+
+void csa_destroy(csa_handle* h)
+{
+    if (!h)
+        return;
+    (void)hipFree(h->key[0]);
+    (void)hipFree(h->key[1]);
+    for (int i = 0; i < 3; ++i)
+        (void)hipFree(h->idx[i]);
+    (void)hipFree(h->gid);
+    (void)hipFree(h->rank);
+    (void)hipFree(h->gprim[0]);
+    (void)hipFree(h->gprim[1]);
+    (void)hipFree(h->lookback);
+    (void)hipFree(h->ghist);
+    (void)hipFree(h->digit_base);
+    (void)hipFree(h->tickets);
+    (void)hipFree(h->counts);
+    if (h->h_pinned)
+        (void)hipHostFree(h->h_pinned);
+    for (auto& e : h->events)
+        (void)hipEventDestroy(e);
+    if (h->ev_gen_ready)
+        for (auto& e : h->ev_gen)
+            (void)hipEventDestroy(e);
+    delete h;
+}
+
+int csa_sort_partition_u16_dev(csa_handle* h, const uint16_t* d_text, uint64_t n, uint64_t index_base,
+                               uint8_t* d_sa40, void* stream, uint32_t flags, csa_stats* stats)
+{
+    if (!h)
+        return fail(CSA_ERR_ARG, "csa_sort_partition_u16_dev: handle is null");
+    if (n > CSA_MAX_PART_SZ)
+        return fail(CSA_ERR_TOO_LARGE, "csa_sort_partition_u16_dev: %llu suffixes exceed the partition limit %llu",
+                    (unsigned long long)n, (unsigned long long)CSA_MAX_PART_SZ);
+    if (index_base > CSA_MAX_INDEX || index_base + n > CSA_MAX_INDEX)
+        return fail(CSA_ERR_TOO_LARGE, "csa_sort_partition_u16_dev: suffix indices up to %llu do not fit 40 bits",
+                    (unsigned long long)(index_base + n));
+    if (n > h->cap)
+        return fail(CSA_ERR_ARG, "csa_sort_partition_u16_dev: %llu suffixes exceed the handle's capacity %llu",
+                    (unsigned long long)n, (unsigned long long)h->cap);
+    csa_stats local;
+    csa_stats* st = stats ? stats : &local;
+    memset(st, 0, sizeof(*st));
+    st->n = n;
+    st->key_words = h->key_words;
+    if (n == 0)
+        return CSA_OK;
+    if (!d_text || !d_sa40)
+        return fail(CSA_ERR_ARG, "csa_sort_partition_u16_dev: null text or output pointer");
+    int rc = ensure_events(h, flags & CSA_FLAG_KERNEL_TIMING);
+    if (rc)
+        return rc;
+    Launch L;
+    L.h = h;
+    L.stream = (hipStream_t)stream;
+    L.flags = flags;
+    L.stats = st;
+    return sort_partition(L, d_text, n, index_base, d_sa40);
+}
+
+int csa_sort_partition_u16(const uint16_t* h_text, uint64_t n, int key_words, uint8_t* h_sa40, csa_stats* stats)
+{
+    if (n > CSA_MAX_PART_SZ)
+        return fail(CSA_ERR_TOO_LARGE, "csa_sort_partition_u16: %llu suffixes exceed the partition limit %llu",
+                    (unsigned long long)n, (unsigned long long)CSA_MAX_PART_SZ);
+    if (n > 0 && (!h_text || !h_sa40))
+        return fail(CSA_ERR_ARG, "csa_sort_partition_u16: null text or output pointer");
+    csa_handle* h = nullptr;
+    int rc = csa_create(n, key_words, &h);
+    if (rc)
+        return rc;
+    uint16_t* d_text = nullptr;
+    uint8_t* d_sa = nullptr;
+    hipError_t e = hipMalloc((void**)&d_text, n ? n * 2 : 4);
+    if (e == hipSuccess)
+        e = hipMalloc((void**)&d_sa, n ? n * 5 : 4);
+    if (e == hipSuccess && n)
+        e = hipMemcpy(d_text, h_text, n * 2, hipMemcpyHostToDevice);
+    if (e != hipSuccess)
+        rc = fail(CSA_ERR_HIP, "csa_sort_partition_u16: %s", hipGetErrorString(e));
+    if (!rc)
+        rc = csa_sort_partition_u16_dev(h, d_text, n, 0, d_sa, nullptr, 0, stats);
+    if (!rc && n) {
+        e = hipMemcpy(h_sa40, d_sa, n * 5, hipMemcpyDeviceToHost);
+        if (e != hipSuccess)
+            rc = fail(CSA_ERR_HIP, "csa_sort_partition_u16: %s", hipGetErrorString(e));
+    }
+    (void)hipFree(d_text);
+    (void)hipFree(d_sa);
+    csa_destroy(h);
+    return rc;
+}
+
+int csa_pack_keys_u16_dev(const uint16_t* d_text, uint64_t n, int key_words, uint64_t* d_keys, void* stream)
+{
+    if (key_words != 1 && key_words != 2)
+        return fail(CSA_ERR_ARG, "csa_pack_keys_u16_dev: key_words must be 1 or 2, got %d", key_words);
+    if (n > CSA_MAX_PART_SZ)
+        return fail(CSA_ERR_TOO_LARGE, "csa_pack_keys_u16_dev: %llu suffixes exceed the partition limit",
+                    (unsigned long long)n);
+    if (n == 0)
+        return CSA_OK;
+    if (!d_text || !d_keys)
+        return fail(CSA_ERR_ARG, "csa_pack_keys_u16_dev: null pointer");
+    hipLaunchKernelGGL(pack_keys_kernel, dim3((u32)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, d_text, (u32)n,
+                       key_words, d_keys);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return CSA_OK;
+}
+
+int csa_radix_sort_pairs_dev(csa_handle* h, uint64_t* d_keys, uint32_t* d_vals, uint64_t n, int begin_bit,
+                             int end_bit, void* stream)
+{
+    if (!h)
+        return fail(CSA_ERR_ARG, "csa_radix_sort_pairs_dev: handle is null");
+    if (begin_bit < 0 || end_bit > 64 || begin_bit > end_bit)
+        return fail(CSA_ERR_ARG, "csa_radix_sort_pairs_dev: bad bit range [%d, %d)", begin_bit, end_bit);
+    if (n > h->cap)
+        return fail(CSA_ERR_ARG, "csa_radix_sort_pairs_dev: %llu pairs exceed the handle's capacity %llu",
+                    (unsigned long long)n, (unsigned long long)h->cap);
+    if (n == 0 || begin_bit == end_bit)
+        return CSA_OK;
+    if (!d_keys || !d_vals)
+        return fail(CSA_ERR_ARG, "csa_radix_sort_pairs_dev: null pointer");
+    Launch L;
+    L.h = h;
+    L.stream = (hipStream_t)stream;
+    L.flags = 0;
+    L.stats = nullptr;
+    HIP_TRY(hipMemsetAsync(h->counts, 0, 4 * sizeof(u32), L.stream));
+    int in_out = 0, passes = 0;
+    const PassPlan plan = make_plan(begin_bit, end_bit);
+    int rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, d_keys, d_vals, h->key[0], h->idx[0], (u32)n, plan, &in_out,
+                        &passes);
+    if (rc)
+        return rc;
+    if (in_out) {
+        HIP_TRY(hipMemcpyAsync(d_keys, h->key[0], n * 8, hipMemcpyDeviceToDevice, L.stream));
+        HIP_TRY(hipMemcpyAsync(d_vals, h->idx[0], n * 4, hipMemcpyDeviceToDevice, L.stream));
+    }
+    u32 a = 0, b = 0;
+    return read_counts(L, &a, &b);
+}
+
+int csa_verify_sa40_dev(csa_handle* h, const uint16_t* d_text, uint64_t n, uint64_t index_base,
+                        const uint8_t* d_sa40, void* stream, int* ok)
+{
+    if (!h || !ok)
+        return fail(CSA_ERR_ARG, "csa_verify_sa40_dev: null handle or result pointer");
+    *ok = 0;
+    if (n > h->cap)
+        return fail(CSA_ERR_ARG, "csa_verify_sa40_dev: %llu suffixes exceed the handle's capacity %llu",
+                    (unsigned long long)n, (unsigned long long)h->cap);
+    if (n == 0) {
+        *ok = 1;
+        return CSA_OK;
+    }
+    if (!d_text || !d_sa40)
+        return fail(CSA_ERR_ARG, "csa_verify_sa40_dev: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    const u32 blocks = (u32)((n + 255) / 256);
+    HIP_TRY(hipMemsetAsync(h->counts + 3, 0, sizeof(u32), s));
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(blocks), dim3(256), 0, s, h->rank, n, 0xFFFFFFFFu);
+    hipLaunchKernelGGL(verify_invert_kernel, dim3(blocks), dim3(256), 0, s, d_sa40, (u32)n, index_base, h->rank,
+                       h->counts + 3);
+    hipLaunchKernelGGL(verify_order_kernel, dim3(blocks), dim3(256), 0, s, d_sa40, d_text, (u32)n, index_base, h->rank,
+                       h->counts + 3);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpyAsync(h->h_pinned + 3, h->counts + 3, sizeof(u32), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    *ok = h->h_pinned[3] ? 0 : 1;
+    return CSA_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,147 @@
+"""Host-side mirror of the reference's builder interface for the one path this package implements.
+
+Reference: `gpu_saca::GPU_SACA<uint16_t>(ip_path, op_path).build_SA()` (include/GPU_SACA.hpp:304-313,
+src/main.cu:12-46) reads a file of little-endian uint16 symbols and writes one 5-byte little-endian suffix
+index per symbol, in suffix order. Here the whole text is one partition, sorted in HBM through the C ABI
+(include/cascade_hip.h). Where the reference prints a message and exits on an error, these raise.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _native
+
+SA_WIDTH = 5  # include/sa40.hpp:24
+
+
+def stats_to_dict(st):
+    g = int(st.generations)
+    return {
+        "n": int(st.n),
+        "key_words": int(st.key_words),
+        "generations": g,
+        "active": [int(st.active[i]) for i in range(g)],
+        "groups": [int(st.groups[i]) for i in range(g)],
+        "passes": [int(st.passes[i]) for i in range(g)],
+        "ms": [float(st.ms[i]) for i in range(g)],
+        "ms_output": float(st.ms_output),
+        "ms_total": float(st.ms_total),
+        "radix_launches": int(st.radix_launches),
+        "radix_pairs": int(st.radix_pairs),
+        "radix_ms": float(st.radix_ms),
+    }
+
+
+class PartitionSorter:
+    """Owns the device scratch for partitions of up to `max_part_sz` suffixes (csa_create / csa_destroy)."""
+
+    def __init__(self, max_part_sz, key_words=1):
+        self._lib = _native.load()
+        self._h = C.c_void_p()
+        _native.check(self._lib.csa_create(int(max_part_sz), int(key_words), C.byref(self._h)))
+        self.max_part_sz = int(max_part_sz)
+        self.key_words = int(key_words)
+        self.last_stats = None
+
+    def close(self):
+        if self._h:
+            self._lib.csa_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    @staticmethod
+    def bytes_per_suffix(key_words=1):
+        return int(_native.load().csa_bytes_per_suffix(int(key_words)))
+
+    def sort_ptr(self, d_text, n, d_sa40, index_base=0, stream=0, flags=0):
+        """Raw device pointers in, statistics out (csa_sort_partition_u16_dev)."""
+        st = _native.CsaStats()
+        _native.check(self._lib.csa_sort_partition_u16_dev(self._h, d_text, int(n), int(index_base), d_sa40,
+                                                           stream or None, int(flags), C.byref(st)))
+        self.last_stats = stats_to_dict(st)
+        return self.last_stats
+
+    def sort(self, text, out=None, index_base=0, flags=0):
+        """text: a uint16 torch tensor on the GPU (viewed as int16 is fine). Returns a uint8 tensor of 5*n bytes."""
+        import torch
+        assert text.is_cuda and text.element_size() == 2 and text.is_contiguous()
+        n = text.numel()
+        if out is None:
+            out = torch.empty(SA_WIDTH * n + 128, dtype=torch.uint8, device=text.device)  # pad: include/sa40.hpp:31-37
+        assert out.is_cuda and out.dtype == torch.uint8 and out.numel() >= SA_WIDTH * n
+        stream = torch.cuda.current_stream(text.device).cuda_stream
+        self.sort_ptr(text.data_ptr(), n, out.data_ptr(), index_base, stream, flags)
+        return out[:SA_WIDTH * n]
+
+    def radix_sort_pairs(self, keys, vals, begin_bit=0, end_bit=64):
+        """In-place stable LSD sort of (uint64 key, uint32 value) device tensors (csa_radix_sort_pairs_dev)."""
+        import torch
+        assert keys.is_cuda and vals.is_cuda and keys.element_size() == 8 and vals.element_size() == 4
+        assert keys.numel() == vals.numel()
+        stream = torch.cuda.current_stream(keys.device).cuda_stream
+        _native.check(self._lib.csa_radix_sort_pairs_dev(self._h, keys.data_ptr(), vals.data_ptr(), keys.numel(),
+                                                         int(begin_bit), int(end_bit), stream or None))
+
+    def verify(self, text, sa40, index_base=0):
+        """Device-side O(n) suffix-array check (csa_verify_sa40_dev). Returns True if sa40 is the suffix array."""
+        import torch
+        ok = C.c_int(0)
+        stream = torch.cuda.current_stream(text.device).cuda_stream
+        _native.check(self._lib.csa_verify_sa40_dev(self._h, text.data_ptr(), text.numel(), int(index_base),
+                                                    sa40.data_ptr(), stream or None, C.byref(ok)))
+        return bool(ok.value)
+
+
+def pack_keys(text, key_words=1):
+    """K-gram keys of every suffix of a uint16 device tensor: int64 tensor [n, key_words] (csa_pack_keys_u16_dev)."""
+    import torch
+    lib = _native.load()
+    n = text.numel()
+    keys = torch.empty((n, key_words), dtype=torch.int64, device=text.device)
+    stream = torch.cuda.current_stream(text.device).cuda_stream
+    _native.check(lib.csa_pack_keys_u16_dev(text.data_ptr(), n, int(key_words), keys.data_ptr(), stream or None))
+    return keys
+
+
+def sort_partition(text, key_words=1):
+    """Host arrays in and out: uint16 numpy text -> uint8 numpy sa40 of 5*n bytes, plus statistics
+    (csa_sort_partition_u16: device memory is allocated and released inside the call)."""
+    lib = _native.load()
+    text = np.ascontiguousarray(text, dtype=np.uint16)
+    n = int(text.size)
+    sa40 = np.zeros(SA_WIDTH * n, dtype=np.uint8)
+    st = _native.CsaStats()
+    _native.check(lib.csa_sort_partition_u16(text.ctypes.data if n else None, n, int(key_words),
+                                             sa40.ctypes.data if n else None, C.byref(st)))
+    return sa40, stats_to_dict(st)
+
+
+class GPU_SACA:
+    """`GPU_SACA(ip_path, op_path).build_SA()`: file of uint16 symbols in, file of 5-byte suffix indices out."""
+
+    def __init__(self, ip_path, op_path, key_words=1):
+        self.ip_path = ip_path
+        self.op_path = op_path
+        self.key_words = key_words
+        self._timings = None
+
+    def build_SA(self):
+        text = np.fromfile(self.ip_path, dtype="<u2")
+        sa40, stats = sort_partition(text, self.key_words)
+        sa40.tofile(self.op_path)
+        self._timings = stats
+        return stats
+
+    def timings(self):
+        return self._timings

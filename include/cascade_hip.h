@@ -1,0 +1,113 @@
+/*
+ * cascade_hip.h : C ABI of the MI355X (gfx950) per-partition suffix sort.
+ *
+ * One partition's suffixes are sorted entirely in HBM by prefix doubling and leave as a
+ * suffix array of 5-byte little-endian entries ("sa40"), in the reference's order: numeric
+ * symbol order, the shorter suffix first, no sentinel.
+ *
+ * Every entry point returns 0 on success and a negative csa_status otherwise; nothing here
+ * ever exits the process. csa_last_error() describes the last failure of the calling thread.
+ * Pointers named d_* are device (HBM) addresses, h_* are host addresses. `stream` is a
+ * hipStream_t passed as void* (NULL = the default stream). A handle owns all device scratch
+ * memory and serves one call at a time; use one handle per stream for concurrent partitions.
+ */
+#ifndef CASCADE_HIP_H
+#define CASCADE_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CSA_MAX_GENERATIONS 64
+
+/* Largest partition: local ranks are 31-bit (reference: include/bit-layout.hpp:51-68, MAX_PART_SZ). */
+#define CSA_MAX_PART_SZ 2147483647ull
+/* Largest suffix index a 5-byte lane holds (reference: include/sa40.hpp:24-27, include/bit-layout.hpp:32,47). */
+#define CSA_MAX_INDEX (1ull << 40)
+
+typedef enum csa_status {
+    CSA_OK = 0,
+    CSA_ERR_ARG = -1,       /* null pointer, bad key_words, n beyond the handle's capacity */
+    CSA_ERR_TOO_LARGE = -2, /* n > CSA_MAX_PART_SZ or index_base + n > CSA_MAX_INDEX */
+    CSA_ERR_HIP = -3,       /* a HIP runtime call failed (out of memory included) */
+    CSA_ERR_INTERNAL = -4   /* a device-side invariant failed (look-back spin limit, generation cap) */
+} csa_status;
+
+/* Flags of csa_sort_partition_u16_dev. */
+#define CSA_FLAG_KERNEL_TIMING 1u /* bracket every radix-pass launch with events (fills the radix_* stats) */
+
+typedef struct csa_stats {
+    uint64_t n;
+    int32_t key_words;
+    int32_t generations;                  /* generations run, generation 0 included */
+    uint64_t active[CSA_MAX_GENERATIONS]; /* suffixes active entering generation g; active[0] = n */
+    uint64_t groups[CSA_MAX_GENERATIONS]; /* unresolved groups entering generation g (0 for g = 0) */
+    int32_t passes[CSA_MAX_GENERATIONS];  /* radix passes run in generation g */
+    float ms[CSA_MAX_GENERATIONS];        /* device time of generation g */
+    float ms_output;                      /* sa40 emission */
+    float ms_total;                       /* first kernel to last kernel, on the stream */
+    /* with CSA_FLAG_KERNEL_TIMING: the radix-pass kernel, summed over all its launches */
+    uint64_t radix_launches;
+    uint64_t radix_pairs; /* (key, index) pairs moved, summed over launches */
+    double radix_ms;
+} csa_stats;
+
+typedef struct csa_handle csa_handle;
+
+/* Device bytes the handle holds per suffix of capacity (text and output excluded).
+ * Replaces the sizing of the reference's GPU_SACA::partition_size_upper_bound / allocate_device_space
+ * (include/GPU_SACA.hpp:209,221; src/GPU_SACA.cu:372,535-590). */
+uint64_t csa_bytes_per_suffix(int key_words);
+
+/* Allocates the scratch for partitions of up to max_part_sz suffixes on the current device.
+ * key_words: 64-bit words of the generation-0 key, 1 or 2 (4 or 8 uint16 symbols; the reference's
+ * PREF_KEY_WORDS, include/Packed_Prefix.hpp:20-24).
+ * Replaces GPU_SACA::allocate_device_space (src/GPU_SACA.cu:535-590). */
+int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out);
+
+/* Frees everything the handle owns (reference: the destructor, src/GPU_SACA.cu:103-120). */
+void csa_destroy(csa_handle* h);
+
+/* Sorts the partition d_text[0, n) (uint16 symbols, no padding required) and writes its suffix
+ * array as n 5-byte little-endian entries to d_sa40 (5 * n bytes; entry = index_base + position).
+ * All generations run in HBM without host round trips of data; the call returns after the
+ * stream has finished. Replaces, for a partition resident in HBM, the sequence
+ * sort_and_init_rank_and_filter -> sort_and_re_rank_and_filter per generation -> scatter_to_rank_order
+ * (include/GPU_SACA.hpp:272,279,288; src/GPU_SACA.cu:1112-1331,1715-1995,1999-2103,2107-2164)
+ * and emits the layout of include/lane.hpp:69-79 / include/sa40.hpp:72-75. */
+int csa_sort_partition_u16_dev(csa_handle* h, const uint16_t* d_text, uint64_t n, uint64_t index_base,
+                               uint8_t* d_sa40, void* stream, uint32_t flags, csa_stats* stats);
+
+/* Convenience for host buffers: creates a handle, copies the text in, sorts, copies the sa40 out
+ * (5 * n bytes), destroys the handle. What `cascade <text> <sa>` does for one partition
+ * (src/main.cu:12-46 -> GPU_SACA::build_SA, src/GPU_SACA.cu:125-216). */
+int csa_sort_partition_u16(const uint16_t* h_text, uint64_t n, int key_words, uint8_t* h_sa40, csa_stats* stats);
+
+/* ---- the stages, exposed one by one so each can be checked against its CPU restatement ---- */
+
+/* K-gram key packing: d_keys[j * key_words + w] = symbols [j + 4w, j + 4w + 4) of the zero-padded text,
+ * first symbol in the most significant bits (reference: util::pack_word, include/utility.hpp:147-162;
+ * Packed_Prefix::pack_prefix, include/Packed_Prefix.hpp:91-104; host loop src/GPU_SACA.cu:1674-1684). */
+int csa_pack_keys_u16_dev(const uint16_t* d_text, uint64_t n, int key_words, uint64_t* d_keys, void* stream);
+
+/* Stable LSD radix sort of (64-bit key, 32-bit value) pairs on key bits [begin_bit, end_bit); the sorted
+ * pairs are left in d_keys / d_vals. Uses the handle's scratch (n <= its capacity).
+ * Replaces cub::DeviceRadixSort::SortPairs (src/GPU_SACA.cu:1175-1181,1203-1210,1783-1789,1849-1855). */
+int csa_radix_sort_pairs_dev(csa_handle* h, uint64_t* d_keys, uint32_t* d_vals, uint64_t n, int begin_bit,
+                             int end_bit, void* stream);
+
+/* O(n) suffix-array check on the device: d_sa40 is a permutation of [index_base, index_base + n) and every
+ * adjacent pair is in order (first symbols, then ranks of the successors; a successor past the end sorts
+ * first). *ok = 1 if correct. Same rule as the reference's validator (test/end-to-end.cpp:13-80). */
+int csa_verify_sa40_dev(csa_handle* h, const uint16_t* d_text, uint64_t n, uint64_t index_base,
+                        const uint8_t* d_sa40, void* stream, int* ok);
+
+/* Message of the calling thread's last failed call ("" if none). */
+const char* csa_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

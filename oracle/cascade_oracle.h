@@ -1,0 +1,88 @@
+/*
+ * CPU oracle for the per-partition suffix sort: TEST INFRASTRUCTURE ONLY.
+ *
+ * Nothing here is part of the product. Only the test suite, the smoke check and the
+ * CPU-baseline leg of the benchmark may link or call it, and only as the checker.
+ * Every function restates a piece of the reference (saltsystemslab/Cascade) in plain C;
+ * the file:line each one follows is given beside its declaration.
+ *
+ * How each function is pinned (what a plausible mistake would trip over):
+ *   orc_cmp_suffixes / orc_build_sa40_u16 : the reference's own known answers and hand cases
+ *       (src/test_query.cu:374-392,405-411), closed forms (a^n, increasing, decreasing,
+ *       (ab)^k, Fibonacci word), the zero-tail corner case (dataset/make-corner-case.py:37),
+ *       and byte-for-byte equality with the reference's compiled build_sa40 where the
+ *       _ref library builds.
+ *   orc_is_correct_sa_u16 : accepts exactly the SA of build_sa40 and rejects a swapped
+ *       pair, an out-of-range entry, a repeated entry and the byte-order SA
+ *       (the negative controls of src/test_query.cu:417-454).
+ *   orc_pack_word_u16 / orc_pack_prefix_u16 : closed form (4-term shift/or) and the order
+ *       invariant key(i) < key(j) <=> T[i..i+4) <lex T[j..j+4).
+ *   orc_fwd_tag : closed form, and the tail-order property it exists for.
+ *   orc_prefix_doubling_u16 : final order equals orc_build_sa40_u16 on every fixture;
+ *       per-generation active counts equal orc_retire_generations (an independent
+ *       closed form over SA + LCP, src/sa_structure.cpp:295-306,375).
+ *   orc_sa40_store / orc_sa40_load : round trip (src/test_query.cu:78-96) and explicit bytes.
+ */
+#ifndef CASCADE_ORACLE_H
+#define CASCADE_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ORC_SA_WIDTH 5        /* include/sa40.hpp:24 */
+#define ORC_SA_PAD_BYTES 128  /* include/sa40.hpp:37 */
+
+/* include/CPU_Reference.hpp:107-123. Order of suffixes i and j of T[0,n), at most max_cmp symbols. */
+int orc_cmp_suffixes_u16(const uint16_t* T, uint64_t n, uint64_t i, uint64_t j, uint64_t max_cmp);
+
+/* include/sa40.hpp:72-75 and :46-60 (host branch). */
+void orc_sa40_store(uint8_t* SA, uint64_t r, uint64_t v);
+uint64_t orc_sa40_load(const uint8_t* SA, uint64_t r);
+
+/* test/query.cpp:42-55. Comparison sort of all suffixes; SA must hold 5*n + ORC_SA_PAD_BYTES bytes
+ * (the pad is zero-filled like the reference's). */
+void orc_build_sa40_u16(const uint16_t* T, uint64_t n, uint8_t* SA);
+
+/* test/end-to-end.cpp:13-43 and :46-80. sa is 8-byte entries. Returns 1 if correct. */
+int orc_is_permutation(const uint64_t* sa, uint64_t n);
+int orc_is_correct_sa_u16(const uint64_t* sa, const uint16_t* T, uint64_t n);
+/* Same check over 5-byte lanes (test/end-to-end.cpp:99-116 widens them first). */
+int orc_is_correct_sa40_u16(const uint8_t* sa40, const uint16_t* T, uint64_t n);
+
+/* include/utility.hpp:147-162: four u16 symbols MSB-first in one word. T must be readable for 4 symbols. */
+uint64_t orc_pack_word_u16(const uint16_t* T);
+/* include/Packed_Prefix.hpp:91-104 over a text whose tail is padded with zeros (src/GPU_SACA.cu:223-236):
+ * words[w] for w in [0,key_words) of suffix j; positions >= n read as 0. */
+void orc_pack_prefix_u16(const uint16_t* T, uint64_t n, uint64_t j, int key_words, uint64_t* words);
+
+/* include/bit-layout.hpp:99-100 with a single partition (id == 0): tag of suffix j whose
+ * next-generation source is tgt = j + ell. */
+uint64_t orc_fwd_tag(uint64_t tgt, uint64_t n, uint64_t ell);
+
+/* The path restated for one partition holding the whole text:
+ * gen 0 = sort by (packed key, fwd tag), rank = head offset of the run, active = run length > 1
+ * (include/GPU_SACA.cuh:191-208, src/GPU_SACA.cu:1165-1247); generation t >= 1 sorts the active set by
+ * (rank(x), rank(x + ell*2^(t-1))) and refines rank += head(key run) - head(primary run)
+ * (include/GPU_SACA.cuh:218-280, src/GPU_SACA.cu:1841-1925); loop of src/GPU_SACA.cu:1999-2103;
+ * output SA[rank(j)] = j (include/GPU_SACA.cuh:167-182).
+ * sa_out: n entries. active_counts[g] = suffixes active entering generation g (g = 0 -> n), up to
+ * max_gens entries; returns the number of generations run (including generation 0). */
+int orc_prefix_doubling_u16(const uint16_t* T, uint64_t n, int key_words, uint64_t* sa_out,
+                            uint64_t* active_counts, int max_gens);
+
+/* src/sa_structure.cpp:295-306,375 with one partition: retirement generation d(j) of every suffix from
+ * the finished SA and brute-force LCPs. d_out[j] in [0, 63]. O(n * lcp): small inputs only. */
+void orc_retire_generations_u16(const uint16_t* T, uint64_t n, const uint64_t* sa, uint64_t ell, uint8_t* d_out);
+
+/* Stable LSD restatements used to check the device primitives at their boundary
+ * (the CUB contracts the reference relies on, src/GPU_SACA.cu:1175-1210,1241-1261). */
+void orc_stable_sort_pairs_u64_u32(uint64_t* keys, uint32_t* vals, uint64_t n, int begin_bit, int end_bit);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,45 @@
+// C-callable doorway into the reference's own CPU oracle, compiled from its sources where they lie
+// (test/query.cpp, test/end-to-end.cpp and the headers they include). TEST INFRASTRUCTURE ONLY:
+// used to validate the C restatement in cascade_oracle.c and as the "reference" CPU baseline.
+// Nothing of the reference is copied here; this file only calls it.
+#include "query_tests.hpp"    // gpu_saca::test::build_sa40      (test/query.cpp:42-55)
+#include "tests.hpp"          // gpu_saca::test::is_correct_SA   (test/end-to-end.cpp:46-80)
+#include "CPU_Reference.hpp"  // gpu_saca::ref::cmp_suffixes     (include/CPU_Reference.hpp:107-123)
+#include "Packed_Prefix.hpp"  // gpu_saca::Packed_Prefix         (include/Packed_Prefix.hpp:91-104)
+#include "bit-layout.hpp"     // gpu_saca::bit_layout::fwd_tag   (include/bit-layout.hpp:99-100)
+#include "utility.hpp"        // gpu_saca::util::pack_word       (include/utility.hpp:147-162)
+
+#include <cstring>
+#include <vector>
+
+extern "C" {
+
+// sa40_out: 5 * n + 128 bytes.
+void ref_build_sa40_u16(const uint16_t* T, uint64_t n, uint8_t* sa40_out)
+{
+    const std::vector<uint16_t> text(T, T + n);
+    const auto SA = gpu_saca::test::build_sa40(text);
+    std::memcpy(sa40_out, SA.data(), SA.size());
+}
+
+int ref_is_correct_sa_u16(const uint64_t* sa, const uint16_t* T, uint64_t n)
+{
+    return gpu_saca::test::is_correct_SA<uint16_t>(sa, T, n) ? 1 : 0;
+}
+
+int ref_cmp_suffixes_u16(const uint16_t* T, uint64_t n, uint64_t i, uint64_t j, uint64_t max_cmp)
+{
+    return gpu_saca::ref::cmp_suffixes(T, n, i, j, max_cmp);
+}
+
+uint64_t ref_pack_word_u16(const uint16_t* T)
+{
+    return gpu_saca::util::pack_word<uint16_t>(T);
+}
+
+uint64_t ref_fwd_tag_single_partition(uint64_t tgt, uint64_t n, uint64_t ell)
+{
+    return gpu_saca::bit_layout::fwd_tag([](const uint64_t) { return 0; }, tgt, n, ell);
+}
+
+}

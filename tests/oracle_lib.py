@@ -1,0 +1,171 @@
+"""ctypes access to the CPU oracle (oracle/_build/libcascade_oracle.so) and, where it was built, to the
+reference's own CPU oracle (oracle/_ref/libcascade_ref.so). Test infrastructure only."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+ORACLE_LIB = os.path.join(ORACLE_DIR, "_build", "libcascade_oracle.so")
+REF_LIB = os.path.join(ORACLE_DIR, "_ref", "libcascade_ref.so")
+SA_PAD = 128
+
+_oracle = None
+_ref = None
+
+
+def oracle():
+    global _oracle
+    if _oracle is None:
+        if not os.path.exists(ORACLE_LIB):
+            subprocess.run(["make", "-C", ORACLE_DIR, "_build/libcascade_oracle.so"], check=True)
+        lib = C.CDLL(ORACLE_LIB)
+        vp, u64, i32 = C.c_void_p, C.c_uint64, C.c_int
+        lib.orc_cmp_suffixes_u16.restype = i32
+        lib.orc_cmp_suffixes_u16.argtypes = [vp, u64, u64, u64, u64]
+        lib.orc_sa40_store.restype = None
+        lib.orc_sa40_store.argtypes = [vp, u64, u64]
+        lib.orc_sa40_load.restype = u64
+        lib.orc_sa40_load.argtypes = [vp, u64]
+        lib.orc_build_sa40_u16.restype = None
+        lib.orc_build_sa40_u16.argtypes = [vp, u64, vp]
+        lib.orc_is_permutation.restype = i32
+        lib.orc_is_permutation.argtypes = [vp, u64]
+        lib.orc_is_correct_sa_u16.restype = i32
+        lib.orc_is_correct_sa_u16.argtypes = [vp, vp, u64]
+        lib.orc_is_correct_sa40_u16.restype = i32
+        lib.orc_is_correct_sa40_u16.argtypes = [vp, vp, u64]
+        lib.orc_pack_word_u16.restype = u64
+        lib.orc_pack_word_u16.argtypes = [vp]
+        lib.orc_pack_prefix_u16.restype = None
+        lib.orc_pack_prefix_u16.argtypes = [vp, u64, u64, i32, vp]
+        lib.orc_fwd_tag.restype = u64
+        lib.orc_fwd_tag.argtypes = [u64, u64, u64]
+        lib.orc_prefix_doubling_u16.restype = i32
+        lib.orc_prefix_doubling_u16.argtypes = [vp, u64, i32, vp, vp, i32]
+        lib.orc_retire_generations_u16.restype = None
+        lib.orc_retire_generations_u16.argtypes = [vp, u64, vp, u64, vp]
+        lib.orc_stable_sort_pairs_u64_u32.restype = None
+        lib.orc_stable_sort_pairs_u64_u32.argtypes = [vp, vp, u64, i32, i32]
+        _oracle = lib
+    return _oracle
+
+
+def ref():
+    """The reference's own CPU oracle, or None where it was not built (no /root/reference and no prebuilt copy)."""
+    global _ref
+    if _ref is None and os.path.exists(REF_LIB):
+        lib = C.CDLL(REF_LIB)
+        vp, u64, i32 = C.c_void_p, C.c_uint64, C.c_int
+        lib.ref_build_sa40_u16.restype = None
+        lib.ref_build_sa40_u16.argtypes = [vp, u64, vp]
+        lib.ref_is_correct_sa_u16.restype = i32
+        lib.ref_is_correct_sa_u16.argtypes = [vp, vp, u64]
+        lib.ref_cmp_suffixes_u16.restype = i32
+        lib.ref_cmp_suffixes_u16.argtypes = [vp, u64, u64, u64, u64]
+        lib.ref_pack_word_u16.restype = u64
+        lib.ref_pack_word_u16.argtypes = [vp]
+        lib.ref_fwd_tag_single_partition.restype = u64
+        lib.ref_fwd_tag_single_partition.argtypes = [u64, u64, u64]
+        _ref = lib
+    return _ref
+
+
+def _text(T):
+    return np.ascontiguousarray(T, dtype=np.uint16)
+
+
+def _ptr(a):
+    return a.ctypes.data if a.size else None
+
+
+def build_sa40(T, lib=None):
+    """sa40 bytes (5*n, pad stripped) of the text by the oracle's comparison sort (or by `lib` = ref())."""
+    T = _text(T)
+    n = T.size
+    out = np.zeros(5 * n + SA_PAD, dtype=np.uint8)
+    if lib is None:
+        oracle().orc_build_sa40_u16(_ptr(T), n, out.ctypes.data)
+    else:
+        lib.ref_build_sa40_u16(_ptr(T), n, out.ctypes.data)
+    assert not out[5 * n:].any()
+    return out[:5 * n].copy()
+
+
+def sa40_to_u64(sa40):
+    sa40 = np.ascontiguousarray(sa40, dtype=np.uint8)
+    n = sa40.size // 5
+    b = sa40[:5 * n].reshape(n, 5).astype(np.uint64)
+    return b[:, 0] | (b[:, 1] << np.uint64(8)) | (b[:, 2] << np.uint64(16)) | (b[:, 3] << np.uint64(24)) | (
+        b[:, 4] << np.uint64(32))
+
+
+def u64_to_sa40(sa):
+    sa = np.ascontiguousarray(sa, dtype=np.uint64)
+    out = np.empty((sa.size, 5), dtype=np.uint8)
+    for b in range(5):
+        out[:, b] = (sa >> np.uint64(8 * b)) & np.uint64(0xFF)
+    return out.reshape(-1)
+
+
+def is_correct_sa(sa, T):
+    T = _text(T)
+    sa = np.ascontiguousarray(sa, dtype=np.uint64)
+    return bool(oracle().orc_is_correct_sa_u16(_ptr(sa), _ptr(T), T.size))
+
+
+def is_correct_sa40(sa40, T):
+    T = _text(T)
+    sa40 = np.ascontiguousarray(sa40, dtype=np.uint8)
+    assert sa40.size == 5 * T.size
+    return bool(oracle().orc_is_correct_sa40_u16(_ptr(sa40), _ptr(T), T.size))
+
+
+def prefix_doubling(T, key_words=1, max_gens=64):
+    T = _text(T)
+    n = T.size
+    sa = np.zeros(n, dtype=np.uint64)
+    counts = np.zeros(max_gens, dtype=np.uint64)
+    g = oracle().orc_prefix_doubling_u16(_ptr(T), n, key_words, _ptr(sa), counts.ctypes.data, max_gens)
+    return sa, [int(c) for c in counts[:g]]
+
+
+def retire_generations(T, sa, ell):
+    T = _text(T)
+    sa = np.ascontiguousarray(sa, dtype=np.uint64)
+    d = np.zeros(T.size, dtype=np.uint8)
+    oracle().orc_retire_generations_u16(_ptr(T), T.size, _ptr(sa), ell, _ptr(d))
+    return d
+
+
+def pack_prefix(T, key_words=1):
+    T = _text(T)
+    n = T.size
+    out = np.zeros((n, key_words), dtype=np.uint64)
+    tmp = np.zeros(key_words, dtype=np.uint64)
+    lib = oracle()
+    for j in range(n):
+        lib.orc_pack_prefix_u16(_ptr(T), n, j, key_words, tmp.ctypes.data)
+        out[j] = tmp
+    return out
+
+
+def pack_prefix_np(T, key_words=1):
+    """Vectorised form of pack_prefix for large inputs (checked against it in the oracle tests)."""
+    T = _text(T)
+    n = T.size
+    P = np.concatenate([T, np.zeros(4 * key_words, dtype=np.uint16)]).astype(np.uint64)
+    out = np.zeros((n, key_words), dtype=np.uint64)
+    for w in range(key_words):
+        for k in range(4):
+            out[:, w] = (out[:, w] << np.uint64(16)) | P[4 * w + k: 4 * w + k + n]
+    return out
+
+
+def stable_sort_pairs(keys, vals, begin_bit=0, end_bit=64):
+    keys = np.array(keys, dtype=np.uint64, copy=True)
+    vals = np.array(vals, dtype=np.uint32, copy=True)
+    oracle().orc_stable_sort_pairs_u64_u32(_ptr(keys), _ptr(vals), keys.size, begin_bit, end_bit)
+    return keys, vals

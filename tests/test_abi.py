@@ -1,0 +1,44 @@
+"""The C-ABI library loads and exports exactly what include/cascade_hip.h declares. No GPU needed."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from cascade_amd import _native
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    src = open(os.path.join(ROOT, "include", "cascade_hip.h")).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return sorted(set(re.findall(r"\b(csa_[a-z0-9_]+)\s*\(", src)))
+
+
+def test_header_and_binding_agree():
+    assert declared_functions() == sorted(_native.EXPORTS)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _native.load()
+    for name in declared_functions():
+        assert hasattr(lib, name), name
+
+
+def test_stats_struct_layout_matches_header():
+    # 8 + 4 + 4 + 64*8 + 64*8 + 64*4 + 64*4 + 4 + 4 + 8 + 8 + 8
+    assert C.sizeof(_native.CsaStats) == 8 + 4 + 4 + 512 + 512 + 256 + 256 + 4 + 4 + 8 + 8 + 8
+
+
+def test_argument_errors_need_no_gpu():
+    lib = _native.load()
+    assert lib.csa_bytes_per_suffix(1) == 40
+    h = C.c_void_p()
+    assert lib.csa_create(10, 3, C.byref(h)) == _native.CSA_ERR_ARG
+    assert b"key_words" in lib.csa_last_error()
+    assert lib.csa_create(1 << 31, 1, C.byref(h)) == _native.CSA_ERR_TOO_LARGE
+    assert lib.csa_sort_partition_u16(None, 1 << 31, 1, None, None) == _native.CSA_ERR_TOO_LARGE
+    assert lib.csa_sort_partition_u16_dev(None, None, 0, 0, None, None, 0, None) == _native.CSA_ERR_ARG
+    with pytest.raises(_native.CascadeError):
+        _native.check(lib.csa_radix_sort_pairs_dev(None, None, None, 0, 0, 64, None))
