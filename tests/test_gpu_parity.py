@@ -1,0 +1,195 @@
+"""Parity of the HIP path with the CPU oracle, through the C ABI, on a real MI355X."""
+import hashlib
+import os
+
+import numpy as np
+import pytest
+
+import oracle_lib
+import texts
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+@pytest.fixture(scope="module")
+def torch_mod():
+    import torch
+    assert torch.cuda.is_available()
+    return torch
+
+
+@pytest.fixture(scope="module")
+def sorter(torch_mod):
+    from cascade_amd import PartitionSorter
+    s = PartitionSorter(1 << 22, key_words=1)
+    yield s
+    s.close()
+
+
+@pytest.fixture(scope="module")
+def sorter2(torch_mod):
+    from cascade_amd import PartitionSorter
+    s = PartitionSorter(1 << 21, key_words=2)
+    yield s
+    s.close()
+
+
+def to_dev(torch, a):
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.uint16:
+        return torch.from_numpy(a.view(np.int16)).cuda()
+    if a.dtype == np.uint64:
+        return torch.from_numpy(a.view(np.int64)).cuda()
+    if a.dtype == np.uint32:
+        return torch.from_numpy(a.view(np.int32)).cuda()
+    return torch.from_numpy(a).cuda()
+
+
+def gpu_sa40(torch, s, T, index_base=0):
+    print(f"  sort n={len(T)} key_words={s.key_words}", flush=True)
+    d = to_dev(torch, np.asarray(T, dtype=np.uint16))
+    out = s.sort(d, index_base=index_base)
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+# ---- stage: K-gram key packing ---------------------------------------------------------------------
+
+@pytest.mark.parametrize("key_words", [1, 2])
+def test_pack_keys_matches_oracle(torch_mod, key_words):
+    from cascade_amd import pack_keys
+    for n, sigma, seed in ((1, 4, 0), (3, 4, 1), (4, 4, 2), (5, 65536, 3), (1000, 65536, 4), (100003, 65536, 5)):
+        T = texts.random_text(n, sigma, seed)
+        got = pack_keys(to_dev(torch_mod, T), key_words).cpu().numpy().view(np.uint64)
+        want = oracle_lib.pack_prefix_np(T, key_words)
+        assert np.array_equal(got, want), (n, key_words)
+
+
+# ---- stage: radix sort -----------------------------------------------------------------------------
+
+@pytest.mark.parametrize("n", [1, 2, 63, 64, 65, 8191, 8192, 8193, 100000, 1 << 20])
+def test_radix_sort_pairs_matches_stable_sort(torch_mod, sorter, n):
+    rng = np.random.default_rng(n)
+    keys = rng.integers(0, 1 << 63, n, dtype=np.uint64) * np.uint64(2) + rng.integers(0, 2, n, dtype=np.uint64)
+    vals = np.arange(n, dtype=np.uint32)
+    dk, dv = to_dev(torch_mod, keys), to_dev(torch_mod, vals)
+    sorter.radix_sort_pairs(dk, dv)
+    wk, wv = oracle_lib.stable_sort_pairs(keys, vals)
+    assert np.array_equal(dk.cpu().numpy().view(np.uint64), wk)
+    assert np.array_equal(dv.cpu().numpy().view(np.uint32), wv)
+
+
+def test_radix_sort_is_stable_on_skewed_keys_and_bit_ranges(torch_mod, sorter):
+    rng = np.random.default_rng(3)
+    n = 300000
+    cases = [
+        (rng.integers(0, 4, n).astype(np.uint64), 0, 64),                       # four values: long runs of ties
+        (np.zeros(n, dtype=np.uint64), 0, 64),                                  # every pass trivial
+        (np.full(n, 0xFFFFFFFFFFFFFFFF, dtype=np.uint64), 0, 64),               # collides with the tile padding
+        (rng.zipf(1.3, n).astype(np.uint64) << np.uint64(13), 13, 40),          # a bit sub-range
+        (rng.integers(0, 1 << 30, n).astype(np.uint64) | (rng.integers(0, 7, n).astype(np.uint64) << np.uint64(30)), 0, 33),
+        (np.where(rng.random(n) < 0.5, np.uint64(0xFF), np.uint64(0xFFFF)).astype(np.uint64), 0, 16),
+    ]
+    for keys, b, e in cases:
+        vals = rng.permutation(n).astype(np.uint32)
+        dk, dv = to_dev(torch_mod, keys), to_dev(torch_mod, vals)
+        sorter.radix_sort_pairs(dk, dv, b, e)
+        wk, wv = oracle_lib.stable_sort_pairs(keys, vals, b, e)
+        assert np.array_equal(dk.cpu().numpy().view(np.uint64), wk)
+        assert np.array_equal(dv.cpu().numpy().view(np.uint32), wv)
+
+
+# ---- whole partition: golden vectors of the reference's CPU sort ----------------------------------------
+
+def test_golden_fixtures_bit_exact(torch_mod, sorter, sorter2):
+    g = np.load(os.path.join(GOLDEN, "fixtures.npz"), allow_pickle=False)
+    for name, T in texts.fixture_suite():
+        want = g[f"{name}.sa40"]
+        for s in (sorter, sorter2):
+            got = gpu_sa40(torch_mod, s, T)
+            assert got.dtype == np.uint8 and got.size == 5 * len(T)
+            assert np.array_equal(got, want), f"{name} key_words={s.key_words}"
+
+
+def test_empty_partition(torch_mod, sorter):
+    d = torch_mod.empty(0, dtype=torch_mod.int16, device="cuda")
+    out = sorter.sort(d)
+    assert out.numel() == 0 and sorter.last_stats["generations"] == 0
+
+
+def test_c1_matches_reference_digest_and_generation_counts(torch_mod, sorter):
+    from cascade_amd import workloads
+    want = dict(line.split() for line in open(os.path.join(GOLDEN, "c1_sha256.txt")))
+    T = workloads.generate(1)
+    got = gpu_sa40(torch_mod, sorter, T)
+    assert hashlib.sha256(got.tobytes()).hexdigest() == want["sa40"]
+    _, counts = oracle_lib.prefix_doubling(T, 1)
+    assert sorter.last_stats["active"] == counts  # suffixes active entering each generation
+
+
+@pytest.mark.parametrize("config,n", [(2, 1 << 20), (3, 1 << 21), (4, 1 << 20), (5, 1 << 20)])
+def test_scaled_configs_against_oracle(torch_mod, sorter, config, n):
+    from cascade_amd import workloads
+    T = workloads.generate(config, n)
+    got = gpu_sa40(torch_mod, sorter, T)
+    sa, counts = oracle_lib.prefix_doubling(T, 1)
+    assert np.array_equal(got, oracle_lib.u64_to_sa40(sa))
+    assert sorter.last_stats["active"] == counts
+    assert oracle_lib.is_correct_sa40(got, T)
+
+
+def test_key_words_2_on_deep_repeats(torch_mod, sorter2):
+    from cascade_amd import workloads
+    for config in (3, 5):
+        T = workloads.generate(config, 1 << 19)
+        got = gpu_sa40(torch_mod, sorter2, T)
+        sa, counts = oracle_lib.prefix_doubling(T, 2)
+        assert np.array_equal(got, oracle_lib.u64_to_sa40(sa))
+        assert sorter2.last_stats["active"] == counts
+
+
+def test_index_base_offsets_every_entry(torch_mod, sorter):
+    T = texts.random_text(5000, 4, 11)
+    base = (1 << 39) + 12345
+    a = oracle_lib.sa40_to_u64(gpu_sa40(torch_mod, sorter, T))
+    b = oracle_lib.sa40_to_u64(gpu_sa40(torch_mod, sorter, T, index_base=base))
+    assert np.array_equal(a + np.uint64(base), b)
+
+
+def test_device_verifier_agrees_with_oracle(torch_mod, sorter):
+    T = texts.random_text(20000, 3, 21)
+    d = to_dev(torch_mod, T)
+    out = sorter.sort(d).clone()
+    assert sorter.verify(d, out)
+    sa = oracle_lib.sa40_to_u64(out.cpu().numpy())
+    for mutate in ("swap", "oob", "repeat"):
+        bad = sa.copy()
+        if mutate == "swap":
+            bad[[100, 101]] = bad[[101, 100]]
+        elif mutate == "oob":
+            bad[7] = len(T) + 3
+        else:
+            bad[11] = bad[10]
+        assert not oracle_lib.is_correct_sa(bad, T)
+        assert not sorter.verify(d, to_dev(torch_mod, oracle_lib.u64_to_sa40(bad)))
+
+
+def test_host_buffer_entry_point_and_file_interface(torch_mod, tmp_path):
+    from cascade_amd import GPU_SACA, sort_partition
+    T = texts.random_text(30000, 16, 5)
+    sa40, stats = sort_partition(T, 1)
+    assert np.array_equal(sa40, oracle_lib.build_sa40(T)) and stats["n"] == len(T)
+    ip, op = tmp_path / "text.u16", tmp_path / "sa.bin"
+    T.astype("<u2").tofile(ip)
+    GPU_SACA(str(ip), str(op)).build_SA()
+    assert np.array_equal(np.fromfile(op, dtype=np.uint8), sa40)
+
+
+def test_repeatable(torch_mod, sorter):
+    from cascade_amd import workloads
+    T = workloads.generate(5, 1 << 18)
+    a = gpu_sa40(torch_mod, sorter, T)
+    b = gpu_sa40(torch_mod, sorter, T)
+    assert np.array_equal(a, b)
