@@ -1,0 +1,161 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-partition suffix sort on one MI355X.
+
+A step = one whole partition sort (all prefix-doubling generations, text resident in HBM at the
+start, sa40 resident in HBM at the end) of a synthetic partition. Prints ONE JSON line:
+suffixes sorted per second, the roofline of the dominant kernel (the radix pass) from HIP events
+recorded on the sort's own stream, and the reference's CPU sort timed on this host beside it.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 3] [--n N]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+# algorithmic bytes of one radix pass per (key, index) pair: read + write of an 8-byte key and a 5-byte index
+RADIX_PASS_BYTES_PER_PAIR = 2 * (8 + 5)
+
+
+def algorithmic_bytes(n, active):
+    """A = A_0 + sum A_g + A_out with 8-byte keys, 5-byte indices, 4-byte ranks and 8-bit digits:
+    A_0 = 252 n + 9 m_1, A_g = 263 m_g + 9 m_{g+1}, A_out = 14 n; active[g] = m_g, active[0] = n."""
+    m = list(active) + [0]
+    per_gen = [252 * n + 9 * m[1]] + [263 * m[g] + 9 * m[g + 1] for g in range(1, len(active))]
+    return per_gen, 14 * n
+
+
+def cpu_baseline(config, sample_n):
+    """The reference's CPU suffix sort (test/query.cpp:42-55, compiled from its sources into oracle/_ref) on a
+    scaled-down partition of the same construction; falls back to the C restatement where _ref is absent."""
+    import oracle_lib
+    from cascade_amd import workloads
+    T = workloads.generate(config, sample_n)
+    ref = oracle_lib.ref()
+    t0 = time.perf_counter()
+    oracle_lib.build_sa40(T, lib=ref)
+    dt = time.perf_counter() - t0
+    return {
+        "value": sample_n / dt,
+        "unit": "suffixes/s",
+        "cores": 1,
+        "kind": "reference" if ref is not None else "port",
+        "sample": f"config C{config} generated at n={sample_n} (same construction, scaled down), "
+                  f"std::sort + cmp_suffixes, {dt:.1f} s; host has {os.cpu_count()} logical cores",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--config", type=int, default=3, help="workload 1..5 (3 = the 1B-token headline)")
+    ap.add_argument("--n", type=int, default=None, help="override the partition size (scaled construction)")
+    ap.add_argument("--key-words", type=int, default=1)
+    ap.add_argument("--cpu-sample", type=int, default=1 << 26, help="symbols of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--no-verify", action="store_true")
+    ap.add_argument("--generations", action="store_true", help="print the per-generation table to stderr")
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU: a partition is sorted inside one device's HBM and nothing here "
+              "shards it; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from cascade_amd import PartitionSorter, _native, workloads
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    n = args.n if args.n is not None else workloads.default_n(args.config)
+
+    t0 = time.perf_counter()
+    T = workloads.generate(args.config, n)
+    t_gen = time.perf_counter() - t0
+    d_text = torch.from_numpy(T.view(np.int16)).to(dev)
+    del T
+    out = torch.empty(5 * n + 128, dtype=torch.uint8, device=dev)
+    sorter = PartitionSorter(n, key_words=args.key_words)
+    print(f"[bench] C{args.config} n={n} generated in {t_gen:.1f}s; scratch {sorter.bytes_per_suffix() * n / 2**30:.1f} GiB",
+          file=sys.stderr, flush=True)
+
+    for _ in range(args.warmup):
+        sorter.sort(d_text, out=out)
+    torch.cuda.synchronize()
+
+    radix_ms = radix_pairs = radix_launches = 0
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        sorter.sort(d_text, out=out, flags=_native.CSA_FLAG_KERNEL_TIMING)
+        st = sorter.last_stats
+        radix_ms += st["radix_ms"]
+        radix_pairs += st["radix_pairs"]
+        radix_launches += st["radix_launches"]
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = 1e3 * elapsed / args.steps
+    st = sorter.last_stats
+
+    verified = None
+    if not args.no_verify:
+        verified = sorter.verify(d_text, out)
+        if not verified:
+            print("[bench] the device verifier REJECTED the suffix array", file=sys.stderr)
+
+    per_gen, a_out = algorithmic_bytes(n, st["active"])
+    a_total = sum(per_gen) + a_out
+    gen_table = []
+    for g in range(st["generations"]):
+        gbs = per_gen[g] / (st["ms"][g] * 1e-3) / 1e9 if st["ms"][g] > 0 else 0.0
+        gen_table.append({"g": g, "active": st["active"][g], "groups": st["groups"][g], "passes": st["passes"][g],
+                          "ms": round(st["ms"][g], 3), "alg_GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4)})
+    if args.generations:
+        for row in gen_table:
+            print("[gen]", json.dumps(row), file=sys.stderr)
+        print(f"[gen] output ms={st['ms_output']:.3f} device ms_total={st['ms_total']:.3f}", file=sys.stderr)
+
+    # dominant kernel: the one-sweep radix pass, timed per launch with HIP events on the sort's stream
+    avg_launch_ms = radix_ms / radix_launches if radix_launches else 0.0
+    achieved = (RADIX_PASS_BYTES_PER_PAIR * radix_pairs / (radix_ms * 1e-3) / 1e9) if radix_ms > 0 else 0.0
+    roofline = {
+        "bound": "hbm", "kernel": "onesweep_kernel (one radix pass over (key, index) pairs)",
+        "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+        "launches_per_step": radix_launches / args.steps, "avg_launch_ms": round(avg_launch_ms, 4),
+        "pairs_per_launch": radix_pairs / radix_launches if radix_launches else 0,
+        "share_of_step": round(radix_ms / args.steps / ms_per_step, 3),
+    }
+
+    result = {
+        "metric": "suffixes sorted/sec per partition at 1 GPU",
+        "value": n / (ms_per_step * 1e-3),
+        "unit": "suffixes/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u64 keys / u32 ranks", "data": "synthetic",
+        "config": {"workload": workloads.NAMES[args.config], "n": n, "key_words": args.key_words,
+                   "generations": st["generations"], "bit_exact_verified": verified},
+        "roofline": roofline,
+        "job_hbm_frac": round(a_total / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        "job_algorithmic_bytes_per_suffix": round(a_total / n, 1),
+        "generations": gen_table,
+    }
+    if args.cpu_sample > 0:
+        result["cpu_baseline"] = cpu_baseline(args.config, min(args.cpu_sample, n))
+    print(json.dumps(result), flush=True)
+    sorter.close()
+    if verified is False:
+        sys.exit(1)
+
+
+if __name__ == "__main__":
+    main()
