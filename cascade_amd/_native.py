@@ -52,11 +52,12 @@ def load():
     global _lib
     if _lib is not None:
         return _lib
-    if not os.path.exists(HIP_LIB_PATH):
+    path = os.environ.get("CASCADE_HIP_LIB", HIP_LIB_PATH)  # a differently tuned build of the same library
+    if not os.path.exists(path):
         raise ImportError(
-            f"{HIP_LIB_PATH} is missing: build it with `python -m cascade_amd.build` "
+            f"{path} is missing: build it with `python -m cascade_amd.build` "
             "(there is no CPU fallback for the partition sort)")
-    lib = C.CDLL(HIP_LIB_PATH)
+    lib = C.CDLL(path)
     vp, u64, u32, i32 = C.c_void_p, C.c_uint64, C.c_uint32, C.c_int
     lib.csa_bytes_per_suffix.restype = u64
     lib.csa_bytes_per_suffix.argtypes = [i32]

@@ -33,8 +33,15 @@ int fail(int code, const char* fmt, ...)
             return fail(CSA_ERR_HIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), __FILE__, __LINE__); \
     } while (0)
 
-constexpr int SORT_BLOCK = 512;
-constexpr int SORT_ITEMS = 16;
+// tile shape of the radix pass; overridable at build time for tuning runs
+#ifndef CSA_SORT_BLOCK
+#define CSA_SORT_BLOCK 512
+#endif
+#ifndef CSA_SORT_ITEMS
+#define CSA_SORT_ITEMS 16
+#endif
+constexpr int SORT_BLOCK = CSA_SORT_BLOCK;
+constexpr int SORT_ITEMS = CSA_SORT_ITEMS;
 constexpr int SORT_TILE = SORT_BLOCK * SORT_ITEMS;
 constexpr int RANK_BLOCK = 256;
 constexpr int RANK_ITEMS = 8;
@@ -109,22 +116,22 @@ u32 next_epoch(csa_handle* h)
     return h->epoch;
 }
 
-template <int SRC>
-void launch_hist(const HistArgs& a, hipStream_t s)
+u32 hist_blocks(u64 items_per_block, u64 n)
 {
-    u64 blocks = ((u64)a.n + 256 * 16 - 1) / (256 * 16);
-    if (blocks > 4096)
-        blocks = 4096;
-    if (blocks == 0)
-        blocks = 1;
-    hipLaunchKernelGGL((radix_hist_kernel<SRC>), dim3((u32)blocks), dim3(256), 0, s, a);
+    u64 blocks = (n + items_per_block - 1) / items_per_block;
+    if (blocks > 2048)
+        blocks = 2048;
+    return (u32)(blocks ? blocks : 1);
 }
 
 template <int SRC>
 void launch_onesweep(const OnesweepArgs& a, hipStream_t s)
 {
     const u32 tiles = (u32)(((u64)a.n + SORT_TILE - 1) / SORT_TILE);
-    hipLaunchKernelGGL((onesweep_kernel<SORT_BLOCK, SORT_ITEMS, SRC>), dim3(tiles), dim3(SORT_BLOCK), 0, s, a);
+    if (a.shift >= 32)
+        hipLaunchKernelGGL((onesweep_kernel<SORT_BLOCK, SORT_ITEMS, SRC, 1>), dim3(tiles), dim3(SORT_BLOCK), 0, s, a);
+    else
+        hipLaunchKernelGGL((onesweep_kernel<SORT_BLOCK, SORT_ITEMS, SRC, 0>), dim3(tiles), dim3(SORT_BLOCK), 0, s, a);
 }
 
 // Sorts n pairs by the digits of `plan`. The first pass that runs takes its input as `src` says
@@ -140,22 +147,27 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
     *passes_run = 0;
     if (n == 0)
         return CSA_OK;
-    HIP_TRY(hipMemsetAsync(h->ghist, 0, MAX_PASSES * RADIX_BINS * sizeof(u32), s));
-    HistArgs ha;
-    ha.keys = kin;
-    ha.vals = vin;
-    ha.text = text;
-    ha.n = n;
-    ha.text_n = text_n;
-    ha.word = word;
-    ha.plan = plan;
-    ha.ghist = h->ghist;
-    if (src == SRC_PAIRS)
-        launch_hist<SRC_PAIRS>(ha, s);
-    else if (src == SRC_TEXT)
-        launch_hist<SRC_TEXT>(ha, s);
-    else
-        launch_hist<SRC_TEXT_IDX>(ha, s);
+    // ghist[MAX_PASSES][256] followed by the two byte histograms of the text
+    HIP_TRY(hipMemsetAsync(h->ghist, 0, (MAX_PASSES + 2) * RADIX_BINS * sizeof(u32), s));
+    if (src == SRC_PAIRS) {
+        HistArgs ha;
+        ha.keys = kin;
+        ha.vals = vin;
+        ha.text = text;
+        ha.n = n;
+        ha.text_n = text_n;
+        ha.word = word;
+        ha.plan = plan;
+        ha.ghist = h->ghist;
+        hipLaunchKernelGGL(radix_hist_kernel, dim3(hist_blocks(256 * 16, n)), dim3(256), 0, s, ha);
+    } else {
+        // every suffix of the text takes part and the plan is the eight bytes of one key word: the digit
+        // histograms follow from the byte histogram of the text, whatever order the pairs are in
+        u32* bytehist = h->ghist + MAX_PASSES * RADIX_BINS;
+        hipLaunchKernelGGL(text_byte_hist_kernel, dim3(hist_blocks(256 * 8 * 16, text_n)), dim3(256), 0, s, text, text_n,
+                           bytehist);
+        hipLaunchKernelGGL(text_hist_expand_kernel, dim3(1), dim3(256), 0, s, text, text_n, word, bytehist, h->ghist);
+    }
     hipLaunchKernelGGL(radix_scan_hist_kernel, dim3(1), dim3(256), 0, s, h->ghist, h->digit_base, plan.num_passes);
     HIP_TRY(hipGetLastError());
     u32* h_hist = h->h_pinned + 16;
@@ -227,10 +239,16 @@ PassPlan make_plan(int begin_bit, int end_bit)
 {
     PassPlan p;
     p.num_passes = 0;
-    for (int s = begin_bit; s < end_bit && p.num_passes < MAX_PASSES; s += RADIX_BITS) {
+    // digits of up to 8 bits that never straddle bit 32 (a pass reads its digit from one half of the key)
+    int s = begin_bit;
+    while (s < end_bit && p.num_passes < MAX_PASSES) {
+        int bits = end_bit - s < RADIX_BITS ? end_bit - s : RADIX_BITS;
+        if (s < 32 && s + bits > 32)
+            bits = 32 - s;
         p.shift[p.num_passes] = s;
-        p.bits[p.num_passes] = end_bit - s < RADIX_BITS ? end_bit - s : RADIX_BITS;
+        p.bits[p.num_passes] = bits;
         p.num_passes++;
+        s += bits;
     }
     return p;
 }
@@ -473,7 +491,7 @@ int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
     alloc((void**)&h->gprim[0], (cap / 2 + 1) * 4);
     alloc((void**)&h->gprim[1], (cap / 2 + 1) * 4);
     alloc((void**)&h->lookback, h->lookback_words * 8);
-    alloc((void**)&h->ghist, MAX_PASSES * RADIX_BINS * 4);
+    alloc((void**)&h->ghist, (MAX_PASSES + 2) * RADIX_BINS * 4);
     alloc((void**)&h->digit_base, MAX_PASSES * RADIX_BINS * 4);
     alloc((void**)&h->tickets, TICKET_POOL * 4);
     alloc((void**)&h->counts, 16 * 4);

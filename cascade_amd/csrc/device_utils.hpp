@@ -70,18 +70,22 @@ __device__ __forceinline__ u64 lb_load(const u64* p)
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Publishes `aggregate` for `tile` on the chain whose word for tile t lives at chain[t * stride],
-// and returns the combination of the aggregates of tiles [0, tile). Combination is max if IS_MAX,
-// else a 32-bit sum. On a spin timeout (a predecessor never published) sets *err and returns what
-// it has, so that every wave still leaves the kernel.
-template <bool IS_MAX>
-__device__ __forceinline__ u32 lb_exclusive_prefix(u64* chain, u32 stride, u32 tile, u32 epoch, u32 aggregate, u32* err)
+// The protocol in two steps, so that a kernel can publish its aggregate as soon as it is known and wait
+// for its predecessors as late as possible.
+// Step 1: publish `aggregate` of `tile` on the chain whose word for tile t lives at chain[t * stride].
+__device__ __forceinline__ void lb_publish(u64* chain, u32 stride, u32 tile, u32 epoch, u32 aggregate)
 {
-    if (tile == 0) {
-        lb_store(chain, lb_pack(epoch, LB_INCL, aggregate));
+    lb_store(chain + (u64)tile * stride, lb_pack(epoch, tile == 0 ? LB_INCL : LB_AGG, aggregate));
+}
+
+// Step 2: returns the combination of the aggregates of tiles [0, tile) and upgrades the tile's own word
+// to "inclusive". Combination is max if IS_MAX, else a 32-bit sum. On a spin timeout (a predecessor never
+// published) sets *err and returns what it has, so that every wave still leaves the kernel.
+template <bool IS_MAX>
+__device__ __forceinline__ u32 lb_wait_exclusive(u64* chain, u32 stride, u32 tile, u32 epoch, u32 aggregate, u32* err)
+{
+    if (tile == 0)
         return 0;
-    }
-    lb_store(chain + (u64)tile * stride, lb_pack(epoch, LB_AGG, aggregate));
     u32 excl = 0;
     u32 t = tile;
     while (t > 0) {
@@ -106,6 +110,13 @@ __device__ __forceinline__ u32 lb_exclusive_prefix(u64* chain, u32 stride, u32 t
     const u32 incl = IS_MAX ? (excl > aggregate ? excl : aggregate) : excl + aggregate;
     lb_store(chain + (u64)tile * stride, lb_pack(epoch, LB_INCL, incl));
     return excl;
+}
+
+template <bool IS_MAX>
+__device__ __forceinline__ u32 lb_exclusive_prefix(u64* chain, u32 stride, u32 tile, u32 epoch, u32 aggregate, u32* err)
+{
+    lb_publish(chain, stride, tile, epoch, aggregate);
+    return lb_wait_exclusive<IS_MAX>(chain, stride, tile, epoch, aggregate, err);
 }
 
 // ---- K-gram key: four uint16 symbols of the zero-padded text, the first one most significant ----

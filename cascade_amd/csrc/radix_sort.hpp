@@ -51,32 +51,97 @@ struct HistArgs {
     u32* ghist; // [MAX_PASSES][256], zeroed by the caller
 };
 
-template <int SRC>
+// Digit counters live in LDS as hist[pass][bin][copy]: a lane adds to copy (lane % COPIES), so the lanes of
+// a wave that meet on one hot digit (Zipf tokens, runs, group ids) spread over COPIES addresses in COPIES
+// banks instead of serialising on one.
+constexpr int HIST_COPIES = 8;
+
 __global__ __launch_bounds__(256) void radix_hist_kernel(HistArgs a)
 {
-    __shared__ u32 s_hist[MAX_PASSES * RADIX_BINS];
-    for (int i = threadIdx.x; i < MAX_PASSES * RADIX_BINS; i += 256)
+    __shared__ u32 s_hist[MAX_PASSES * RADIX_BINS * HIST_COPIES];
+    for (int i = threadIdx.x; i < MAX_PASSES * RADIX_BINS * HIST_COPIES; i += 256)
         s_hist[i] = 0;
     __syncthreads();
+    const u32 copy = threadIdx.x & (HIST_COPIES - 1);
     const u64 stride = (u64)gridDim.x * 256;
     for (u64 i = (u64)blockIdx.x * 256 + threadIdx.x; i < a.n; i += stride) {
-        u64 key;
-        if (SRC == SRC_PAIRS)
-            key = a.keys[i];
-        else if (SRC == SRC_TEXT)
-            key = load_kgram(a.text, a.text_n, (u32)i, a.word); // a histogram does not care about the order
-        else
-            key = load_kgram(a.text, a.text_n, a.vals[i], a.word);
+        const u64 key = a.keys[i];
         for (int p = 0; p < a.plan.num_passes; ++p) {
             const u32 d = (u32)(key >> a.plan.shift[p]) & ((1u << a.plan.bits[p]) - 1u);
-            atomicAdd(&s_hist[p * RADIX_BINS + d], 1u);
+            atomicAdd(&s_hist[(p * RADIX_BINS + d) * HIST_COPIES + copy], 1u);
         }
     }
     __syncthreads();
     for (int i = threadIdx.x; i < a.plan.num_passes * RADIX_BINS; i += 256) {
-        const u32 v = s_hist[i];
+        u32 v = 0;
+#pragma unroll
+        for (int c = 0; c < HIST_COPIES; ++c)
+            v += s_hist[i * HIST_COPIES + c];
         if (v)
             atomicAdd(&a.ghist[i], v);
+    }
+}
+
+// Histogram of the low and of the high byte of every symbol of the text: bytehist[0][d], bytehist[1][d].
+// The eight digit histograms of a K-gram key word follow from these two (text_hist_expand_kernel).
+constexpr int TEXT_HIST_COPIES = 16;
+
+__global__ __launch_bounds__(256) void text_byte_hist_kernel(const u16* __restrict__ text, u32 n, u32* bytehist)
+{
+    __shared__ u32 s_hist[2 * RADIX_BINS * TEXT_HIST_COPIES];
+    for (int i = threadIdx.x; i < 2 * RADIX_BINS * TEXT_HIST_COPIES; i += 256)
+        s_hist[i] = 0;
+    __syncthreads();
+    const u32 copy = threadIdx.x & (TEXT_HIST_COPIES - 1);
+    const u64 stride = (u64)gridDim.x * 256 * 8;
+    for (u64 i = ((u64)blockIdx.x * 256 + threadIdx.x) * 8; i < n; i += stride) {
+        u16 sym[8];
+        if (i + 8 <= n) {
+            __builtin_memcpy(sym, text + i, 16); // 16-byte aligned: hipMalloc base + 16 * k
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                sym[k] = i + k < n ? text[i + k] : 0;
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            if (i + k < n) {
+                atomicAdd(&s_hist[(0 * RADIX_BINS + (sym[k] & 0xFFu)) * TEXT_HIST_COPIES + copy], 1u);
+                atomicAdd(&s_hist[(1 * RADIX_BINS + (sym[k] >> 8)) * TEXT_HIST_COPIES + copy], 1u);
+            }
+        }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 2 * RADIX_BINS; i += 256) {
+        u32 v = 0;
+#pragma unroll
+        for (int c = 0; c < TEXT_HIST_COPIES; ++c)
+            v += s_hist[i * TEXT_HIST_COPIES + c];
+        if (v)
+            atomicAdd(&bytehist[i], v);
+    }
+}
+
+// ghist[p][d] for the 8 byte-wide passes of key word `word` over all n suffixes. Pass p looks at byte (p & 1) of
+// the symbol at offset pos = 4 * word + 3 - p / 2 of each suffix, i.e. at T[pos .. n) followed by min(pos, n) padding
+// zeros: the whole-text byte histogram minus the first min(pos, n) symbols, plus that many zeros.
+__global__ __launch_bounds__(256) void text_hist_expand_kernel(const u16* __restrict__ text, u32 n, u32 word,
+                                                               const u32* __restrict__ bytehist, u32* ghist)
+{
+    const u32 d = threadIdx.x;
+    for (int p = 0; p < 8; ++p) {
+        const u32 byte = p & 1;
+        const u32 pos = 4 * word + 3 - p / 2;
+        const u32 cut = pos < n ? pos : n;
+        u32 v = bytehist[byte * RADIX_BINS + d];
+        for (u32 i = 0; i < cut; ++i) {
+            const u32 b = byte ? (text[i] >> 8) : (text[i] & 0xFFu);
+            if (b == d)
+                --v;
+        }
+        if (d == 0)
+            v += cut;
+        ghist[p * RADIX_BINS + d] = v;
     }
 }
 
@@ -118,8 +183,15 @@ struct OnesweepArgs {
     u32* err;
 };
 
-template <int BLOCK, int ITEMS, int SRC>
-__global__ __launch_bounds__(BLOCK) void onesweep_kernel(OnesweepArgs a)
+// minimum waves per SIMD the compiler must leave room for (caps the VGPR budget of the radix pass)
+#ifndef CSA_SORT_MIN_WAVES
+#define CSA_SORT_MIN_WAVES 1
+#endif
+
+// HI selects the 32-bit half of the key that holds this pass's digit (digits never straddle the halves:
+// shifts are multiples of 8), so that the digit is one bit-field extract of a 32-bit register.
+template <int BLOCK, int ITEMS, int SRC, int HI>
+__global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(OnesweepArgs a)
 {
     constexpr int TILE = BLOCK * ITEMS;
     constexpr int WAVES = BLOCK / WAVE;
@@ -144,7 +216,10 @@ __global__ __launch_bounds__(BLOCK) void onesweep_kernel(OnesweepArgs a)
     const u32 tile = s_tile;
     const u64 base = (u64)tile * TILE;
     const u32 valid = (u32)((u64)a.n - base < (u64)TILE ? (u64)a.n - base : (u64)TILE);
-    const u32 mask = (1u << a.bits) - 1u;
+    const u32 sh = (u32)a.shift & 31u;
+    const u32 bits = (u32)a.bits;
+    const u32 mask = (1u << bits) - 1u;
+#define CSA_DIGIT(k64) __builtin_amdgcn_ubfe(HI ? (u32)((k64) >> 32) : (u32)(k64), sh, bits)
 
     // ---- load: wave-striped, so that consecutive lanes read consecutive pairs ----
     u64 key[ITEMS];
@@ -171,31 +246,34 @@ __global__ __launch_bounds__(BLOCK) void onesweep_kernel(OnesweepArgs a)
     }
 
     // ---- rank each pair among the pairs of its wave that share its digit ----
+    // For every digit bit, (ballot of "bit set") XOR (all-ones if my own bit is set) has a 0 exactly at the lanes
+    // that agree with me on that bit; OR-ed over the bits, `differ` marks the lanes whose digit is not mine.
     volatile u32* whist = s_whist + w * RADIX_BINS;
-    const u64 lt_mask = (1ull << lane) - 1ull;
     u32 pos[ITEMS];
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
-        const u32 d = (u32)(key[k] >> a.shift) & mask;
-        u64 same = ~0ull;
+        const u32 d = CSA_DIGIT(key[k]);
+        u32 differ_lo = 0, differ_hi = 0;
 #pragma unroll
         for (int b = 0; b < RADIX_BITS; ++b) {
-            const bool bit = (d >> b) & 1u;
-            const u64 bal = __ballot(bit);
-            same &= bit ? bal : ~bal;
+            const u32 mine = (u32)__builtin_amdgcn_sbfe(d, b, 1); // 0 or 0xFFFFFFFF
+            const u64 bal = __ballot(mine != 0);
+            differ_lo |= (u32)bal ^ mine;
+            differ_hi |= (u32)(bal >> 32) ^ mine;
         }
-        const u32 before = __popcll(same & lt_mask);
+        const u32 same_lo = ~differ_lo, same_hi = ~differ_hi;
+        const u32 before = __builtin_amdgcn_mbcnt_hi(same_hi, __builtin_amdgcn_mbcnt_lo(same_lo, 0u));
         const u32 prev = whist[d];
         __builtin_amdgcn_wave_barrier();
         if (before == 0)
-            whist[d] = prev + __popcll(same);
+            whist[d] = prev + __popc(same_lo) + __popc(same_hi);
         __builtin_amdgcn_wave_barrier();
         pos[k] = prev + before;
     }
     __syncthreads();
 
-    // ---- one thread per digit: offsets of the waves inside the tile, tile totals, look-back ----
-    u32 total = 0;
+    // ---- one thread per digit: offsets of the waves inside the tile, tile totals; publish them at once ----
+    u32 total = 0, real = 0;
     if (t < RADIX_BINS) {
 #pragma unroll
         for (int ww = 0; ww < WAVES; ++ww) {
@@ -203,8 +281,13 @@ __global__ __launch_bounds__(BLOCK) void onesweep_kernel(OnesweepArgs a)
             s_whist[ww * RADIX_BINS + t] = total;
             total += c;
         }
+        real = total;
+        if (t == mask)
+            real -= (u32)TILE - valid; // padding pairs all carry the largest digit
+        lb_publish(a.lookback + t, RADIX_BINS, tile, a.epoch, real);
     }
     // exclusive scan of the 256 totals (padding included: it occupies LDS slots too)
+    u32 binstart = 0;
     {
         const u32 incl = wave_incl_sum(total);
         if (t < RADIX_BINS && lane == 63u)
@@ -214,33 +297,33 @@ __global__ __launch_bounds__(BLOCK) void onesweep_kernel(OnesweepArgs a)
             u32 prefix = 0;
             for (u32 ww = 0; ww < w; ++ww)
                 prefix += s_wsum[ww];
-            const u32 binstart = prefix + incl - total;
+            binstart = prefix + incl - total;
             s_binstart[t] = binstart;
-            u32 real = total;
-            if (t == mask)
-                real -= (u32)TILE - valid; // padding pairs all carry the largest digit
-            const u32 excl = lb_exclusive_prefix<false>(a.lookback + t, RADIX_BINS, tile, a.epoch, real, a.err);
-            s_delta[t] = a.digit_base[t] + excl - binstart; // wraps; added back to an LDS slot below
         }
     }
     __syncthreads();
 
-    // ---- order the tile in LDS, then write runs of equal digits to their global places ----
+    // ---- order the tile in LDS (needs tile-local offsets only), then wait for the tiles before this one ----
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
-        const u32 d = (u32)(key[k] >> a.shift) & mask;
+        const u32 d = CSA_DIGIT(key[k]);
         pos[k] += s_binstart[d] + s_whist[w * RADIX_BINS + d];
         s_keys[pos[k]] = key[k];
     }
+    if (t < RADIX_BINS) {
+        const u32 excl = lb_wait_exclusive<false>(a.lookback + t, RADIX_BINS, tile, a.epoch, real, a.err);
+        s_delta[t] = a.digit_base[t] + excl - binstart; // wraps; added back to an LDS slot below
+    }
     __syncthreads();
+
+    // ---- write runs of equal digits to their global places ----
     u32 dst[ITEMS];
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         const u32 q = k * BLOCK + t;
         if (q < valid) {
             const u64 kk = s_keys[q];
-            const u32 d = (u32)(kk >> a.shift) & mask;
-            dst[k] = q + s_delta[d];
+            dst[k] = q + s_delta[CSA_DIGIT(kk)];
             a.keys_out[dst[k]] = kk;
         }
     }
@@ -256,6 +339,7 @@ __global__ __launch_bounds__(BLOCK) void onesweep_kernel(OnesweepArgs a)
         if (q < valid)
             a.vals_out[dst[k]] = s_vals[q];
     }
+#undef CSA_DIGIT
 }
 
 } // namespace csa
