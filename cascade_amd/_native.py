@@ -28,6 +28,7 @@ class CsaStats(C.Structure):
         ("generations", C.c_int32),
         ("active", C.c_uint64 * CSA_MAX_GENERATIONS),
         ("groups", C.c_uint64 * CSA_MAX_GENERATIONS),
+        ("big", C.c_uint64 * CSA_MAX_GENERATIONS),
         ("passes", C.c_int32 * CSA_MAX_GENERATIONS),
         ("ms", C.c_float * CSA_MAX_GENERATIONS),
         ("ms_output", C.c_float),

@@ -46,6 +46,14 @@ constexpr int SORT_TILE = SORT_BLOCK * SORT_ITEMS;
 constexpr int RANK_BLOCK = 256;
 constexpr int RANK_ITEMS = 8;
 constexpr int RANK_TILE = RANK_BLOCK * RANK_ITEMS;
+// groups of up to SMALL_MAXG suffixes are sorted inside one tile of the small-group kernel
+#ifndef CSA_SMALL_MAXG
+#define CSA_SMALL_MAXG 64
+#endif
+constexpr int SMALL_BLOCK = 256;
+constexpr int SMALL_ITEMS = 8;
+constexpr int SMALL_TILE = SMALL_BLOCK * SMALL_ITEMS;
+constexpr int SMALL_MAXG = CSA_SMALL_MAXG;
 constexpr u32 TICKET_POOL = 4096;
 constexpr int EVENT_POOL = 2 * CSA_MAX_GENERATIONS * MAX_PASSES * 2;
 
@@ -65,11 +73,12 @@ struct csa_handle {
     int device = 0;
     u64 cap = 0;
     int key_words = 1;
-    u64* key[2] = {nullptr, nullptr};
-    u32* idx[3] = {nullptr, nullptr, nullptr};
+    u64* key[3] = {nullptr, nullptr, nullptr};
+    u32* idx[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
     u32* gid = nullptr;
     u32* rank = nullptr;
     u32* gprim[2] = {nullptr, nullptr};
+    u32* gstart[2] = {nullptr, nullptr};
     u64* lookback = nullptr;
     u64 lookback_words = 0;
     u32* ghist = nullptr;      // [MAX_PASSES][256]
@@ -268,15 +277,26 @@ int ensure_events(csa_handle* h, bool kernel_timing)
     return CSA_OK;
 }
 
-int read_counts(Launch& L, u32* survivors, u32* groups)
+// counts: [0] survivors, [1] their groups, [2] device error flag, [3] verifier flag, [4] members of large groups
+int read_counts(Launch& L, u32* survivors, u32* groups, u32* big)
 {
     csa_handle* h = L.h;
-    HIP_TRY(hipMemcpyAsync(h->h_pinned, h->counts, 4 * sizeof(u32), hipMemcpyDeviceToHost, L.stream));
+    HIP_TRY(hipMemcpyAsync(h->h_pinned, h->counts, 8 * sizeof(u32), hipMemcpyDeviceToHost, L.stream));
     HIP_TRY(hipStreamSynchronize(L.stream));
-    if (h->h_pinned[2])
-        return fail(CSA_ERR_INTERNAL, "a look-back wait ran into its spin limit");
-    *survivors = h->h_pinned[0];
-    *groups = h->h_pinned[1];
+    if (h->h_pinned[2]) {
+        static const char* const what[] = {"", "a look-back wait ran into its spin limit",
+                                           "an active suffix lies outside its group's range (small-group sort)",
+                                           "a large-group member was sent outside the active list (place)",
+                                           "a rank or suffix index out of range in the sorted active list (rerank)"};
+        const u32 code = h->h_pinned[2];
+        return fail(CSA_ERR_INTERNAL, "device invariant %u failed: %s", code, code < 5 ? what[code] : "unknown");
+    }
+    if (survivors)
+        *survivors = h->h_pinned[0];
+    if (groups)
+        *groups = h->h_pinned[1];
+    if (big)
+        *big = h->h_pinned[4];
     return CSA_OK;
 }
 
@@ -335,11 +355,14 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
         passes += p1;
     }
     u64* k_sorted = K[cur];
-    u32* sa32 = V[cur];      // from here on the suffix array under construction
-    u32* act_a = V[cur ^ 1]; // the two index arrays left for the active lists
-    u32* act_b = h->idx[2];
-    u64* key_a = K[cur ^ 1]; // key array that travels with act_a
-    u64* key_b = k_sorted;   // free once generation 0 has been ranked; travels with act_b
+    u32* sa32 = V[cur]; // from here on the suffix array under construction
+    // roles of the remaining arrays in generations t >= 1
+    u32* ax = V[cur ^ 1];        // active list: suffixes ...
+    u32* agid = h->gid;          // ... and their dense group ids
+    u64* key_out = K[cur ^ 1];   // the active list sorted by (group, rank[x + h])
+    u32* x_out = h->idx[2];
+    u64* bkey[2] = {h->key[2], k_sorted}; // large groups on their way through the radix sort
+    u32* bx[2] = {h->idx[3], h->idx[4]};  // (k_sorted is free once generation 0 has been ranked)
 
     RerankArgs ra;
     memset(&ra, 0, sizeof(ra));
@@ -355,14 +378,15 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     ra.gprim_in = nullptr;
     ra.rank = h->rank;
     ra.sa32 = sa32;
-    ra.sufs_out = act_a;
-    ra.gids_out = h->gid;
+    ra.sufs_out = ax;
+    ra.gids_out = agid;
     ra.gprim_out = h->gprim[0];
+    ra.gstart_out = h->gstart[0];
     rc = launch_rerank(L, ra);
     if (rc)
         return rc;
-    u32 m = 0, groups = 0;
-    rc = read_counts(L, &m, &groups);
+    u32 m = 0, groups = 0, big = 0;
+    rc = read_counts(L, &m, &groups, &big);
     if (rc)
         return rc;
     st->passes[0] = passes;
@@ -372,7 +396,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
 
     // ---- generations t >= 1 (reference loop: src/GPU_SACA.cu:1999-2103) ----
     int gen = 1;
-    int gp = 0; // gprim[gp] holds the first ranks of the current groups
+    int gp = 0; // gprim[gp] / gstart[gp] describe the current groups
     const int sec_bits = bit_length(n > 1 ? n - 1 : 1);
     u64 h_ctx = ell;
     while (m > 0) {
@@ -380,17 +404,61 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
             return fail(CSA_ERR_INTERNAL, "generation cap reached with %u suffixes still active", m);
         st->active[gen] = m;
         st->groups[gen] = groups;
-        const u32 hh = (u32)h_ctx;
-        hipLaunchKernelGGL(gather_keys_kernel, dim3((m + 255) / 256), dim3(256), 0, s, act_a, h->gid, h->rank, m, n, hh,
-                           sec_bits, key_a);
-        const int gid_bits = bit_length(groups > 1 ? groups - 1 : 0);
-        const PassPlan plan = make_plan(0, sec_bits + gid_bits);
-        rc = radix_sort(L, SRC_PAIRS, nullptr, n, 0, 0, key_a, act_a, key_b, act_b, m, plan, &in_out, &passes);
+        // small groups are sorted in place by one kernel; the members of large groups are set aside
+        HIP_TRY(hipMemsetAsync(h->counts + 4, 0, sizeof(u32), s));
+        SmallSortArgs sa;
+        sa.sufs = ax;
+        sa.gids = agid;
+        sa.gstart = h->gstart[gp];
+        sa.rank = h->rank;
+        sa.m = m;
+        sa.n = n;
+        sa.h = (u32)h_ctx;
+        sa.sec_bits = sec_bits;
+        sa.groups = groups;
+        sa.err = h->counts + 2;
+        sa.keys_out = key_out;
+        sa.sufs_out = x_out;
+        sa.big_keys = bkey[0];
+        sa.big_sufs = bx[0];
+        sa.big_count = h->counts + 4;
+        hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG>),
+                           dim3((m + SMALL_TILE - 1) / SMALL_TILE), dim3(SMALL_BLOCK), 0, s, sa);
+        HIP_TRY(hipGetLastError());
+        rc = read_counts(L, nullptr, nullptr, &big);
         if (rc)
             return rc;
+        st->big[gen] = big;
+        passes = 0;
+        if (big > 0) {
+            const int gid_bits = bit_length(groups > 1 ? groups - 1 : 0);
+            const PassPlan plan = make_plan(0, sec_bits + gid_bits);
+            rc = radix_sort(L, SRC_PAIRS, nullptr, n, 0, 0, bkey[0], bx[0], bkey[1], bx[1], big, plan, &in_out, &passes);
+            if (rc)
+                return rc;
+            PlaceArgs pa;
+            pa.big_keys = bkey[in_out];
+            pa.big_sufs = bx[in_out];
+            pa.mb = big;
+            pa.m = m;
+            pa.groups = groups;
+            pa.sec_bits = sec_bits;
+            pa.gstart = h->gstart[gp];
+            pa.keys_out = key_out;
+            pa.sufs_out = x_out;
+            pa.lookback = h->lookback;
+            pa.epoch = next_epoch(h);
+            pa.err = h->counts + 2;
+            rc = next_ticket(L, &pa.ticket);
+            if (rc)
+                return rc;
+            hipLaunchKernelGGL((place_big_kernel<RANK_BLOCK, RANK_ITEMS>), dim3((big + RANK_TILE - 1) / RANK_TILE),
+                               dim3(RANK_BLOCK), 0, s, pa);
+            HIP_TRY(hipGetLastError());
+        }
         memset(&ra, 0, sizeof(ra));
-        ra.keys = in_out ? key_b : key_a;
-        ra.sufs = in_out ? act_b : act_a;
+        ra.keys = key_out;
+        ra.sufs = x_out;
         ra.m = m;
         ra.gen0 = 0;
         ra.key_words = h->key_words;
@@ -399,20 +467,18 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
         ra.ell = ell;
         ra.text = d_text;
         ra.gprim_in = h->gprim[gp];
+        ra.groups_in = groups;
         ra.rank = h->rank;
         ra.sa32 = sa32;
-        ra.sufs_out = in_out ? act_a : act_b;
-        ra.gids_out = h->gid;
+        ra.sufs_out = ax;
+        ra.gids_out = agid;
         ra.gprim_out = h->gprim[gp ^ 1];
+        ra.gstart_out = h->gstart[gp ^ 1];
         rc = launch_rerank(L, ra);
         if (rc)
             return rc;
-        if (in_out == 0) { // survivors went to act_b: it becomes the current list
-            std::swap(act_a, act_b);
-            std::swap(key_a, key_b);
-        }
         gp ^= 1;
-        rc = read_counts(L, &m, &groups);
+        rc = read_counts(L, &m, &groups, nullptr);
         if (rc)
             return rc;
         st->passes[gen] = passes;
@@ -454,8 +520,8 @@ const char* csa_last_error(void) { return g_err; }
 uint64_t csa_bytes_per_suffix(int key_words)
 {
     (void)key_words;
-    // two key arrays (8 B), three index arrays (4 B), group ids, ranks, two half-size group tables
-    return 2 * 8 + 3 * 4 + 4 + 4 + 4;
+    // three key arrays (8 B), five index arrays (4 B), group ids, ranks, four half-size group tables
+    return 3 * 8 + 5 * 4 + 4 + 4 + 4 * 2;
 }
 
 int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
@@ -482,14 +548,16 @@ int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
         if (e == hipSuccess)
             e = hipMalloc(p, bytes ? bytes : 4);
     };
-    alloc((void**)&h->key[0], cap * 8);
-    alloc((void**)&h->key[1], cap * 8);
     for (int i = 0; i < 3; ++i)
+        alloc((void**)&h->key[i], cap * 8);
+    for (int i = 0; i < 5; ++i)
         alloc((void**)&h->idx[i], cap * 4);
     alloc((void**)&h->gid, cap * 4);
     alloc((void**)&h->rank, cap * 4);
     alloc((void**)&h->gprim[0], (cap / 2 + 1) * 4);
     alloc((void**)&h->gprim[1], (cap / 2 + 1) * 4);
+    alloc((void**)&h->gstart[0], (cap / 2 + 2) * 4);
+    alloc((void**)&h->gstart[1], (cap / 2 + 2) * 4);
     alloc((void**)&h->lookback, h->lookback_words * 8);
     alloc((void**)&h->ghist, (MAX_PASSES + 2) * RADIX_BINS * 4);
     alloc((void**)&h->digit_base, MAX_PASSES * RADIX_BINS * 4);
@@ -519,10 +587,12 @@ void csa_destroy(csa_handle* h)
 {
     if (!h)
         return;
-    (void)hipFree(h->key[0]);
-    (void)hipFree(h->key[1]);
     for (int i = 0; i < 3; ++i)
+        (void)hipFree(h->key[i]);
+    for (int i = 0; i < 5; ++i)
         (void)hipFree(h->idx[i]);
+    (void)hipFree(h->gstart[0]);
+    (void)hipFree(h->gstart[1]);
     (void)hipFree(h->gid);
     (void)hipFree(h->rank);
     (void)hipFree(h->gprim[0]);
@@ -657,8 +727,7 @@ int csa_radix_sort_pairs_dev(csa_handle* h, uint64_t* d_keys, uint32_t* d_vals, 
         HIP_TRY(hipMemcpyAsync(d_keys, h->key[0], n * 8, hipMemcpyDeviceToDevice, L.stream));
         HIP_TRY(hipMemcpyAsync(d_vals, h->idx[0], n * 4, hipMemcpyDeviceToDevice, L.stream));
     }
-    u32 a = 0, b = 0;
-    return read_counts(L, &a, &b);
+    return read_counts(L, nullptr, nullptr, nullptr);
 }
 
 int csa_verify_sa40_dev(csa_handle* h, const uint16_t* d_text, uint64_t n, uint64_t index_base,

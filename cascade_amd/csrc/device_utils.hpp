@@ -14,6 +14,13 @@ namespace csa {
 
 constexpr int WAVE = 64;
 
+// Values of the device error word (0 = no error). Kernels report a broken invariant there instead of
+// reading or writing out of bounds; the host turns it into CSA_ERR_INTERNAL.
+constexpr unsigned DEV_ERR_LOOKBACK_TIMEOUT = 1;
+constexpr unsigned DEV_ERR_SMALLSORT_TABLES = 2;
+constexpr unsigned DEV_ERR_PLACE_RANGE = 3;
+constexpr unsigned DEV_ERR_RERANK_RANGE = 4;
+
 __device__ __forceinline__ u32 lane_id() { return __lane_id(); }
 
 // ---- wave64 inclusive scans by shuffles ----

@@ -1,6 +1,6 @@
-// Kernels of the prefix-doubling generations: rank assignment / compaction after a sort, the
-// rank[x + h] gather that builds the next generation's keys, sa40 emission, K-gram packing and the
-// device-side suffix-array check.
+// Kernels of the prefix-doubling generations: rank assignment / compaction after a sort, the in-tile
+// sort of small groups (which gathers rank[x + h]), the return of radix-sorted large groups, sa40
+// emission, K-gram packing and the device-side suffix-array check.
 #pragma once
 
 #include "device_utils.hpp"
@@ -33,11 +33,13 @@ struct RerankArgs {
     u32 ell;       // symbols in the generation-0 key
     const u16* text;
     const u32* gprim_in; // generation t: first rank of each incoming group
+    u32 groups_in;       // generation t: number of incoming groups
     u32* rank;           // [n] by text position
     u32* sa32;           // [n] suffix array under construction
     u32* sufs_out;       // next active list
     u32* gids_out;
     u32* gprim_out;
+    u32* gstart_out; // index in the next active list where each new group starts; [groups] = survivors
     u32* counts; // [0] = survivors, [1] = their groups (written by the last tile)
     u64* lookback; // [tiles][4]
     u32* ticket;
@@ -52,6 +54,7 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
     constexpr int WAVES = BLOCK / WAVE;
     __shared__ u32 s_wagg[WAVES][4];
     __shared__ u32 s_tileprefix[4];
+    __shared__ u32 s_tiletotal[4];
     __shared__ u32 s_tile;
 
     const u32 t = threadIdx.x;
@@ -143,10 +146,14 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
         else
             excl = lb_exclusive_prefix<false>(a.lookback + lane, 4, tile, a.epoch, agg, a.err);
         s_tileprefix[lane] = excl;
-        if ((u64)(tile + 1) * TILE >= m && lane >= 2) // the last tile knows the totals
-            a.counts[lane - 2] = excl + agg;
+        s_tiletotal[lane] = excl + agg;
     }
     __syncthreads();
+    if (t == 0 && (u64)(tile + 1) * TILE >= m) { // the last tile knows the totals
+        a.counts[0] = s_tiletotal[2];
+        a.counts[1] = s_tiletotal[3];
+        a.gstart_out[s_tiletotal[3]] = s_tiletotal[2]; // one-past-the-end entry: gstart[groups] = survivors
+    }
     u32 ra = xa > s_tileprefix[0] ? xa : s_tileprefix[0];
     u32 rb = xb > s_tileprefix[1] ? xb : s_tileprefix[1];
     u32 rc = xc + s_tileprefix[2];
@@ -165,9 +172,15 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
                 rb = (u32)c;
             const u32 x = suf[k + 1];
             u32 prim = 0;
-            if (!a.gen0)
-                prim = a.gprim_in[(u32)(key[k + 1] >> a.sec_bits)];
+            if (!a.gen0) {
+                const u32 g = (u32)(key[k + 1] >> a.sec_bits);
+                prim = g < a.groups_in ? a.gprim_in[g] : a.n;
+            }
             const u32 nr = prim + (ra - rb);
+            if (nr >= a.n || x >= a.n) { // a corrupt sorted list: report it instead of writing out of bounds
+                atomicExch(a.err, DEV_ERR_RERANK_RANGE);
+                continue;
+            }
             if (a.gen0 || ra != rb)
                 a.rank[x] = nr;
             if (single) {
@@ -176,6 +189,7 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
             } else {
                 if (ka) {
                     a.gprim_out[rh] = nr;
+                    a.gstart_out[rh] = rc;
                     rh++;
                 }
                 a.sufs_out[rc] = x;
@@ -186,19 +200,196 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
     }
 }
 
-// key[c] = (group id << sec_bits) | rank[x + h]; every active x has x + h < n
-// (reference: the joined key of include/GPU_SACA.cuh:362-389 with secondary = the rank of suffix x + ctx/2,
-// include/bit-layout.hpp:128; here the rank is read straight from HBM by text position).
-__global__ __launch_bounds__(256) void gather_keys_kernel(const u32* __restrict__ sufs, const u32* __restrict__ gids,
-                                                          const u32* __restrict__ rank, u32 m, u32 n, u32 h,
-                                                          int sec_bits, u64* __restrict__ keys)
+// ---------------------------------------------------------------------------------------------
+// Generation t >= 1, small groups: gather rank[x + h] and sort inside each group in one pass.
+//
+// The active list is grouped (members of a group are contiguous, group g = [gstart[g], gstart[g + 1])).
+// A tile stages the gathered ranks of its elements plus a halo of MAXG elements on either side in LDS;
+// each element of a group of at most MAXG members then counts the members that sort before it
+// (smaller rank[x + h], ties by position) and writes its (key, suffix) pair straight to its sorted
+// place. Elements of larger groups are appended, in no particular order, to a list that goes through
+// the radix sort instead (place_big_kernel brings them back).
+// Replaces, for such groups, the 62-bit key sort of the reference (src/GPU_SACA.cu:1841-1871).
+// ---------------------------------------------------------------------------------------------
+
+struct SmallSortArgs {
+    const u32* sufs;   // active list
+    const u32* gids;
+    const u32* gstart; // [groups + 1]
+    const u32* rank;
+    u32 m, n, h;
+    u32 groups;
+    int sec_bits;
+    u32* err; // set to a DEV_ERR_* code if an invariant of the group tables is violated
+    u64* keys_out; // sorted active list (small groups written here directly)
+    u32* sufs_out;
+    u64* big_keys; // elements of groups larger than MAXG
+    u32* big_sufs;
+    u32* big_count; // zero before the launch
+};
+
+template <int BLOCK, int ITEMS, int MAXG>
+__global__ __launch_bounds__(BLOCK) void smallsort_kernel(SmallSortArgs a)
 {
-    const u64 c = (u64)blockIdx.x * 256 + threadIdx.x;
-    if (c >= m)
-        return;
-    const u64 src = (u64)sufs[c] + h;
-    const u32 sec = src < n ? rank[src] : 0u;
-    keys[c] = ((u64)gids[c] << sec_bits) | (u64)sec;
+    constexpr int TILE = BLOCK * ITEMS;
+    constexpr int SPAN = TILE + 2 * MAXG;
+    __shared__ u32 s_sec[SPAN];
+
+    const u32 t = threadIdx.x;
+    const long long t0 = (long long)blockIdx.x * TILE;
+    const long long lo = t0 - MAXG; // list index of s_sec[0]
+
+    u32 x[ITEMS], sec[ITEMS];
+    // own elements (striped: consecutive lanes hold consecutive elements) and the two halos
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const long long e = t0 + k * BLOCK + t;
+        x[k] = 0;
+        sec[k] = 0;
+        if (e < (long long)a.m) {
+            x[k] = a.sufs[e];
+            const u64 src = (u64)x[k] + a.h;
+            sec[k] = src < a.n ? a.rank[src] : 0u;
+            s_sec[MAXG + k * BLOCK + t] = sec[k];
+        }
+    }
+    for (int i = t; i < 2 * MAXG; i += BLOCK) {
+        const int slot = i < MAXG ? i : TILE + i; // [0, MAXG) and [MAXG + TILE, SPAN)
+        const long long e = lo + slot;
+        if (e >= 0 && e < (long long)a.m) {
+            const u64 src = (u64)a.sufs[e] + a.h;
+            s_sec[slot] = src < a.n ? a.rank[src] : 0u;
+        }
+    }
+    __syncthreads();
+
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const long long e = t0 + k * BLOCK + t;
+        bool in = e < (long long)a.m;
+        u32 g = 0, gs = 0, ge = 0;
+        if (in) {
+            g = a.gids[e];
+            if (g < a.groups) {
+                gs = a.gstart[g];
+                ge = a.gstart[g + 1];
+            }
+            if (g >= a.groups || !((long long)gs <= e && e < (long long)ge && ge <= a.m)) {
+                atomicExch(a.err, DEV_ERR_SMALLSORT_TABLES); // the element is not inside its group's range
+                in = false;
+            }
+        }
+        const bool big = in && (ge - gs > (u32)MAXG);
+        const u64 key = ((u64)g << a.sec_bits) | (u64)sec[k];
+        if (in && !big) {
+            u32 cnt = 0;
+            for (u32 j = gs; j < ge; ++j) {
+                const u32 v = s_sec[(long long)j - lo];
+                cnt += (v < sec[k] || (v == sec[k] && (long long)j < e)) ? 1u : 0u;
+            }
+            a.keys_out[gs + cnt] = key;
+            a.sufs_out[gs + cnt] = x[k];
+        }
+        // big groups: one atomic per wave reserves the slots
+        const u64 bal = __ballot(big);
+        if (bal) {
+            const u32 lane = lane_id();
+            const u32 leader = (u32)__builtin_ctzll(bal);
+            u32 basepos = 0;
+            if (lane == leader)
+                basepos = atomicAdd(a.big_count, (u32)__popcll(bal));
+            basepos = __shfl(basepos, leader);
+            if (big) {
+                const u32 slot = basepos + (u32)__popcll(bal & ((1ull << lane) - 1ull));
+                a.big_keys[slot] = key;
+                a.big_sufs[slot] = x[k];
+            }
+        }
+    }
+}
+
+// Brings the radix-sorted elements of the large groups back into the sorted active list: the k-th sorted
+// element of group g goes to gstart[g] + (k - index of g's first element). One max look-back chain finds
+// that first element.
+struct PlaceArgs {
+    const u64* big_keys; // sorted by (group id, rank[x + h])
+    const u32* big_sufs;
+    u32 mb;
+    u32 m;      // size of the active list
+    u32 groups; // its groups
+    int sec_bits;
+    const u32* gstart;
+    u64* keys_out;
+    u32* sufs_out;
+    u64* lookback; // [tiles]
+    u32* ticket;
+    u32 epoch;
+    u32* err;
+};
+
+template <int BLOCK, int ITEMS>
+__global__ __launch_bounds__(BLOCK) void place_big_kernel(PlaceArgs a)
+{
+    constexpr int TILE = BLOCK * ITEMS;
+    constexpr int WAVES = BLOCK / WAVE;
+    __shared__ u32 s_wagg[WAVES];
+    __shared__ u32 s_prefix;
+    __shared__ u32 s_tile;
+    const u32 t = threadIdx.x;
+    const u32 lane = t & 63u;
+    const u32 w = t >> 6;
+    if (t == 0)
+        s_tile = atomicAdd(a.ticket, 1u);
+    __syncthreads();
+    const u32 tile = s_tile;
+    const u64 base = (u64)tile * TILE + (u64)t * ITEMS;
+
+    u64 key[ITEMS + 1]; // element base - 1 first
+#pragma unroll
+    for (int k = 0; k < ITEMS + 1; ++k) {
+        const u64 c = base + k;
+        key[k] = (c >= 1 && c - 1 < a.mb) ? a.big_keys[c - 1] : 0;
+    }
+    u32 lhead = 0;
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const u64 c = base + k;
+        if (c < a.mb && (c == 0 || (key[k] >> a.sec_bits) != (key[k + 1] >> a.sec_bits)))
+            lhead = (u32)c;
+    }
+    const u32 incl = wave_incl_max(lhead);
+    if (lane == 63u)
+        s_wagg[w] = incl;
+    __syncthreads();
+    u32 excl = __shfl_up(incl, 1);
+    if (lane == 0)
+        excl = 0;
+    for (u32 ww = 0; ww < w; ++ww)
+        excl = excl > s_wagg[ww] ? excl : s_wagg[ww];
+    if (t == 0) {
+        u32 agg = 0;
+        for (int ww = 0; ww < WAVES; ++ww)
+            agg = agg > s_wagg[ww] ? agg : s_wagg[ww];
+        s_prefix = lb_exclusive_prefix<true>(a.lookback, 1, tile, a.epoch, agg, a.err);
+    }
+    __syncthreads();
+    u32 head = excl > s_prefix ? excl : s_prefix;
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const u64 c = base + k;
+        if (c < a.mb) {
+            const u32 g = (u32)(key[k + 1] >> a.sec_bits);
+            if (c == 0 || (key[k] >> a.sec_bits) != g)
+                head = (u32)c;
+            const u32 dest = g < a.groups ? a.gstart[g] + ((u32)c - head) : a.m;
+            if (dest >= a.m || head > (u32)c) {
+                atomicExch(a.err, DEV_ERR_PLACE_RANGE);
+                continue;
+            }
+            a.keys_out[dest] = key[k + 1];
+            a.sufs_out[dest] = a.big_sufs[c];
+        }
+    }
 }
 
 // Four suffix-array entries per thread: 16 bytes in, 20 bytes out (include/lane.hpp:69-79, include/sa40.hpp:72-75).

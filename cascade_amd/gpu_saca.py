@@ -22,6 +22,7 @@ def stats_to_dict(st):
         "generations": g,
         "active": [int(st.active[i]) for i in range(g)],
         "groups": [int(st.groups[i]) for i in range(g)],
+        "big": [int(st.big[i]) for i in range(g)],
         "passes": [int(st.passes[i]) for i in range(g)],
         "ms": [float(st.ms[i]) for i in range(g)],
         "ms_output": float(st.ms_output),

@@ -44,7 +44,8 @@ typedef struct csa_stats {
     int32_t generations;                  /* generations run, generation 0 included */
     uint64_t active[CSA_MAX_GENERATIONS]; /* suffixes active entering generation g; active[0] = n */
     uint64_t groups[CSA_MAX_GENERATIONS]; /* unresolved groups entering generation g (0 for g = 0) */
-    int32_t passes[CSA_MAX_GENERATIONS];  /* radix passes run in generation g */
+    uint64_t big[CSA_MAX_GENERATIONS];    /* of active[g], members of groups too large for the in-tile sort */
+    int32_t passes[CSA_MAX_GENERATIONS];  /* radix passes run in generation g (over the large groups for g > 0) */
     float ms[CSA_MAX_GENERATIONS];        /* device time of generation g */
     float ms_output;                      /* sa40 emission */
     float ms_total;                       /* first kernel to last kernel, on the stream */

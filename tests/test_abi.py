@@ -27,13 +27,13 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_stats_struct_layout_matches_header():
-    # 8 + 4 + 4 + 64*8 + 64*8 + 64*4 + 64*4 + 4 + 4 + 8 + 8 + 8
-    assert C.sizeof(_native.CsaStats) == 8 + 4 + 4 + 512 + 512 + 256 + 256 + 4 + 4 + 8 + 8 + 8
+    # 8 + 4 + 4 + 3 * 64*8 + 64*4 + 64*4 + 4 + 4 + 8 + 8 + 8
+    assert C.sizeof(_native.CsaStats) == 8 + 4 + 4 + 512 + 512 + 512 + 256 + 256 + 4 + 4 + 8 + 8 + 8
 
 
 def test_argument_errors_need_no_gpu():
     lib = _native.load()
-    assert lib.csa_bytes_per_suffix(1) == 40
+    assert lib.csa_bytes_per_suffix(1) == 60
     h = C.c_void_p()
     assert lib.csa_create(10, 3, C.byref(h)) == _native.CSA_ERR_ARG
     assert b"key_words" in lib.csa_last_error()

@@ -1,0 +1,79 @@
+"""The kernel sources of cascade_amd/csrc, compiled for the CPU against tests/cpu_emu (a stand-in for the HIP
+runtime and the wave64 intrinsics), must reproduce the oracle's suffix arrays. This checks the kernels' logic
+and indexing where no GPU exists; the library built here is test infrastructure and is never loaded by the
+product. Small inputs only: every wave operation is a thread barrier on the CPU."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import oracle_lib
+import texts
+from cascade_amd import _native
+
+EMU_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpu_emu")
+EMU_LIB = os.path.join(EMU_DIR, "libcascade_emu.so")
+
+
+@pytest.fixture(scope="module")
+def emu():
+    subprocess.run(["make", "-C", EMU_DIR, "libcascade_emu.so"], check=True, capture_output=True)
+    lib = C.CDLL(EMU_LIB)
+    vp, u64, u32, i32 = C.c_void_p, C.c_uint64, C.c_uint32, C.c_int
+    lib.csa_create.argtypes = [u64, i32, C.POINTER(vp)]
+    lib.csa_destroy.argtypes = [vp]
+    lib.csa_sort_partition_u16_dev.argtypes = [vp, vp, u64, u64, vp, vp, u32, C.POINTER(_native.CsaStats)]
+    lib.csa_radix_sort_pairs_dev.argtypes = [vp, vp, vp, u64, i32, i32, vp]
+    lib.csa_last_error.restype = C.c_char_p
+    return lib
+
+
+def emu_sort(lib, T, key_words):
+    T = np.ascontiguousarray(T, dtype=np.uint16)
+    n = T.size
+    h = C.c_void_p()
+    assert lib.csa_create(max(n, 1), key_words, C.byref(h)) == 0
+    out = np.zeros(5 * n + 8, dtype=np.uint8)
+    st = _native.CsaStats()
+    rc = lib.csa_sort_partition_u16_dev(h, T.ctypes.data, n, 0, out.ctypes.data, None, 0, C.byref(st))
+    lib.csa_destroy(h)
+    assert rc == 0, lib.csa_last_error()
+    return out[:5 * n], [int(st.active[i]) for i in range(st.generations)], [int(st.big[i]) for i in range(st.generations)]
+
+
+CASES = ["rand_n17_s2", "rand_n1000_s2", "rand_n1000_s65536", "hand_1", "hand_15", "hand_18", "hand_23"]
+
+
+@pytest.mark.parametrize("key_words", [1, 2])
+def test_fixtures_through_the_emulated_kernels(emu, key_words):
+    suite = dict(texts.fixture_suite())
+    for name in CASES:
+        T = suite[name]
+        got, active, _ = emu_sort(emu, T, key_words)
+        assert np.array_equal(got, oracle_lib.build_sa40(T)), name
+        _, counts = oracle_lib.prefix_doubling(T, key_words)
+        assert active == counts, name
+
+
+def test_small_and_large_groups_take_both_paths(emu):
+    # 2 symbols, no separators: generation 1 has a few huge groups (radix path), later ones small groups (in-tile path)
+    T = texts.random_text(6000, 2, 5, sep_every=0)
+    got, active, big = emu_sort(emu, T, 1)
+    assert np.array_equal(got, oracle_lib.build_sa40(T))
+    assert big[1] > 0 and any(b == 0 and a > 0 for a, b in zip(active[2:], big[2:]))
+
+
+def test_emulated_radix_sort_matches_stable_sort(emu):
+    rng = np.random.default_rng(1)
+    n = 5000
+    keys = rng.integers(0, 1 << 40, n).astype(np.uint64)
+    vals = np.arange(n, dtype=np.uint32)
+    wk, wv = oracle_lib.stable_sort_pairs(keys, vals, 3, 37)
+    h = C.c_void_p()
+    assert emu.csa_create(n, 1, C.byref(h)) == 0
+    k, v = keys.copy(), vals.copy()
+    assert emu.csa_radix_sort_pairs_dev(h, k.ctypes.data, v.ctypes.data, n, 3, 37, None) == 0
+    emu.csa_destroy(h)
+    assert np.array_equal(k, wk) and np.array_equal(v, wv)

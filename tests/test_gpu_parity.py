@@ -193,3 +193,19 @@ def test_repeatable(torch_mod, sorter):
     a = gpu_sa40(torch_mod, sorter, T)
     b = gpu_sa40(torch_mod, sorter, T)
     assert np.array_equal(a, b)
+
+
+def test_many_small_partitions_of_low_entropy(torch_mod):
+    """Low-entropy texts around the tile sizes of the kernels (2048 and 8192): large groups, groups that straddle
+    tiles, several generations. Fresh handles sized exactly to the partition, so any index out of range shows."""
+    from cascade_amd import PartitionSorter
+    rng = np.random.default_rng(2024)
+    for n in (2047, 2048, 2049, 4100, 8000, 8191, 8192, 8193, 12000, 20000, 50000):
+        for sigma in (2, 3, 5):
+            T = texts.random_text(n, sigma, int(rng.integers(1 << 30)), sep_every=int(rng.choice([0, 50, 500])))
+            with PartitionSorter(n, key_words=1) as s:
+                got = gpu_sa40(torch_mod, s, T)
+                stats = s.last_stats
+            sa, counts = oracle_lib.prefix_doubling(T, 1)
+            assert stats["active"] == counts, (n, sigma)
+            assert np.array_equal(got, oracle_lib.u64_to_sa40(sa)), (n, sigma)
