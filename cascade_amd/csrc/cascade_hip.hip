@@ -8,6 +8,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -43,8 +44,14 @@ int fail(int code, const char* fmt, ...)
 constexpr int SORT_BLOCK = CSA_SORT_BLOCK;
 constexpr int SORT_ITEMS = CSA_SORT_ITEMS;
 constexpr int SORT_TILE = SORT_BLOCK * SORT_ITEMS;
-constexpr int RANK_BLOCK = 256;
-constexpr int RANK_ITEMS = 8;
+#ifndef CSA_RANK_BLOCK
+#define CSA_RANK_BLOCK 256
+#endif
+#ifndef CSA_RANK_ITEMS
+#define CSA_RANK_ITEMS 8
+#endif
+constexpr int RANK_BLOCK = CSA_RANK_BLOCK;
+constexpr int RANK_ITEMS = CSA_RANK_ITEMS;
 constexpr int RANK_TILE = RANK_BLOCK * RANK_ITEMS;
 // groups of up to SMALL_MAXG suffixes are sorted inside one tile of the small-group kernel
 #ifndef CSA_SMALL_MAXG
@@ -56,6 +63,13 @@ constexpr int SMALL_TILE = SMALL_BLOCK * SMALL_ITEMS;
 constexpr int SMALL_MAXG = CSA_SMALL_MAXG;
 constexpr u32 TICKET_POOL = 4096;
 constexpr int EVENT_POOL = 2 * CSA_MAX_GENERATIONS * MAX_PASSES * 2;
+
+// Lists of at least this many suffixes update rank[] through two radix passes on the text position instead of
+// scattering 4-byte writes over the whole array.
+#ifndef CSA_DEFER_MIN
+#define CSA_DEFER_MIN (1u << 23)
+#endif
+constexpr u32 DEFER_MIN = CSA_DEFER_MIN;
 
 int bit_length(u64 v)
 {
@@ -81,6 +95,7 @@ struct csa_handle {
     u32* gstart[2] = {nullptr, nullptr};
     u64* lookback = nullptr;
     u64 lookback_words = 0;
+    u64 lookback_tile_words = 0;
     u32* ghist = nullptr;      // [MAX_PASSES][256]
     u32* digit_base = nullptr; // [MAX_PASSES][256]
     u32* tickets = nullptr;    // [TICKET_POOL]
@@ -88,6 +103,7 @@ struct csa_handle {
     u32* counts = nullptr; // [2] survivors, groups; [2] error flag; [3] verifier flag
     u32* h_pinned = nullptr; // host mirror: [0..3] counts/err, [16 ..) histogram
     u32 epoch = 0;
+    u32 defer_min = DEFER_MIN; // lists at least this long use the bucketed rank update (env CASCADE_DEFER_MIN overrides)
     std::vector<hipEvent_t> events;
     hipEvent_t ev_gen[CSA_MAX_GENERATIONS + 2] = {};
     bool ev_gen_ready = false;
@@ -138,9 +154,15 @@ void launch_onesweep(const OnesweepArgs& a, hipStream_t s)
 {
     const u32 tiles = (u32)(((u64)a.n + SORT_TILE - 1) / SORT_TILE);
     if (a.shift >= 32)
-        hipLaunchKernelGGL((onesweep_kernel<SORT_BLOCK, SORT_ITEMS, SRC, 1>), dim3(tiles), dim3(SORT_BLOCK), 0, s, a);
+        hipLaunchKernelGGL((onesweep_kernel<u64, SORT_BLOCK, SORT_ITEMS, SRC, 1>), dim3(tiles), dim3(SORT_BLOCK), 0, s, a);
     else
-        hipLaunchKernelGGL((onesweep_kernel<SORT_BLOCK, SORT_ITEMS, SRC, 0>), dim3(tiles), dim3(SORT_BLOCK), 0, s, a);
+        hipLaunchKernelGGL((onesweep_kernel<u64, SORT_BLOCK, SORT_ITEMS, SRC, 0>), dim3(tiles), dim3(SORT_BLOCK), 0, s, a);
+}
+
+void launch_onesweep32(const OnesweepArgs& a, hipStream_t s)
+{
+    const u32 tiles = (u32)(((u64)a.n + SORT_TILE - 1) / SORT_TILE);
+    hipLaunchKernelGGL((onesweep_kernel<u32, SORT_BLOCK, SORT_ITEMS, SRC_PAIRS, 0>), dim3(tiles), dim3(SORT_BLOCK), 0, s, a);
 }
 
 // Sorts n pairs by the digits of `plan`. The first pass that runs takes its input as `src` says
@@ -215,6 +237,7 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
         a.bits = plan.bits[p];
         a.digit_base = h->digit_base + p * RADIX_BINS;
         a.lookback = h->lookback;
+        a.lookback_groups = h->lookback + h->lookback_tile_words;
         a.epoch = next_epoch(h);
         a.err = h->counts + 2;
         int rc = next_ticket(L, &a.ticket);
@@ -223,6 +246,14 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
         const bool timed = (L.flags & CSA_FLAG_KERNEL_TIMING) && L.events_used + 2 <= (int)h->events.size();
         if (timed)
             HIP_TRY(hipEventRecord(h->events[L.events_used], s));
+#ifdef CSA_TIMING_DEBUG
+        static unsigned long long* odbg = nullptr; // experiments only: stamps of one chosen full-size pass
+        static int pass_no = 0;
+        if (!odbg)
+            (void)hipMalloc((void**)&odbg, (size_t)8 * 8 * ((h->cap + SORT_TILE - 1) / SORT_TILE + 1));
+        ++pass_no;
+        a.dbg = (pass_no == 3 && getenv("CSA_OTIMING_DUMP")) ? odbg : nullptr;
+#endif
         const int use_src = first ? src : SRC_PAIRS;
         if (use_src == SRC_PAIRS)
             launch_onesweep<SRC_PAIRS>(a, s);
@@ -235,6 +266,18 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
             L.timed.push_back({L.events_used, (u64)n});
             L.events_used += 2;
         }
+#ifdef CSA_TIMING_DEBUG
+        if (a.dbg) {
+            (void)hipStreamSynchronize(s);
+            const u32 tiles = (u32)(((u64)n + SORT_TILE - 1) / SORT_TILE);
+            std::vector<unsigned long long> hbuf((size_t)tiles * 8);
+            (void)hipMemcpy(hbuf.data(), odbg, hbuf.size() * 8, hipMemcpyDeviceToHost);
+            if (FILE* f = fopen(getenv("CSA_OTIMING_DUMP"), "wb")) {
+                fwrite(hbuf.data(), 8, hbuf.size(), f);
+                fclose(f);
+            }
+        }
+#endif
         first = false;
         where ^= 1;
         (*passes_run)++;
@@ -300,6 +343,99 @@ int read_counts(Launch& L, u32* survivors, u32* groups, u32* big)
     return CSA_OK;
 }
 
+
+struct DeferBuffers {
+    u32* vals;    // [m] new ranks in sorted-list order (written by the rerank kernel)
+    u32* t1_pos;  // ping
+    u32* t1_val;
+    u32* t2_pos;  // pong
+    u32* t2_val;
+};
+
+// After a rerank launched with rank_vals = buf.vals: rank[pos[c]] = vals[c] for all c < m.
+// pos[0, n) is a permutation of the text positions [0, n) (the sorted suffixes of generation 0), which makes the
+// digit counts of the passes a closed form. The pairs are sorted on the position bits above the window size
+// (windows of at most 1 << 14 positions, 1 << 15 for the largest partitions), then placed window by window.
+int deferred_rank_update(Launch& L, const u32* pos, const DeferBuffers& buf, u32 n)
+{
+    csa_handle* h = L.h;
+    hipStream_t s = L.stream;
+    const int nb = bit_length(n - 1); // <= 31
+    int top = nb - 14;                // position bits to sort on
+    if (top < 0)
+        top = 0;
+    if (top > 16)
+        top = 16;
+    const int window_log2 = nb - top;
+    int n_pass = 0, xshift[2] = {0, 0}, xbits[2] = {0, 0};
+    if (top > 8) {
+        xshift[0] = window_log2;
+        xbits[0] = top - 8;
+        xshift[1] = window_log2 + top - 8;
+        xbits[1] = 8;
+        n_pass = 2;
+    } else if (top > 0) {
+        xshift[0] = window_log2;
+        xbits[0] = top;
+        n_pass = 1;
+    }
+    const u32* in_pos = pos;
+    const u32* in_val = buf.vals;
+    if (n_pass > 0) {
+        u32* h_hist = h->h_pinned + 16;
+        for (int p = 0; p < n_pass; ++p) {
+            // positions x in [0, n) whose digit (x >> shift) & mask equals d: whole periods plus a clamped remainder
+            const u64 unit = 1ull << xshift[p], period = unit << xbits[p];
+            const u64 whole = (u64)n / period, rest = (u64)n % period;
+            for (u32 d = 0; d < (u32)RADIX_BINS; ++d) {
+                u64 c = 0;
+                if (d < (1u << xbits[p])) {
+                    c = whole * unit;
+                    if (rest > d * unit)
+                        c += rest - d * unit < unit ? rest - d * unit : unit;
+                }
+                h_hist[p * RADIX_BINS + d] = (u32)c;
+            }
+        }
+        HIP_TRY(hipMemcpyAsync(h->ghist, h_hist, n_pass * RADIX_BINS * sizeof(u32), hipMemcpyHostToDevice, s));
+        hipLaunchKernelGGL(radix_scan_hist_kernel, dim3(1), dim3(256), 0, s, h->ghist, h->digit_base, n_pass);
+        u32* out_pos[2] = {buf.t1_pos, buf.t2_pos};
+        u32* out_val[2] = {buf.t1_val, buf.t2_val};
+        for (int p = 0; p < n_pass; ++p) {
+            OnesweepArgs a;
+            a.keys_in = in_pos;
+            a.vals_in = in_val;
+            a.keys_out = out_pos[p];
+            a.vals_out = out_val[p];
+            a.text = nullptr;
+            a.n = n;
+            a.text_n = n;
+            a.tail = 0;
+            a.word = 0;
+            a.shift = xshift[p];
+            a.bits = xbits[p];
+            a.digit_base = h->digit_base + p * RADIX_BINS;
+            a.lookback = h->lookback;
+            a.lookback_groups = h->lookback + h->lookback_tile_words;
+            a.epoch = next_epoch(h);
+            a.err = h->counts + 2;
+            int rc = next_ticket(L, &a.ticket);
+            if (rc)
+                return rc;
+            launch_onesweep32(a, s);
+            in_pos = out_pos[p];
+            in_val = out_val[p];
+        }
+    }
+    const u32 windows = (u32)((((u64)n - 1) >> window_log2) + 1);
+    if (window_log2 <= 14)
+        hipLaunchKernelGGL((place_ranks_kernel<14>), dim3(windows), dim3(1024), 0, s, in_pos, in_val, n, window_log2, h->rank);
+    else
+        hipLaunchKernelGGL((place_ranks_kernel<15>), dim3(windows), dim3(1024), 0, s, in_pos, in_val, n, window_log2, h->rank);
+    HIP_TRY(hipGetLastError());
+    return CSA_OK;
+}
+
 int launch_rerank(Launch& L, RerankArgs& a)
 {
     csa_handle* h = L.h;
@@ -311,8 +447,49 @@ int launch_rerank(Launch& L, RerankArgs& a)
     if (rc)
         return rc;
     const u32 tiles = (u32)(((u64)a.m + RANK_TILE - 1) / RANK_TILE);
+#ifdef CSA_TIMING_DEBUG
+    static unsigned long long* dbg = nullptr; // experiments only: stamps of the first (largest) launch are dumped
+    static bool dumped = false;
+    if (!dbg)
+        (void)hipMalloc((void**)&dbg, (size_t)8 * 8 * ((h->cap + RANK_TILE - 1) / RANK_TILE + 1));
+    a.dbg = dumped ? nullptr : dbg;
+#endif
     hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS>), dim3(tiles), dim3(RANK_BLOCK), 0, L.stream, a);
     HIP_TRY(hipGetLastError());
+#ifdef CSA_TIMING_DEBUG
+    if (!dumped && getenv("CSA_TIMING_DUMP")) {
+        (void)hipStreamSynchronize(L.stream);
+        std::vector<unsigned long long> hbuf((size_t)tiles * 8);
+        (void)hipMemcpy(hbuf.data(), dbg, hbuf.size() * 8, hipMemcpyDeviceToHost);
+        if (FILE* f = fopen(getenv("CSA_TIMING_DUMP"), "wb")) {
+            fwrite(hbuf.data(), 8, hbuf.size(), f);
+            fclose(f);
+        }
+        dumped = true;
+    }
+#endif
+    return CSA_OK;
+}
+
+// Ranks the sorted list described by `ra`, reads back the survivor counts and brings rank[] up to date
+// (directly from the kernel for short lists, through the bucketed update for long ones).
+int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivors, u32* groups)
+{
+    csa_handle* h = L.h;
+    (void)h;
+    // generation 0 ranks every suffix of the partition: on large partitions the n scattered writes go through
+    // the bucketed update instead
+    const bool defer = ra.gen0 && ra.m >= h->defer_min;
+    if (defer)
+        ra.rank_vals = buf.vals;
+    int rc = launch_rerank(L, ra);
+    if (rc)
+        return rc;
+    rc = read_counts(L, survivors, groups, nullptr);
+    if (rc)
+        return rc;
+    if (defer)
+        return deferred_rank_update(L, ra.sufs, buf, ra.n);
     return CSA_OK;
 }
 
@@ -382,11 +559,11 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     ra.gids_out = agid;
     ra.gprim_out = h->gprim[0];
     ra.gstart_out = h->gstart[0];
-    rc = launch_rerank(L, ra);
-    if (rc)
-        return rc;
+    // scratch of the bucketed rank update: all free while (and after) a list is being ranked
+    const DeferBuffers defer_buf = {bx[0], bx[1], reinterpret_cast<u32*>(bkey[0]), reinterpret_cast<u32*>(bkey[1]),
+                                    reinterpret_cast<u32*>(bkey[1]) + h->cap};
     u32 m = 0, groups = 0, big = 0;
-    rc = read_counts(L, &m, &groups, &big);
+    rc = rerank_step(L, ra, defer_buf, &m, &groups);
     if (rc)
         return rc;
     st->passes[0] = passes;
@@ -474,13 +651,10 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
         ra.gids_out = agid;
         ra.gprim_out = h->gprim[gp ^ 1];
         ra.gstart_out = h->gstart[gp ^ 1];
-        rc = launch_rerank(L, ra);
+        rc = rerank_step(L, ra, defer_buf, &m, &groups);
         if (rc)
             return rc;
         gp ^= 1;
-        rc = read_counts(L, &m, &groups, nullptr);
-        if (rc)
-            return rc;
         st->passes[gen] = passes;
         HIP_TRY(hipEventRecord(h->ev_gen[gen + 1], s));
         gen++;
@@ -537,10 +711,13 @@ int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
     csa_handle* h = new csa_handle();
     h->cap = max_part_sz ? max_part_sz : 1;
     h->key_words = key_words;
+    if (const char* e = getenv("CASCADE_DEFER_MIN"))
+        h->defer_min = (u32)strtoul(e, nullptr, 10);
     const u64 cap = h->cap;
     const u64 sort_tiles = (cap + SORT_TILE - 1) / SORT_TILE;
     const u64 rank_tiles = (cap + RANK_TILE - 1) / RANK_TILE;
-    h->lookback_words = sort_tiles * RADIX_BINS;
+    h->lookback_tile_words = sort_tiles * RADIX_BINS; // the group words of the radix pass follow the tile words
+    h->lookback_words = h->lookback_tile_words + (sort_tiles / LB_GROUP + 1) * RADIX_BINS;
     if (rank_tiles * 4 > h->lookback_words)
         h->lookback_words = rank_tiles * 4;
     hipError_t e = hipGetDevice(&h->device);

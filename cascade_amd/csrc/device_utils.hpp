@@ -86,44 +86,235 @@ __device__ __forceinline__ void lb_publish(u64* chain, u32 stride, u32 tile, u32
 }
 
 // Step 2: returns the combination of the aggregates of tiles [0, tile) and upgrades the tile's own word
-// to "inclusive". Combination is max if IS_MAX, else a 32-bit sum. On a spin timeout (a predecessor never
-// published) sets *err and returns what it has, so that every wave still leaves the kernel.
-template <bool IS_MAX>
+// to "inclusive". Combination is max if IS_MAX, else a 32-bit sum.
+// The walk towards tile 0 reads W predecessor words per round, all loads in flight together, and then consumes
+// them in order up to the first inclusive one. A serial walk (one dependent load per predecessor) would cap
+// the whole launch at one tile per memory round trip, because the nearest inclusive word is about as far back
+// as there are unresolved tiles in flight.
+// On a timeout (a predecessor never published) sets *err and returns what it has, so that every wave still
+// leaves the kernel.
+template <bool IS_MAX, int W = 8>
 __device__ __forceinline__ u32 lb_wait_exclusive(u64* chain, u32 stride, u32 tile, u32 epoch, u32 aggregate, u32* err)
 {
     if (tile == 0)
         return 0;
+#ifdef CSA_EXPERIMENT_NO_LOOKBACK_WAIT
+    return 0; // timing experiment only: results are wrong
+#endif
     u32 excl = 0;
-    u32 t = tile;
-    while (t > 0) {
-        --t;
-        u64 w = 0;
-        u32 spins = 0;
-        for (;;) {
-            w = lb_load(chain + (u64)t * stride);
-            if ((u32)(w >> 34) == epoch && ((w >> 32) & 3u) != 0)
-                break;
-            if (++spins >= LB_SPIN_LIMIT) {
-                atomicExch(err, 1u);
+    long long next = (long long)tile - 1; // nearest predecessor not yet consumed
+    u32 idle = 0;
+    bool done = false;
+    while (!done) {
+        u64 word[W];
+#pragma unroll
+        for (int j = 0; j < W; ++j) {
+            const long long idx = next - j;
+            word[j] = idx >= 0 ? lb_load(chain + (u64)idx * stride) : 0ull;
+        }
+        u32 consumed = 0;
+#pragma unroll
+        for (int j = 0; j < W; ++j) {
+            if (done || consumed != (u32)j)
+                continue; // stopped at an earlier word of this round
+            if (next - j < 0) { // cannot happen: tile 0 publishes an inclusive word
+                done = true;
+                continue;
+            }
+            const u64 wd = word[j];
+            const u32 status = (u32)(wd >> 32) & 3u;
+            if ((u32)(wd >> 34) != epoch || status == 0)
+                continue; // not published yet: poll again from here
+            const u32 v = (u32)wd;
+            excl = IS_MAX ? (excl > v ? excl : v) : excl + v;
+            consumed++;
+            if (status == LB_INCL)
+                done = true;
+        }
+        next -= consumed;
+        if (!done && consumed == 0) {
+            if (++idle >= LB_SPIN_LIMIT) {
+                atomicExch(err, DEV_ERR_LOOKBACK_TIMEOUT);
                 return excl;
             }
             __builtin_amdgcn_s_sleep(1);
+        } else {
+            idle = 0;
         }
-        const u32 v = (u32)w;
-        excl = IS_MAX ? (excl > v ? excl : v) : excl + v;
-        if (((w >> 32) & 3u) == LB_INCL)
-            break;
     }
     const u32 incl = IS_MAX ? (excl > aggregate ? excl : aggregate) : excl + aggregate;
     lb_store(chain + (u64)tile * stride, lb_pack(epoch, LB_INCL, incl));
     return excl;
 }
 
-template <bool IS_MAX>
+template <bool IS_MAX, int W = 16>
 __device__ __forceinline__ u32 lb_exclusive_prefix(u64* chain, u32 stride, u32 tile, u32 epoch, u32 aggregate, u32* err)
 {
     lb_publish(chain, stride, tile, epoch, aggregate);
-    return lb_wait_exclusive<IS_MAX>(chain, stride, tile, epoch, aggregate, err);
+    return lb_wait_exclusive<IS_MAX, W>(chain, stride, tile, epoch, aggregate, err);
+}
+
+// ---- two-level look-back (one chain per thread, many chains per tile: the radix pass) ----
+//
+// With one level, every waiting tile walks back over all the unresolved tiles in flight, re-reading their words
+// over the fabric; the walks grow with the number of resident tiles and end up costing more traffic and time
+// than the data. Here tiles form groups of LB_GROUP consecutive tiles. A tile sums the aggregates of the
+// (at most LB_GROUP - 1) earlier tiles of its own group: those are published early by tiles that started
+// together with it, so nothing there waits for a resolution. The last tile of a group publishes the group's
+// total and chains the groups with the ordinary protocol; every tile adds the inclusive prefix of the group
+// before its own. Group words arrive LB_GROUP times more slowly than tile words, so that chain stays short.
+
+constexpr u32 LB_GROUP = 16;
+
+// spins until the word is published for this launch; returns it (0 after a timeout, with *err set)
+__device__ __forceinline__ u64 lb_wait_word(const u64* p, u32 epoch, u32* err)
+{
+    u32 idle = 0;
+    for (;;) {
+        const u64 w = lb_load(p);
+        if ((u32)(w >> 34) == epoch && ((w >> 32) & 3u) != 0)
+            return w;
+        if (++idle >= LB_SPIN_LIMIT) {
+            atomicExch(err, DEV_ERR_LOOKBACK_TIMEOUT);
+            return 0;
+        }
+        __builtin_amdgcn_s_sleep(2);
+    }
+}
+
+// tile_chain: word of tile t at tile_chain[t * stride], published with lb_publish_aggregate_only beforehand.
+// group_chain: word of group g at group_chain[g * stride]. Returns the sum of the aggregates of tiles [0, tile).
+__device__ __forceinline__ void lb2_publish(u64* tile_chain, u32 stride, u32 tile, u32 epoch, u32 aggregate)
+{
+    lb_store(tile_chain + (u64)tile * stride, lb_pack(epoch, LB_AGG, aggregate));
+}
+
+__device__ __forceinline__ u32 lb2_wait_exclusive(u64* tile_chain, u64* group_chain, u32 stride, u32 tile, u32 epoch,
+                                                  u32 aggregate, u32* err)
+{
+    const u32 j = tile % LB_GROUP, g = tile / LB_GROUP;
+    // aggregates of the earlier tiles of this group: all loads in flight together, stragglers polled one by one
+    u64 word[LB_GROUP - 1];
+#pragma unroll
+    for (u32 k = 1; k < LB_GROUP; ++k)
+        word[k - 1] = k <= j ? lb_load(tile_chain + (u64)(tile - k) * stride) : 0ull;
+    u32 within = 0;
+#pragma unroll
+    for (u32 k = 1; k < LB_GROUP; ++k) {
+        if (k <= j) {
+            u64 w = word[k - 1];
+            if ((u32)(w >> 34) != epoch || ((w >> 32) & 3u) == 0)
+                w = lb_wait_word(tile_chain + (u64)(tile - k) * stride, epoch, err);
+            within += (u32)w;
+        }
+    }
+    const bool closes_group = j == LB_GROUP - 1;
+    const u32 total = within + aggregate;
+    if (closes_group)
+        lb_store(group_chain + (u64)g * stride, lb_pack(epoch, g == 0 ? LB_INCL : LB_AGG, total));
+    // inclusive prefix of the groups before this one
+    u32 gexcl = 0;
+    for (u32 gi = g; gi > 0;) {
+        --gi;
+        const u64 w = lb_wait_word(group_chain + (u64)gi * stride, epoch, err);
+        gexcl += (u32)w;
+        if (((w >> 32) & 3u) == LB_INCL || w == 0)
+            break;
+    }
+    if (closes_group && g > 0)
+        lb_store(group_chain + (u64)g * stride, lb_pack(epoch, LB_INCL, gexcl + total));
+    return gexcl + within;
+}
+
+// ---- wave-wide look-back ----
+// The same protocol walked by a whole wave: each round every lane loads the word of one predecessor (LOADS words
+// per lane, 64 * LOADS predecessors per round), ballots find the run of published words nearest to the tile and
+// the first inclusive word inside it, and a wave reduction combines that run. The number of tiles a launch can
+// resolve per unit time is (predecessors inspected per round) / (memory round trip); with one word per round
+// trip the kernels stall with every resident tile waiting in its look-back.
+// Must be called by all 64 lanes of a wave, converged; returns the same value in every lane.
+
+__device__ __forceinline__ u32 wave_reduce_sum(u32 v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        v += __shfl_xor(v, o);
+    return v;
+}
+
+__device__ __forceinline__ u32 wave_reduce_max(u32 v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const u32 t = __shfl_xor(v, o);
+        v = v > t ? v : t;
+    }
+    return v;
+}
+
+#ifndef CSA_LB_LOADS
+#define CSA_LB_LOADS 2
+#endif
+
+template <bool IS_MAX, int LOADS = CSA_LB_LOADS>
+__device__ __forceinline__ u32 lb_wave_exclusive(u64* chain, u32 stride, u32 tile, u32 epoch, u32 aggregate, u32* err)
+{
+    const u32 lane = lane_id();
+    if (lane == 0)
+        lb_publish(chain, stride, tile, epoch, aggregate);
+    if (tile == 0)
+        return 0;
+    u32 excl = 0;
+    long long next = (long long)tile - 1; // nearest predecessor not yet consumed
+    u32 idle = 0;
+    bool done = false;
+    while (!done) {
+        u64 word[LOADS];
+#pragma unroll
+        for (int j = 0; j < LOADS; ++j) {
+            const long long idx = next - (long long)(j * WAVE + lane);
+            word[j] = idx >= 0 ? lb_load(chain + (u64)idx * stride) : 0ull;
+        }
+        u32 consumed = 0;
+#pragma unroll
+        for (int j = 0; j < LOADS; ++j) {
+            // words of this batch, nearest predecessor in lane 0; a batch is looked at only if every earlier one
+            // of the round was consumed whole
+            const bool look = !done && consumed == (u32)(j * WAVE);
+            const long long idx = next - (long long)(j * WAVE + lane);
+            const u32 status = (idx >= 0 && (u32)(word[j] >> 34) == epoch) ? ((u32)(word[j] >> 32) & 3u) : 0u;
+            const u64 ready = __ballot(status != 0);
+            const u64 incl = __ballot(status == LB_INCL);
+            if (look) {
+                const u32 lead = ready == ~0ull ? 64u : (u32)__builtin_ctzll(~ready);
+                const u64 lead_mask = lead == 64u ? ~0ull : ((1ull << lead) - 1ull);
+                const u64 incl_in = incl & lead_mask;
+                const u32 take = incl_in ? (u32)__builtin_ctzll(incl_in) + 1u : lead;
+                const u32 mine = lane < take ? (u32)word[j] : 0u;
+                const u32 part = IS_MAX ? wave_reduce_max(mine) : wave_reduce_sum(mine);
+                excl = IS_MAX ? (excl > part ? excl : part) : excl + part;
+                consumed += take;
+                if (incl_in)
+                    done = true;
+            }
+        }
+        next -= consumed;
+        if (!done && consumed == 0) {
+            if (++idle >= LB_SPIN_LIMIT) {
+                if (lane == 0)
+                    atomicExch(err, DEV_ERR_LOOKBACK_TIMEOUT);
+                return excl;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        } else {
+            idle = 0;
+        }
+    }
+    if (lane == 0) {
+        const u32 inclusive = IS_MAX ? (excl > aggregate ? excl : aggregate) : excl + aggregate;
+        lb_store(chain + (u64)tile * stride, lb_pack(epoch, LB_INCL, inclusive));
+    }
+    return excl;
 }
 
 // ---- K-gram key: four uint16 symbols of the zero-padded text, the first one most significant ----

@@ -35,6 +35,11 @@ struct RerankArgs {
     const u32* gprim_in; // generation t: first rank of each incoming group
     u32 groups_in;       // generation t: number of incoming groups
     u32* rank;           // [n] by text position
+    // Deferred rank update (generation 0 of large partitions): instead of the scattered write rank[x] = r,
+    // the new rank of the suffix at sorted index c is stored at rank_vals[c] (a coalesced stream; the suffix
+    // itself is sufs[c]). The (x, r) pairs then go through two radix passes on the high bits of x before they
+    // are written to rank[], so that those writes fall into one small window of rank[] at a time.
+    u32* rank_vals; // null: write rank[x] directly
     u32* sa32;           // [n] suffix array under construction
     u32* sufs_out;       // next active list
     u32* gids_out;
@@ -45,37 +50,82 @@ struct RerankArgs {
     u32* ticket;
     u32 epoch;
     u32* err;
+#ifdef CSA_TIMING_DEBUG
+    unsigned long long* dbg; // [tiles][8] cycle stamps (experiments only)
+#endif
 };
+
+#ifdef CSA_TIMING_DEBUG
+#define CSA_STAMP(slot)                                                    \
+    if (a.dbg && threadIdx.x == 0)                                         \
+    a.dbg[(unsigned long long)tile * 8 + (slot)] = __builtin_readcyclecounter()
+#else
+#define CSA_STAMP(slot)
+#endif
 
 template <int BLOCK, int ITEMS>
 __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
 {
     constexpr int TILE = BLOCK * ITEMS;
     constexpr int WAVES = BLOCK / WAVE;
+    // The tile is read from and written to HBM in striped order (consecutive lanes, consecutive elements) and
+    // exchanged through LDS with the blocked order (each thread, ITEMS consecutive elements) the scans want.
+    // One pad slot per ITEMS elements keeps the blocked LDS accesses off a single bank.
+    constexpr int SLOTS = TILE + 2;               // element tile_base - 1, the tile, element tile_base + TILE
+    constexpr int PADDED = SLOTS + SLOTS / ITEMS + 1;
+    __shared__ u64 s_key[PADDED]; // later: compacted survivors (suffixes, group ids)
+    __shared__ u32 s_suf[PADDED]; // later: tables of the new groups (first rank, start)
+    __shared__ u32 s_rv[TILE];    // new ranks in list order (deferred rank update only)
     __shared__ u32 s_wagg[WAVES][4];
     __shared__ u32 s_tileprefix[4];
     __shared__ u32 s_tiletotal[4];
     __shared__ u32 s_tile;
+#define CSA_PAD(q) ((q) + (q) / ITEMS)
 
     const u32 t = threadIdx.x;
     const u32 lane = t & 63u;
     const u32 w = t >> 6;
+#ifdef CSA_NO_TICKET
+    if (t == 0)
+        s_tile = blockIdx.x;
+#else
     if (t == 0)
         s_tile = atomicAdd(a.ticket, 1u);
+#endif
     __syncthreads();
     const u32 tile = s_tile;
-    const u64 base = (u64)tile * TILE + (u64)t * ITEMS;
+    const u64 tile_base = (u64)tile * TILE;
+    const u64 base = tile_base + (u64)t * ITEMS;
     const u32 m = a.m;
+    CSA_STAMP(0);
 
-    // keys of c-1 .. c+ITEMS, and whether two neighbours are tied
+    // striped load into LDS: slot q holds element tile_base + q - 1
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        const u32 q = j * BLOCK + t + 1;
+        const u64 c = tile_base + q - 1;
+        const bool in = c < m;
+        s_key[CSA_PAD(q)] = in ? a.keys[c] : 0;
+        s_suf[CSA_PAD(q)] = in ? a.sufs[c] : 0;
+    }
+    if (t < 2) {
+        const u32 q = t == 0 ? 0u : (u32)TILE + 1u;
+        const bool in = t == 0 ? tile_base >= 1 : tile_base + TILE < m;
+        const u64 c = tile_base + q - 1;
+        s_key[CSA_PAD(q)] = in ? a.keys[c] : 0;
+        s_suf[CSA_PAD(q)] = in ? a.sufs[c] : 0;
+    }
+    __syncthreads();
+    CSA_STAMP(1);
+
+    // blocked read: elements base - 1 .. base + ITEMS
     u64 key[ITEMS + 2];
     u32 suf[ITEMS + 2];
 #pragma unroll
     for (int k = 0; k < ITEMS + 2; ++k) {
-        const u64 c = base + k; // index c-1 of the array, shifted by one
-        const bool in = c >= 1 && c - 1 < m;
-        key[k] = in ? a.keys[c - 1] : 0;
-        suf[k] = in ? a.sufs[c - 1] : 0;
+        const u32 q = t * ITEMS + k;
+        key[k] = s_key[CSA_PAD(q)];
+        suf[k] = s_suf[CSA_PAD(q)];
     }
     // eq[k]: elements (base+k-1) and (base+k) exist and belong to one run of equal keys
     // pq[k]: ... and to one primary group
@@ -125,7 +175,7 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
         s_wagg[w][2] = ic;
         s_wagg[w][3] = ih;
     }
-    __syncthreads();
+    __syncthreads(); // also: every thread holds its elements in registers, the staging arrays may be reused
     u32 xa = __shfl_up(ia, 1), xb = __shfl_up(ib, 1), xc = __shfl_up(ic, 1), xh = __shfl_up(ih, 1);
     if (lane == 0)
         xa = xb = xc = xh = 0;
@@ -135,29 +185,39 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
         xc += s_wagg[ww][2];
         xh += s_wagg[ww][3];
     }
-    // tile aggregate -> look-back, one lane per chain
-    if (w == 0 && lane < 4) {
+    // tile aggregate -> look-back, one wave per chain (max a, max b, sum survivors, sum new groups)
+    CSA_STAMP(2);
+    static_assert(WAVES >= 4, "one wave per look-back chain");
+    if (w < 4) {
         u32 agg = 0;
         for (int ww = 0; ww < WAVES; ++ww)
-            agg = lane < 2 ? (agg > s_wagg[ww][lane] ? agg : s_wagg[ww][lane]) : agg + s_wagg[ww][lane];
+            agg = w < 2 ? (agg > s_wagg[ww][w] ? agg : s_wagg[ww][w]) : agg + s_wagg[ww][w];
         u32 excl;
-        if (lane < 2)
-            excl = lb_exclusive_prefix<true>(a.lookback + lane, 4, tile, a.epoch, agg, a.err);
+        if (w < 2)
+            excl = lb_wave_exclusive<true>(a.lookback + w, 4, tile, a.epoch, agg, a.err);
         else
-            excl = lb_exclusive_prefix<false>(a.lookback + lane, 4, tile, a.epoch, agg, a.err);
-        s_tileprefix[lane] = excl;
-        s_tiletotal[lane] = excl + agg;
+            excl = lb_wave_exclusive<false>(a.lookback + w, 4, tile, a.epoch, agg, a.err);
+        if (lane == 0) {
+            s_tileprefix[w] = excl;
+            s_tiletotal[w] = excl + agg;
+        }
     }
+    CSA_STAMP(3);
     __syncthreads();
-    if (t == 0 && (u64)(tile + 1) * TILE >= m) { // the last tile knows the totals
+    if (t == 0 && tile_base + TILE >= m) { // the last tile knows the totals
         a.counts[0] = s_tiletotal[2];
         a.counts[1] = s_tiletotal[3];
         a.gstart_out[s_tiletotal[3]] = s_tiletotal[2]; // one-past-the-end entry: gstart[groups] = survivors
     }
+    const u32 tile_rc = s_tileprefix[2], tile_rh = s_tileprefix[3]; // survivors / new groups before this tile
     u32 ra = xa > s_tileprefix[0] ? xa : s_tileprefix[0];
     u32 rb = xb > s_tileprefix[1] ? xb : s_tileprefix[1];
-    u32 rc = xc + s_tileprefix[2];
-    u32 rh = xh + s_tileprefix[3];
+    u32 rc = xc; // tile-local from here on
+    u32 rh = xh;
+    u32* s_osuf = reinterpret_cast<u32*>(s_key); // [TILE] survivors of the tile, compacted
+    u32* s_ogid = s_osuf + TILE;                 // [TILE] their new group ids
+    u32* s_oprim = s_suf;                        // [TILE / 2] first rank of each new group of the tile
+    u32* s_ostart = s_suf + TILE / 2;            // [TILE / 2] and its start in the next active list
 
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
@@ -181,23 +241,66 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
                 atomicExch(a.err, DEV_ERR_RERANK_RANGE);
                 continue;
             }
-            if (a.gen0 || ra != rb)
+            if (a.rank_vals) {
+                s_rv[t * ITEMS + k] = nr;
+            } else if (a.gen0 || ra != rb) {
                 a.rank[x] = nr;
+            }
             if (single) {
                 if (!a.gen0)
                     a.sa32[nr] = x;
             } else {
                 if (ka) {
-                    a.gprim_out[rh] = nr;
-                    a.gstart_out[rh] = rc;
+                    s_oprim[rh] = nr;
+                    s_ostart[rh] = tile_rc + rc;
                     rh++;
                 }
-                a.sufs_out[rc] = x;
-                a.gids_out[rc] = rh - 1;
+                s_osuf[rc] = x;
+                s_ogid[rc] = tile_rh + rh - 1;
                 rc++;
             }
         }
     }
+    CSA_STAMP(4);
+    __syncthreads();
+    // striped write-out of what the tile produced
+    const u32 n_surv = s_tiletotal[2] - tile_rc, n_heads = s_tiletotal[3] - tile_rh;
+    for (u32 i = t; i < n_surv; i += BLOCK) {
+        a.sufs_out[tile_rc + i] = s_osuf[i];
+        a.gids_out[tile_rc + i] = s_ogid[i];
+    }
+    for (u32 i = t; i < n_heads; i += BLOCK) {
+        a.gprim_out[tile_rh + i] = s_oprim[i];
+        a.gstart_out[tile_rh + i] = s_ostart[i];
+    }
+    if (a.rank_vals)
+        for (u32 i = t; i < (u32)TILE && tile_base + i < m; i += BLOCK)
+            a.rank_vals[tile_base + i] = s_rv[i];
+    CSA_STAMP(5);
+#undef CSA_PAD
+}
+
+// Last step of the deferred rank update. The (text position, rank) pairs of generation 0 arrive sorted by the
+// high bits of the position; the positions are a permutation of [0, n), so the pairs of window w (positions
+// [w * S, (w + 1) * S), S = 1 << window_log2) are exactly pairs [w * S, (w + 1) * S) of the list. One workgroup
+// per window scatters the ranks into an LDS image of the window and writes the image out in full lines.
+template <int MAX_LOG2>
+__global__ __launch_bounds__(1024) void place_ranks_kernel(const u32* __restrict__ pos, const u32* __restrict__ val, u32 n,
+                                                           int window_log2, u32* __restrict__ rank)
+{
+    __shared__ u32 s_win[1 << MAX_LOG2];
+    const u32 S = 1u << window_log2;
+    const u64 first = (u64)blockIdx.x << window_log2;
+    const u32 count = (u32)((u64)n - first < S ? (u64)n - first : S);
+    for (u32 i = threadIdx.x; i < count; i += 1024) {
+        const u32 x = pos[first + i];
+        const u32 off = x - (u32)first;
+        if (off < count) // always, for a permutation sorted by window
+            s_win[off] = val[first + i];
+    }
+    __syncthreads();
+    for (u32 i = threadIdx.x; i < count; i += 1024)
+        rank[first + i] = s_win[i];
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -366,11 +469,13 @@ __global__ __launch_bounds__(BLOCK) void place_big_kernel(PlaceArgs a)
         excl = 0;
     for (u32 ww = 0; ww < w; ++ww)
         excl = excl > s_wagg[ww] ? excl : s_wagg[ww];
-    if (t == 0) {
+    if (w == 0) {
         u32 agg = 0;
         for (int ww = 0; ww < WAVES; ++ww)
             agg = agg > s_wagg[ww] ? agg : s_wagg[ww];
-        s_prefix = lb_exclusive_prefix<true>(a.lookback, 1, tile, a.epoch, agg, a.err);
+        const u32 prefix = lb_wave_exclusive<true>(a.lookback, 1, tile, a.epoch, agg, a.err);
+        if (lane == 0)
+            s_prefix = prefix;
     }
     __syncthreads();
     u32 head = excl > s_prefix ? excl : s_prefix;

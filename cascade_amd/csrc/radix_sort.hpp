@@ -165,9 +165,9 @@ __global__ __launch_bounds__(256) void radix_scan_hist_kernel(const u32* ghist, 
 }
 
 struct OnesweepArgs {
-    const u64* keys_in;
+    const void* keys_in; // u64 keys, or u32 keys for the narrow instantiation
     const u32* vals_in;
-    u64* keys_out;
+    void* keys_out;
     u32* vals_out;
     const u16* text;
     u32 n;      // pairs
@@ -178,26 +178,47 @@ struct OnesweepArgs {
     int bits;
     const u32* digit_base; // [256] for this pass
     u64* lookback;         // [tiles][256]
+    u64* lookback_groups;  // [ceil(tiles / LB_GROUP)][256]
     u32* ticket;           // zero before the launch
     u32 epoch;
     u32* err;
+#ifdef CSA_TIMING_DEBUG
+    unsigned long long* dbg; // [tiles][8] cycle stamps (experiments only)
+#endif
 };
+
+#ifdef CSA_TIMING_DEBUG
+#define CSA_OSTAMP(slot)                                                   \
+    if (a.dbg && threadIdx.x == 0)                                         \
+    a.dbg[(unsigned long long)tile * 8 + (slot)] = __builtin_readcyclecounter()
+#else
+#define CSA_OSTAMP(slot)
+#endif
+
+// predecessors a digit's look-back inspects per round
+#ifndef CSA_SORT_LB_W
+#define CSA_SORT_LB_W 8
+#endif
 
 // minimum waves per SIMD the compiler must leave room for (caps the VGPR budget of the radix pass)
 #ifndef CSA_SORT_MIN_WAVES
 #define CSA_SORT_MIN_WAVES 1
 #endif
 
-// HI selects the 32-bit half of the key that holds this pass's digit (digits never straddle the halves:
-// shifts are multiples of 8), so that the digit is one bit-field extract of a 32-bit register.
-template <int BLOCK, int ITEMS, int SRC, int HI>
+// KeyT is u64 (the suffix-sort keys) or u32 (the (text position, rank) pairs of the bucketed rank update).
+// HI selects the 32-bit half of a 64-bit key that holds this pass's digit (digits never straddle the halves),
+// so that the digit is one bit-field extract of a 32-bit register.
+template <typename KeyT, int BLOCK, int ITEMS, int SRC, int HI>
 __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(OnesweepArgs a)
 {
     constexpr int TILE = BLOCK * ITEMS;
     constexpr int WAVES = BLOCK / WAVE;
     static_assert(BLOCK >= RADIX_BINS, "one thread per digit is assumed");
+    static_assert(sizeof(KeyT) == 8 || (SRC == SRC_PAIRS && HI == 0), "narrow keys are plain pairs");
+    const KeyT* __restrict__ keys_in = static_cast<const KeyT*>(a.keys_in);
+    KeyT* __restrict__ keys_out = static_cast<KeyT*>(a.keys_out);
 
-    __shared__ u64 s_keys[TILE];
+    __shared__ KeyT s_keys[TILE];
     __shared__ u32 s_whist[WAVES * RADIX_BINS];
     __shared__ u32 s_binstart[RADIX_BINS];
     __shared__ u32 s_delta[RADIX_BINS];
@@ -219,36 +240,62 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
     const u32 sh = (u32)a.shift & 31u;
     const u32 bits = (u32)a.bits;
     const u32 mask = (1u << bits) - 1u;
-#define CSA_DIGIT(k64) __builtin_amdgcn_ubfe(HI ? (u32)((k64) >> 32) : (u32)(k64), sh, bits)
+#define CSA_DIGIT(kk) __builtin_amdgcn_ubfe(HI ? (u32)((u64)(kk) >> 32) : (u32)(kk), sh, bits)
+#ifdef __HIP_DEVICE_COMPILE__
+#define CSA_LDS_ORDER() asm volatile("" ::: "memory")
+#else
+#define CSA_LDS_ORDER() __builtin_amdgcn_wave_barrier() /* CPU emulation: lanes are threads, order them for real */
+#endif
 
+    CSA_OSTAMP(0);
     // ---- load: wave-striped, so that consecutive lanes read consecutive pairs ----
-    u64 key[ITEMS];
+    KeyT key[ITEMS];
     u32 val[ITEMS];
+    const u32 first_local = w * (WAVE * ITEMS) + lane;
+    if (valid == (u32)TILE) { // every tile but the last: no bounds checks, all loads in flight at once
 #pragma unroll
-    for (int k = 0; k < ITEMS; ++k) {
-        const u32 local = w * (WAVE * ITEMS) + k * WAVE + lane;
-        const u64 i = base + local;
-        if (local < valid) {
+        for (int k = 0; k < ITEMS; ++k) {
+            const u64 i = base + first_local + k * WAVE;
             if (SRC == SRC_PAIRS) {
-                key[k] = a.keys_in[i];
+                key[k] = keys_in[i];
                 val[k] = a.vals_in[i];
             } else if (SRC == SRC_TEXT) {
                 val[k] = virtual_to_suffix((u32)i, a.text_n, a.tail);
-                key[k] = load_kgram(a.text, a.text_n, val[k], a.word);
+                key[k] = (KeyT)load_kgram(a.text, a.text_n, val[k], a.word);
             } else {
                 val[k] = a.vals_in[i];
-                key[k] = load_kgram(a.text, a.text_n, val[k], a.word);
+                key[k] = (KeyT)load_kgram(a.text, a.text_n, val[k], a.word);
             }
-        } else {
-            key[k] = ~0ull; // padding: largest digit, and behind every real pair of the tile
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            const u32 local = first_local + k * WAVE;
+            const u64 i = base + local;
+            key[k] = ~(KeyT)0; // padding: largest digit, and behind every real pair of the tile
             val[k] = 0;
+            if (local < valid) {
+                if (SRC == SRC_PAIRS) {
+                    key[k] = keys_in[i];
+                    val[k] = a.vals_in[i];
+                } else if (SRC == SRC_TEXT) {
+                    val[k] = virtual_to_suffix((u32)i, a.text_n, a.tail);
+                    key[k] = (KeyT)load_kgram(a.text, a.text_n, val[k], a.word);
+                } else {
+                    val[k] = a.vals_in[i];
+                    key[k] = (KeyT)load_kgram(a.text, a.text_n, val[k], a.word);
+                }
+            }
         }
     }
 
     // ---- rank each pair among the pairs of its wave that share its digit ----
     // For every digit bit, (ballot of "bit set") XOR (all-ones if my own bit is set) has a 0 exactly at the lanes
     // that agree with me on that bit; OR-ed over the bits, `differ` marks the lanes whose digit is not mine.
-    volatile u32* whist = s_whist + w * RADIX_BINS;
+    // The per-wave counters are plain LDS words: a wave executes its LDS instructions in order, so the counter
+    // update of one item is seen by the next item's read; the empty asm statements only keep the compiler from
+    // moving those accesses across each other.
+    u32* whist = s_whist + w * RADIX_BINS;
     u32 pos[ITEMS];
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
@@ -264,13 +311,14 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
         const u32 same_lo = ~differ_lo, same_hi = ~differ_hi;
         const u32 before = __builtin_amdgcn_mbcnt_hi(same_hi, __builtin_amdgcn_mbcnt_lo(same_lo, 0u));
         const u32 prev = whist[d];
-        __builtin_amdgcn_wave_barrier();
+        CSA_LDS_ORDER();
         if (before == 0)
             whist[d] = prev + __popc(same_lo) + __popc(same_hi);
-        __builtin_amdgcn_wave_barrier();
+        CSA_LDS_ORDER();
         pos[k] = prev + before;
     }
     __syncthreads();
+    CSA_OSTAMP(1);
 
     // ---- one thread per digit: offsets of the waves inside the tile, tile totals; publish them at once ----
     u32 total = 0, real = 0;
@@ -284,7 +332,7 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
         real = total;
         if (t == mask)
             real -= (u32)TILE - valid; // padding pairs all carry the largest digit
-        lb_publish(a.lookback + t, RADIX_BINS, tile, a.epoch, real);
+        lb2_publish(a.lookback + t, RADIX_BINS, tile, a.epoch, real);
     }
     // exclusive scan of the 256 totals (padding included: it occupies LDS slots too)
     u32 binstart = 0;
@@ -310,11 +358,14 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
         pos[k] += s_binstart[d] + s_whist[w * RADIX_BINS + d];
         s_keys[pos[k]] = key[k];
     }
+    CSA_OSTAMP(2);
     if (t < RADIX_BINS) {
-        const u32 excl = lb_wait_exclusive<false>(a.lookback + t, RADIX_BINS, tile, a.epoch, real, a.err);
+        const u32 excl = lb2_wait_exclusive(a.lookback + t, a.lookback_groups + t, RADIX_BINS, tile, a.epoch, real, a.err);
         s_delta[t] = a.digit_base[t] + excl - binstart; // wraps; added back to an LDS slot below
     }
+    CSA_OSTAMP(3);
     __syncthreads();
+    CSA_OSTAMP(4);
 
     // ---- write runs of equal digits to their global places ----
     u32 dst[ITEMS];
@@ -322,9 +373,9 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
     for (int k = 0; k < ITEMS; ++k) {
         const u32 q = k * BLOCK + t;
         if (q < valid) {
-            const u64 kk = s_keys[q];
+            const KeyT kk = s_keys[q];
             dst[k] = q + s_delta[CSA_DIGIT(kk)];
-            a.keys_out[dst[k]] = kk;
+            keys_out[dst[k]] = kk;
         }
     }
     __syncthreads();
@@ -339,7 +390,9 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
         if (q < valid)
             a.vals_out[dst[k]] = s_vals[q];
     }
+    CSA_OSTAMP(5);
 #undef CSA_DIGIT
+#undef CSA_LDS_ORDER
 }
 
 } // namespace csa

@@ -127,6 +127,17 @@ inline T __shfl_up(T var, unsigned delta)
     return r;
 }
 
+template <typename T>
+inline T __shfl_xor(T var, unsigned mask)
+{
+    hipemu::Wave* w = hipemu::wave;
+    w->buf[hipemu::lane] = (uint64_t)var;
+    w->bar.arrive_and_wait();
+    const T r = (T)w->buf[(hipemu::lane ^ mask) & 63u];
+    w->bar.arrive_and_wait();
+    return r;
+}
+
 inline int __popc(unsigned v) { return __builtin_popcount(v); }
 inline int __popcll(unsigned long long v) { return __builtin_popcountll(v); }
 
