@@ -366,47 +366,70 @@ __global__ __launch_bounds__(BLOCK) void smallsort_kernel(SmallSortArgs a)
     }
     __syncthreads();
 
+    // group of every own element; members of large groups are counted so that the block reserves their slots in
+    // the large-group list with ONE atomic (one atomic per wave on a single counter serialises the whole launch
+    // when most of the list is in large groups)
+    u32 g[ITEMS], gs[ITEMS], ge[ITEMS];
+    u32 kind = 0; // 2 bits per item: 0 = not mine, 1 = small group, 2 = large group
+    u32 n_big = 0;
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         const long long e = t0 + k * BLOCK + t;
-        bool in = e < (long long)a.m;
-        u32 g = 0, gs = 0, ge = 0;
-        if (in) {
-            g = a.gids[e];
-            if (g < a.groups) {
-                gs = a.gstart[g];
-                ge = a.gstart[g + 1];
+        g[k] = gs[k] = ge[k] = 0;
+        if (e < (long long)a.m) {
+            g[k] = a.gids[e];
+            bool ok = g[k] < a.groups;
+            if (ok) {
+                gs[k] = a.gstart[g[k]];
+                ge[k] = a.gstart[g[k] + 1];
+                ok = (long long)gs[k] <= e && e < (long long)ge[k] && ge[k] <= a.m;
             }
-            if (g >= a.groups || !((long long)gs <= e && e < (long long)ge && ge <= a.m)) {
+            if (!ok) {
                 atomicExch(a.err, DEV_ERR_SMALLSORT_TABLES); // the element is not inside its group's range
-                in = false;
+            } else if (ge[k] - gs[k] > (u32)MAXG) {
+                kind |= 2u << (2 * k);
+                n_big++;
+            } else {
+                kind |= 1u << (2 * k);
             }
         }
-        const bool big = in && (ge - gs > (u32)MAXG);
-        const u64 key = ((u64)g << a.sec_bits) | (u64)sec[k];
-        if (in && !big) {
+    }
+    __shared__ u32 s_wbig[BLOCK / WAVE];
+    __shared__ u32 s_bigbase;
+    const u32 lane = t & 63u, w = t >> 6;
+    const u32 incl = wave_incl_sum(n_big);
+    if (lane == 63u)
+        s_wbig[w] = incl;
+    __syncthreads();
+    u32 slot = incl - n_big; // exclusive prefix inside the block
+    u32 block_big = 0;
+    for (u32 ww = 0; ww < BLOCK / WAVE; ++ww) {
+        if (ww < w)
+            slot += s_wbig[ww];
+        block_big += s_wbig[ww];
+    }
+    if (t == 0)
+        s_bigbase = block_big ? atomicAdd(a.big_count, block_big) : 0u;
+    __syncthreads();
+    slot += s_bigbase;
+
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const long long e = t0 + k * BLOCK + t;
+        const u32 what = (kind >> (2 * k)) & 3u;
+        const u64 key = ((u64)g[k] << a.sec_bits) | (u64)sec[k];
+        if (what == 1u) {
             u32 cnt = 0;
-            for (u32 j = gs; j < ge; ++j) {
+            for (u32 j = gs[k]; j < ge[k]; ++j) {
                 const u32 v = s_sec[(long long)j - lo];
                 cnt += (v < sec[k] || (v == sec[k] && (long long)j < e)) ? 1u : 0u;
             }
-            a.keys_out[gs + cnt] = key;
-            a.sufs_out[gs + cnt] = x[k];
-        }
-        // big groups: one atomic per wave reserves the slots
-        const u64 bal = __ballot(big);
-        if (bal) {
-            const u32 lane = lane_id();
-            const u32 leader = (u32)__builtin_ctzll(bal);
-            u32 basepos = 0;
-            if (lane == leader)
-                basepos = atomicAdd(a.big_count, (u32)__popcll(bal));
-            basepos = __shfl(basepos, leader);
-            if (big) {
-                const u32 slot = basepos + (u32)__popcll(bal & ((1ull << lane) - 1ull));
-                a.big_keys[slot] = key;
-                a.big_sufs[slot] = x[k];
-            }
+            a.keys_out[gs[k] + cnt] = key;
+            a.sufs_out[gs[k] + cnt] = x[k];
+        } else if (what == 2u) {
+            a.big_keys[slot] = key;
+            a.big_sufs[slot] = x[k];
+            slot++;
         }
     }
 }
