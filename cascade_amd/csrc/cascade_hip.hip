@@ -96,6 +96,8 @@ struct csa_handle {
     u64* lookback = nullptr;
     u64 lookback_words = 0;
     u64 lookback_tile_words = 0;
+    u32* tile_tables = nullptr; // rerank: [rank_tiles_cap][4] tile aggregates, the same of prefixes, [RERANK_SLABS][4] slab totals
+    u64 rank_tiles_cap = 0;
     u32* ghist = nullptr;      // [MAX_PASSES][256]
     u32* digit_base = nullptr; // [MAX_PASSES][256]
     u32* tickets = nullptr;    // [TICKET_POOL]
@@ -439,35 +441,19 @@ int deferred_rank_update(Launch& L, const u32* pos, const DeferBuffers& buf, u32
 int launch_rerank(Launch& L, RerankArgs& a)
 {
     csa_handle* h = L.h;
-    a.lookback = h->lookback;
-    a.epoch = next_epoch(h);
+    const u32 tiles = (u32)(((u64)a.m + RANK_TILE - 1) / RANK_TILE);
+    a.tile_agg = h->tile_tables;
+    a.tile_prefix = h->tile_tables + (u64)h->rank_tiles_cap * 4;
+    a.slab_total = h->tile_tables + (u64)h->rank_tiles_cap * 8;
+    a.slab = (tiles + RERANK_SLABS - 1) / RERANK_SLABS;
     a.err = h->counts + 2;
     a.counts = h->counts;
-    int rc = next_ticket(L, &a.ticket);
-    if (rc)
-        return rc;
-    const u32 tiles = (u32)(((u64)a.m + RANK_TILE - 1) / RANK_TILE);
-#ifdef CSA_TIMING_DEBUG
-    static unsigned long long* dbg = nullptr; // experiments only: stamps of the first (largest) launch are dumped
-    static bool dumped = false;
-    if (!dbg)
-        (void)hipMalloc((void**)&dbg, (size_t)8 * 8 * ((h->cap + RANK_TILE - 1) / RANK_TILE + 1));
-    a.dbg = dumped ? nullptr : dbg;
-#endif
-    hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS>), dim3(tiles), dim3(RANK_BLOCK), 0, L.stream, a);
+    const u32 slabs = (tiles + a.slab - 1) / a.slab;
+    hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS, false>), dim3(tiles), dim3(RANK_BLOCK), 0, L.stream, a);
+    hipLaunchKernelGGL(rerank_scan_kernel, dim3(slabs), dim3(1024), 0, L.stream, a.tile_agg, a.tile_prefix, tiles, a.slab,
+                       a.slab_total);
+    hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS, true>), dim3(tiles), dim3(RANK_BLOCK), 0, L.stream, a);
     HIP_TRY(hipGetLastError());
-#ifdef CSA_TIMING_DEBUG
-    if (!dumped && getenv("CSA_TIMING_DUMP")) {
-        (void)hipStreamSynchronize(L.stream);
-        std::vector<unsigned long long> hbuf((size_t)tiles * 8);
-        (void)hipMemcpy(hbuf.data(), dbg, hbuf.size() * 8, hipMemcpyDeviceToHost);
-        if (FILE* f = fopen(getenv("CSA_TIMING_DUMP"), "wb")) {
-            fwrite(hbuf.data(), 8, hbuf.size(), f);
-            fclose(f);
-        }
-        dumped = true;
-    }
-#endif
     return CSA_OK;
 }
 
@@ -736,6 +722,8 @@ int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
     alloc((void**)&h->gstart[0], (cap / 2 + 2) * 4);
     alloc((void**)&h->gstart[1], (cap / 2 + 2) * 4);
     alloc((void**)&h->lookback, h->lookback_words * 8);
+    h->rank_tiles_cap = rank_tiles + 1;
+    alloc((void**)&h->tile_tables, (h->rank_tiles_cap * 4 * 2 + RERANK_SLABS * 4) * sizeof(u32));
     alloc((void**)&h->ghist, (MAX_PASSES + 2) * RADIX_BINS * 4);
     alloc((void**)&h->digit_base, MAX_PASSES * RADIX_BINS * 4);
     alloc((void**)&h->tickets, TICKET_POOL * 4);
@@ -775,6 +763,7 @@ void csa_destroy(csa_handle* h)
     (void)hipFree(h->gprim[0]);
     (void)hipFree(h->gprim[1]);
     (void)hipFree(h->lookback);
+    (void)hipFree(h->tile_tables);
     (void)hipFree(h->ghist);
     (void)hipFree(h->digit_base);
     (void)hipFree(h->tickets);

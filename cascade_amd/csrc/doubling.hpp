@@ -8,7 +8,10 @@
 namespace csa {
 
 // ---------------------------------------------------------------------------------------------
-// Rank assignment + compaction, one pass with decoupled look-back (four chains).
+// Rank assignment + compaction in three launches: per-tile aggregates, a scan of the aggregates over the tiles,
+// and the pass that applies them. (A single launch with a decoupled look-back over four chains was measured at
+// 2.5 to 4 times the duration of these three on this part: with 8 XCDs the look-back words travel over the
+// fabric, and the few resident workgroups per CU spent most of their life waiting for their predecessors.)
 //
 // Input: the active suffixes sorted by key, keys[c] / sufs[c] for c in [0, m).
 //   generation 0 : key = packed K-gram(s); one primary group (the whole partition, rank 0)
@@ -46,24 +49,16 @@ struct RerankArgs {
     u32* gprim_out;
     u32* gstart_out; // index in the next active list where each new group starts; [groups] = survivors
     u32* counts; // [0] = survivors, [1] = their groups (written by the last tile)
-    u64* lookback; // [tiles][4]
-    u32* ticket;
-    u32 epoch;
+    u32* tile_agg;    // [tiles][4]: last key-run head, last group head, survivors, new groups of each tile
+    u32* tile_prefix; // [tiles][4]: the same, combined over the earlier tiles of the tile's slab (max, max, sum, sum)
+    u32* slab_total;  // [RERANK_SLABS][4]: combination over each slab of tiles
+    u32 slab;         // tiles per slab
     u32* err;
-#ifdef CSA_TIMING_DEBUG
-    unsigned long long* dbg; // [tiles][8] cycle stamps (experiments only)
-#endif
 };
 
-#ifdef CSA_TIMING_DEBUG
-#define CSA_STAMP(slot)                                                    \
-    if (a.dbg && threadIdx.x == 0)                                         \
-    a.dbg[(unsigned long long)tile * 8 + (slot)] = __builtin_readcyclecounter()
-#else
-#define CSA_STAMP(slot)
-#endif
-
-template <int BLOCK, int ITEMS>
+// APPLY = false: writes the tile's aggregates to tile_agg. APPLY = true: reads the tile's exclusive prefix from
+// tile_prefix (rerank_scan_kernel in between) and does the work.
+template <int BLOCK, int ITEMS, bool APPLY>
 __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
 {
     constexpr int TILE = BLOCK * ITEMS;
@@ -77,27 +72,15 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
     __shared__ u32 s_suf[PADDED]; // later: tables of the new groups (first rank, start)
     __shared__ u32 s_rv[TILE];    // new ranks in list order (deferred rank update only)
     __shared__ u32 s_wagg[WAVES][4];
-    __shared__ u32 s_tileprefix[4];
-    __shared__ u32 s_tiletotal[4];
-    __shared__ u32 s_tile;
 #define CSA_PAD(q) ((q) + (q) / ITEMS)
 
     const u32 t = threadIdx.x;
     const u32 lane = t & 63u;
     const u32 w = t >> 6;
-#ifdef CSA_NO_TICKET
-    if (t == 0)
-        s_tile = blockIdx.x;
-#else
-    if (t == 0)
-        s_tile = atomicAdd(a.ticket, 1u);
-#endif
-    __syncthreads();
-    const u32 tile = s_tile;
+    const u32 tile = blockIdx.x;
     const u64 tile_base = (u64)tile * TILE;
     const u64 base = tile_base + (u64)t * ITEMS;
     const u32 m = a.m;
-    CSA_STAMP(0);
 
     // striped load into LDS: slot q holds element tile_base + q - 1
 #pragma unroll
@@ -116,7 +99,6 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
         s_suf[CSA_PAD(q)] = in ? a.sufs[c] : 0;
     }
     __syncthreads();
-    CSA_STAMP(1);
 
     // blocked read: elements base - 1 .. base + ITEMS
     u64 key[ITEMS + 2];
@@ -185,35 +167,40 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
         xc += s_wagg[ww][2];
         xh += s_wagg[ww][3];
     }
-    // tile aggregate -> look-back, one wave per chain (max a, max b, sum survivors, sum new groups)
-    CSA_STAMP(2);
-    static_assert(WAVES >= 4, "one wave per look-back chain");
-    if (w < 4) {
-        u32 agg = 0;
-        for (int ww = 0; ww < WAVES; ++ww)
-            agg = w < 2 ? (agg > s_wagg[ww][w] ? agg : s_wagg[ww][w]) : agg + s_wagg[ww][w];
-        u32 excl;
-        if (w < 2)
-            excl = lb_wave_exclusive<true>(a.lookback + w, 4, tile, a.epoch, agg, a.err);
-        else
-            excl = lb_wave_exclusive<false>(a.lookback + w, 4, tile, a.epoch, agg, a.err);
-        if (lane == 0) {
-            s_tileprefix[w] = excl;
-            s_tiletotal[w] = excl + agg;
+    if (!APPLY) {
+        if (t < 4) {
+            u32 agg = 0;
+            for (int ww = 0; ww < WAVES; ++ww)
+                agg = t < 2 ? (agg > s_wagg[ww][t] ? agg : s_wagg[ww][t]) : agg + s_wagg[ww][t];
+            a.tile_agg[(u64)tile * 4 + t] = agg;
         }
+        return;
     }
-    CSA_STAMP(3);
-    __syncthreads();
+    u32 tile_total_surv = 0, tile_total_heads = 0;
+    for (int ww = 0; ww < WAVES; ++ww) {
+        tile_total_surv += s_wagg[ww][2];
+        tile_total_heads += s_wagg[ww][3];
+    }
+    // prefix of the tile = totals of the slabs before its slab, combined with its prefix inside the slab
+    u32 pre_a = a.tile_prefix[(u64)tile * 4 + 0], pre_b = a.tile_prefix[(u64)tile * 4 + 1];
+    u32 tile_rc = a.tile_prefix[(u64)tile * 4 + 2], tile_rh = a.tile_prefix[(u64)tile * 4 + 3];
+    for (u32 sl = 0; sl < tile / a.slab; ++sl) {
+        const u32 sa_ = a.slab_total[sl * 4 + 0], sb_ = a.slab_total[sl * 4 + 1];
+        pre_a = pre_a > sa_ ? pre_a : sa_;
+        pre_b = pre_b > sb_ ? pre_b : sb_;
+        tile_rc += a.slab_total[sl * 4 + 2];
+        tile_rh += a.slab_total[sl * 4 + 3];
+    }
     if (t == 0 && tile_base + TILE >= m) { // the last tile knows the totals
-        a.counts[0] = s_tiletotal[2];
-        a.counts[1] = s_tiletotal[3];
-        a.gstart_out[s_tiletotal[3]] = s_tiletotal[2]; // one-past-the-end entry: gstart[groups] = survivors
+        a.counts[0] = tile_rc + tile_total_surv;
+        a.counts[1] = tile_rh + tile_total_heads;
+        a.gstart_out[tile_rh + tile_total_heads] = tile_rc + tile_total_surv; // gstart[groups] = survivors
     }
-    const u32 tile_rc = s_tileprefix[2], tile_rh = s_tileprefix[3]; // survivors / new groups before this tile
-    u32 ra = xa > s_tileprefix[0] ? xa : s_tileprefix[0];
-    u32 rb = xb > s_tileprefix[1] ? xb : s_tileprefix[1];
+    u32 ra = xa > pre_a ? xa : pre_a;
+    u32 rb = xb > pre_b ? xb : pre_b;
     u32 rc = xc; // tile-local from here on
     u32 rh = xh;
+    __syncthreads(); // every thread has read s_wagg and holds its elements in registers: the staging arrays are free
     u32* s_osuf = reinterpret_cast<u32*>(s_key); // [TILE] survivors of the tile, compacted
     u32* s_ogid = s_osuf + TILE;                 // [TILE] their new group ids
     u32* s_oprim = s_suf;                        // [TILE / 2] first rank of each new group of the tile
@@ -261,10 +248,9 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
             }
         }
     }
-    CSA_STAMP(4);
     __syncthreads();
     // striped write-out of what the tile produced
-    const u32 n_surv = s_tiletotal[2] - tile_rc, n_heads = s_tiletotal[3] - tile_rh;
+    const u32 n_surv = tile_total_surv, n_heads = tile_total_heads;
     for (u32 i = t; i < n_surv; i += BLOCK) {
         a.sufs_out[tile_rc + i] = s_osuf[i];
         a.gids_out[tile_rc + i] = s_ogid[i];
@@ -276,8 +262,72 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
     if (a.rank_vals)
         for (u32 i = t; i < (u32)TILE && tile_base + i < m; i += BLOCK)
             a.rank_vals[tile_base + i] = s_rv[i];
-    CSA_STAMP(5);
 #undef CSA_PAD
+}
+
+// Exclusive combination of the tile aggregates (max, max, sum, sum) over the tiles of one slab: workgroup s handles
+// tiles [s * slab, (s + 1) * slab) and writes each tile's prefix relative to the slab start plus the slab's total.
+// The applying pass adds the totals of the slabs before its own (at most RERANK_SLABS of them).
+constexpr u32 RERANK_SLABS = 64;
+
+__global__ __launch_bounds__(1024) void rerank_scan_kernel(const u32* __restrict__ tile_agg, u32* __restrict__ tile_prefix,
+                                                           u32 tiles, u32 slab, u32* __restrict__ slab_total)
+{
+    __shared__ u32 s_w[16][4];
+    const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
+    const u32 slab_first = blockIdx.x * slab;
+    const u32 slab_last = slab_first + slab < tiles ? slab_first + slab : tiles;
+    const u32 per = (slab + 1023) / 1024;
+    const u32 first = slab_first + t * per < slab_last ? slab_first + t * per : slab_last;
+    const u32 last = first + per < slab_last ? first + per : slab_last;
+    const uint4* agg4 = reinterpret_cast<const uint4*>(tile_agg);
+    uint4* pre4 = reinterpret_cast<uint4*>(tile_prefix);
+    u32 ra = 0, rb = 0, rc = 0, rh = 0;
+    for (u32 i = first; i < last; ++i) {
+        const uint4 v = agg4[i];
+        ra = ra > v.x ? ra : v.x;
+        rb = rb > v.y ? rb : v.y;
+        rc += v.z;
+        rh += v.w;
+    }
+    const u32 ia = wave_incl_max(ra), ib = wave_incl_max(rb), ic = wave_incl_sum(rc), ih = wave_incl_sum(rh);
+    if (lane == 63u) {
+        s_w[w][0] = ia;
+        s_w[w][1] = ib;
+        s_w[w][2] = ic;
+        s_w[w][3] = ih;
+    }
+    __syncthreads();
+    u32 xa = __shfl_up(ia, 1), xb = __shfl_up(ib, 1), xc = __shfl_up(ic, 1), xh = __shfl_up(ih, 1);
+    if (lane == 0)
+        xa = xb = xc = xh = 0;
+    u32 ta = 0, tb = 0, tc = 0, th = 0;
+    for (u32 ww = 0; ww < 16; ++ww) {
+        if (ww < w) {
+            xa = xa > s_w[ww][0] ? xa : s_w[ww][0];
+            xb = xb > s_w[ww][1] ? xb : s_w[ww][1];
+            xc += s_w[ww][2];
+            xh += s_w[ww][3];
+        }
+        ta = ta > s_w[ww][0] ? ta : s_w[ww][0];
+        tb = tb > s_w[ww][1] ? tb : s_w[ww][1];
+        tc += s_w[ww][2];
+        th += s_w[ww][3];
+    }
+    for (u32 i = first; i < last; ++i) {
+        const uint4 v = agg4[i];
+        pre4[i] = make_uint4(xa, xb, xc, xh);
+        xa = xa > v.x ? xa : v.x;
+        xb = xb > v.y ? xb : v.y;
+        xc += v.z;
+        xh += v.w;
+    }
+    if (t == 0) {
+        slab_total[blockIdx.x * 4 + 0] = ta;
+        slab_total[blockIdx.x * 4 + 1] = tb;
+        slab_total[blockIdx.x * 4 + 2] = tc;
+        slab_total[blockIdx.x * 4 + 3] = th;
+    }
 }
 
 // Last step of the deferred rank update. The (text position, rank) pairs of generation 0 arrive sorted by the
