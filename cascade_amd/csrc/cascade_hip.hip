@@ -69,6 +69,7 @@ constexpr int EVENT_POOL = 2 * CSA_MAX_GENERATIONS * MAX_PASSES * 2;
 #ifndef CSA_DEFER_MIN
 #define CSA_DEFER_MIN (1u << 23)
 #endif
+constexpr u32 XCD_CHUNK = 16;
 constexpr u32 DEFER_MIN = CSA_DEFER_MIN;
 
 int bit_length(u64 v)
@@ -105,6 +106,7 @@ struct csa_handle {
     u32* counts = nullptr; // [2] survivors, groups; [2] error flag; [3] verifier flag
     u32* h_pinned = nullptr; // host mirror: [0..3] counts/err, [16 ..) histogram
     u32 epoch = 0;
+    u32 xcd_chunk = 0;         // tiles of a radix pass that one XCD takes in a row (0: numbered by arrival)
     u32 defer_min = DEFER_MIN; // lists at least this long use the bucketed rank update (env CASCADE_DEFER_MIN overrides)
     std::vector<hipEvent_t> events;
     hipEvent_t ev_gen[CSA_MAX_GENERATIONS + 2] = {};
@@ -242,20 +244,13 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
         a.lookback_groups = h->lookback + h->lookback_tile_words;
         a.epoch = next_epoch(h);
         a.err = h->counts + 2;
+        a.xcd_chunk = h->xcd_chunk;
         int rc = next_ticket(L, &a.ticket);
         if (rc)
             return rc;
         const bool timed = (L.flags & CSA_FLAG_KERNEL_TIMING) && L.events_used + 2 <= (int)h->events.size();
         if (timed)
             HIP_TRY(hipEventRecord(h->events[L.events_used], s));
-#ifdef CSA_TIMING_DEBUG
-        static unsigned long long* odbg = nullptr; // experiments only: stamps of one chosen full-size pass
-        static int pass_no = 0;
-        if (!odbg)
-            (void)hipMalloc((void**)&odbg, (size_t)8 * 8 * ((h->cap + SORT_TILE - 1) / SORT_TILE + 1));
-        ++pass_no;
-        a.dbg = (pass_no == 3 && getenv("CSA_OTIMING_DUMP")) ? odbg : nullptr;
-#endif
         const int use_src = first ? src : SRC_PAIRS;
         if (use_src == SRC_PAIRS)
             launch_onesweep<SRC_PAIRS>(a, s);
@@ -268,18 +263,6 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
             L.timed.push_back({L.events_used, (u64)n});
             L.events_used += 2;
         }
-#ifdef CSA_TIMING_DEBUG
-        if (a.dbg) {
-            (void)hipStreamSynchronize(s);
-            const u32 tiles = (u32)(((u64)n + SORT_TILE - 1) / SORT_TILE);
-            std::vector<unsigned long long> hbuf((size_t)tiles * 8);
-            (void)hipMemcpy(hbuf.data(), odbg, hbuf.size() * 8, hipMemcpyDeviceToHost);
-            if (FILE* f = fopen(getenv("CSA_OTIMING_DUMP"), "wb")) {
-                fwrite(hbuf.data(), 8, hbuf.size(), f);
-                fclose(f);
-            }
-        }
-#endif
         first = false;
         where ^= 1;
         (*passes_run)++;
@@ -421,6 +404,7 @@ int deferred_rank_update(Launch& L, const u32* pos, const DeferBuffers& buf, u32
             a.lookback_groups = h->lookback + h->lookback_tile_words;
             a.epoch = next_epoch(h);
             a.err = h->counts + 2;
+            a.xcd_chunk = h->xcd_chunk;
             int rc = next_ticket(L, &a.ticket);
             if (rc)
                 return rc;
@@ -707,6 +691,14 @@ int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
     if (rank_tiles * 4 > h->lookback_words)
         h->lookback_words = rank_tiles * 4;
     hipError_t e = hipGetDevice(&h->device);
+    // The XCD-aware tile order of the radix pass needs 8 * (XCD_CHUNK - 1) + 1 workgroups resident at once; every
+    // CU holds at least one, so a full MI355X (256 CUs) qualifies and a small partition of it falls back.
+    int cus = 0;
+    if (e == hipSuccess)
+        e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, h->device);
+    h->xcd_chunk = cus >= 2 * 8 * (int)XCD_CHUNK ? XCD_CHUNK : 0;
+    if (const char* c = getenv("CASCADE_XCD_CHUNK"))
+        h->xcd_chunk = (u32)strtoul(c, nullptr, 10);
     auto alloc = [&](void** p, u64 bytes) {
         if (e == hipSuccess)
             e = hipMalloc(p, bytes ? bytes : 4);

@@ -56,7 +56,9 @@ __device__ __forceinline__ u32 wave_incl_max(u32 v)
 // between launches. Words are read and written with relaxed agent-scope atomics only: status and
 // value travel in the same word, so no fence is needed and the accesses are coherent across XCDs.
 // Tiles are numbered by an atomic ticket taken when a workgroup starts, hence every predecessor
-// of a waiting tile is already resident or finished.
+// of a waiting tile is already resident or finished. (The radix pass may instead derive the tile from
+// the workgroup index; its predecessors are then at most a bounded number of dispatches behind.)
+// Every wait has a spin limit that turns a predecessor that never shows up into an error word.
 
 constexpr u32 LB_AGG = 1;  // value = this tile's aggregate
 constexpr u32 LB_INCL = 2; // value = aggregate of tiles [0, tile]
@@ -98,9 +100,6 @@ __device__ __forceinline__ u32 lb_wait_exclusive(u64* chain, u32 stride, u32 til
 {
     if (tile == 0)
         return 0;
-#ifdef CSA_EXPERIMENT_NO_LOOKBACK_WAIT
-    return 0; // timing experiment only: results are wrong
-#endif
     u32 excl = 0;
     long long next = (long long)tile - 1; // nearest predecessor not yet consumed
     u32 idle = 0;

@@ -179,21 +179,11 @@ struct OnesweepArgs {
     const u32* digit_base; // [256] for this pass
     u64* lookback;         // [tiles][256]
     u64* lookback_groups;  // [ceil(tiles / LB_GROUP)][256]
-    u32* ticket;           // zero before the launch
+    u32* ticket;           // zero before the launch (used when xcd_chunk == 0)
+    u32 xcd_chunk;         // consecutive tiles given to one XCD, or 0: tiles numbered by arrival
     u32 epoch;
     u32* err;
-#ifdef CSA_TIMING_DEBUG
-    unsigned long long* dbg; // [tiles][8] cycle stamps (experiments only)
-#endif
 };
-
-#ifdef CSA_TIMING_DEBUG
-#define CSA_OSTAMP(slot)                                                   \
-    if (a.dbg && threadIdx.x == 0)                                         \
-    a.dbg[(unsigned long long)tile * 8 + (slot)] = __builtin_readcyclecounter()
-#else
-#define CSA_OSTAMP(slot)
-#endif
 
 // predecessors a digit's look-back inspects per round
 #ifndef CSA_SORT_LB_W
@@ -229,8 +219,29 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
     const u32 lane = t & 63u;
     const u32 w = t >> 6;
 
-    if (t == 0)
-        s_tile = atomicAdd(a.ticket, 1u);
+    // Tile numbering. The hardware deals workgroups to the 8 XCDs round-robin (workgroup b runs on XCD b % 8), and
+    // each XCD has an L2 of its own. With xcd_chunk = C, every XCD works on chunks of C consecutive tiles, so the
+    // runs of one digit written by neighbouring tiles meet in the same L2 and leave it as full lines; measured
+    // 15% faster per pass than arrival order at C = 16. The predecessor of a tile may then belong to a workgroup
+    // dispatched up to 8 (C - 1) places later, so C is only used where that many workgroups are resident at
+    // once (the host decides). Tiles past the last whole group of 8 chunks, and every tile when C = 0, are
+    // numbered so that all predecessors have started.
+    if (t == 0) {
+        u32 tl;
+        if (a.xcd_chunk == 0) {
+            tl = atomicAdd(a.ticket, 1u);
+        } else {
+            const u32 b = blockIdx.x;
+            const u32 span = 8u * a.xcd_chunk;
+            const u32 whole = (gridDim.x / span) * span;
+            tl = b;
+            if (b < whole) {
+                const u32 x = b % 8u, q = b / 8u;
+                tl = ((q / a.xcd_chunk) * 8u + x) * a.xcd_chunk + q % a.xcd_chunk;
+            }
+        }
+        s_tile = tl;
+    }
     for (int i = t; i < WAVES * RADIX_BINS; i += BLOCK)
         s_whist[i] = 0;
     __syncthreads();
@@ -246,8 +257,6 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
 #else
 #define CSA_LDS_ORDER() __builtin_amdgcn_wave_barrier() /* CPU emulation: lanes are threads, order them for real */
 #endif
-
-    CSA_OSTAMP(0);
     // ---- load: wave-striped, so that consecutive lanes read consecutive pairs ----
     KeyT key[ITEMS];
     u32 val[ITEMS];
@@ -318,7 +327,6 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
         pos[k] = prev + before;
     }
     __syncthreads();
-    CSA_OSTAMP(1);
 
     // ---- one thread per digit: offsets of the waves inside the tile, tile totals; publish them at once ----
     u32 total = 0, real = 0;
@@ -358,14 +366,11 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
         pos[k] += s_binstart[d] + s_whist[w * RADIX_BINS + d];
         s_keys[pos[k]] = key[k];
     }
-    CSA_OSTAMP(2);
     if (t < RADIX_BINS) {
         const u32 excl = lb2_wait_exclusive(a.lookback + t, a.lookback_groups + t, RADIX_BINS, tile, a.epoch, real, a.err);
         s_delta[t] = a.digit_base[t] + excl - binstart; // wraps; added back to an LDS slot below
     }
-    CSA_OSTAMP(3);
     __syncthreads();
-    CSA_OSTAMP(4);
 
     // ---- write runs of equal digits to their global places ----
     u32 dst[ITEMS];
@@ -390,7 +395,6 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
         if (q < valid)
             a.vals_out[dst[k]] = s_vals[q];
     }
-    CSA_OSTAMP(5);
 #undef CSA_DIGIT
 #undef CSA_LDS_ORDER
 }

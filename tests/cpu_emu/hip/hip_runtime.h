@@ -201,6 +201,8 @@ constexpr unsigned hipHostMallocDefault = 0;
 inline const char* hipGetErrorString(hipError_t e) { return e == hipSuccess ? "success" : "emulated failure"; }
 inline hipError_t hipGetLastError() { return hipSuccess; }
 inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
+enum hipDeviceAttribute_t { hipDeviceAttributeMultiprocessorCount = 63 };
+inline hipError_t hipDeviceGetAttribute(int* v, hipDeviceAttribute_t, int) { *v = 1; return hipSuccess; } // one "CU"
 inline hipError_t hipMalloc(void** p, size_t bytes)
 {
     *p = std::malloc(bytes ? bytes : 1);
