@@ -31,6 +31,22 @@ def algorithmic_bytes(n, active):
     return per_gen, 14 * n
 
 
+def measured_traffic_per_pair():
+    """HBM bytes one radix pass moves per pair, from the FETCH_SIZE / WRITE_SIZE counter runs of this same command
+    that are summarised in profiles/ (lines 'fetch_bytes_per_pair = X' and 'write_bytes_per_pair = Y', already
+    scaled by what the counters read for the plain copy below). None where no summary is committed."""
+    path = os.path.join(ROOT, "profiles", "onesweep_c3_1b_pmc_traffic.txt")
+    got = {}
+    try:
+        for line in open(path):
+            for key in ("fetch_bytes_per_pair", "write_bytes_per_pair"):
+                if line.startswith(key) and "=" in line:
+                    got[key] = float(line.split("=")[1].split()[0])
+    except OSError:
+        return None
+    return got["fetch_bytes_per_pair"] + got["write_bytes_per_pair"] if len(got) == 2 else None
+
+
 def cpu_baseline(config, sample_n):
     """The reference's CPU suffix sort (test/query.cpp:42-55, compiled from its sources into oracle/_ref) on a
     scaled-down partition of the same construction; falls back to the C restatement where _ref is absent."""
@@ -87,6 +103,16 @@ def main():
     print(f"[bench] C{args.config} n={n} generated in {t_gen:.1f}s; scratch {sorter.bytes_per_suffix() * n / 2**30:.1f} GiB",
           file=sys.stderr, flush=True)
 
+    # One plain copy of known size (1 GiB read, 1 GiB written), outside the timed region: a counter run of this same
+    # command scales FETCH_SIZE / WRITE_SIZE by what they read for it.
+    cal = torch.empty(1 << 28, dtype=torch.int32, device=dev)
+    cal.fill_(1)
+    cal2 = torch.empty_like(cal)
+    cal2.copy_(cal)
+    torch.cuda.synchronize()
+    del cal, cal2
+    torch.cuda.empty_cache()
+
     for _ in range(args.warmup):
         sorter.sort(d_text, out=out)
     torch.cuda.synchronize()
@@ -125,12 +151,16 @@ def main():
     # dominant kernel: the one-sweep radix pass, timed per launch with HIP events on the sort's stream
     avg_launch_ms = radix_ms / radix_launches if radix_launches else 0.0
     achieved = (RADIX_PASS_BYTES_PER_PAIR * radix_pairs / (radix_ms * 1e-3) / 1e9) if radix_ms > 0 else 0.0
+    pairs_per_launch = radix_pairs / radix_launches if radix_launches else 0
+    per_pair = measured_traffic_per_pair() if (args.config == 3 and args.n is None and args.key_words == 1) else None
     roofline = {
         "bound": "hbm", "kernel": "onesweep_kernel (one radix pass over (key, index) pairs)",
         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+        "frac": round(achieved / HBM_PEAK_GBS, 4),
+        "traffic": round(per_pair * pairs_per_launch) if per_pair is not None else None,
+        "algorithmic_bytes_per_launch": round(RADIX_PASS_BYTES_PER_PAIR * pairs_per_launch),
         "launches_per_step": radix_launches / args.steps, "avg_launch_ms": round(avg_launch_ms, 4),
-        "pairs_per_launch": radix_pairs / radix_launches if radix_launches else 0,
+        "pairs_per_launch": pairs_per_launch,
         "share_of_step": round(radix_ms / args.steps / ms_per_step, 3),
     }
 

@@ -41,9 +41,14 @@ int fail(int code, const char* fmt, ...)
 #ifndef CSA_SORT_ITEMS
 #define CSA_SORT_ITEMS 16
 #endif
+#ifndef CSA_SORT32_ITEMS
+#define CSA_SORT32_ITEMS CSA_SORT_ITEMS
+#endif
 constexpr int SORT_BLOCK = CSA_SORT_BLOCK;
 constexpr int SORT_ITEMS = CSA_SORT_ITEMS;
+constexpr int SORT32_ITEMS = CSA_SORT32_ITEMS; // pairs per thread when the keys are 32-bit (same LDS bytes at twice the items)
 constexpr int SORT_TILE = SORT_BLOCK * SORT_ITEMS;
+static_assert(SORT32_ITEMS >= SORT_ITEMS, "the look-back words are sized for tiles of SORT_TILE pairs or more");
 #ifndef CSA_RANK_BLOCK
 #define CSA_RANK_BLOCK 256
 #endif
@@ -165,8 +170,9 @@ void launch_onesweep(const OnesweepArgs& a, hipStream_t s)
 
 void launch_onesweep32(const OnesweepArgs& a, hipStream_t s)
 {
-    const u32 tiles = (u32)(((u64)a.n + SORT_TILE - 1) / SORT_TILE);
-    hipLaunchKernelGGL((onesweep_kernel<u32, SORT_BLOCK, SORT_ITEMS, SRC_PAIRS, 0>), dim3(tiles), dim3(SORT_BLOCK), 0, s, a);
+    constexpr u32 TILE32 = SORT_BLOCK * SORT32_ITEMS;
+    const u32 tiles = (u32)(((u64)a.n + TILE32 - 1) / TILE32);
+    hipLaunchKernelGGL((onesweep_kernel<u32, SORT_BLOCK, SORT32_ITEMS, SRC_PAIRS, 0>), dim3(tiles), dim3(SORT_BLOCK), 0, s, a);
 }
 
 // Sorts n pairs by the digits of `plan`. The first pass that runs takes its input as `src` says
