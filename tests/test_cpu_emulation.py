@@ -57,6 +57,23 @@ def test_fixtures_through_the_emulated_kernels(emu, key_words):
         assert active == counts, name
 
 
+@pytest.mark.parametrize("key_words", [1, 2])
+def test_text_at_every_alignment_inside_an_eight_byte_word(emu, key_words):
+    # the first pass stages the text with aligned 8-byte loads: the text may start anywhere inside such a word, and
+    # its end (here a run of zeros, which ties with the key padding) anywhere too
+    rng = np.random.default_rng(7)
+    backing = np.zeros(2600, dtype=np.uint16)
+    base_off = (-backing.ctypes.data // 2) % 4  # symbols to the next 8-byte boundary
+    for off in range(4):
+        for n in (1301 + off, 1304):
+            T = backing[base_off + off:base_off + off + n]
+            T[:] = rng.integers(0, 3, n)
+            T[-5:] = 0
+            assert (T.ctypes.data % 8) == 2 * off
+            got, _, _ = emu_sort(emu, T, key_words)
+            assert np.array_equal(got, oracle_lib.build_sa40(np.array(T))), (off, n)
+
+
 def test_small_and_large_groups_take_both_paths(emu):
     # 2 symbols, no separators: generation 1 has a few huge groups (radix path), later ones small groups (in-tile path)
     T = texts.random_text(6000, 2, 5, sep_every=0)

@@ -187,6 +187,25 @@ def test_host_buffer_entry_point_and_file_interface(torch_mod, tmp_path):
     assert np.array_equal(np.fromfile(op, dtype=np.uint8), sa40)
 
 
+def test_text_pointer_at_every_alignment(torch_mod, sorter, sorter2):
+    # the text may start anywhere inside an aligned 8-byte word (a window of a larger buffer), and end anywhere too
+    torch = torch_mod
+    rng = np.random.default_rng(11)
+    backing = torch.zeros(40000, dtype=torch.int16, device="cuda")
+    for off in range(4):
+        for n in (20001 + off, 24576, 8193 - off):
+            T = rng.integers(0, 3, n).astype(np.uint16)
+            T[-6:] = 0
+            window = backing[off:off + n]
+            window.copy_(torch.from_numpy(T.view(np.int16)))
+            assert window.data_ptr() % 8 == 2 * off
+            want = oracle_lib.build_sa40(T)
+            for s in (sorter, sorter2):
+                print(f"  sort off={off} n={n} key_words={s.key_words}", flush=True)
+                got = s.sort(window).cpu().numpy()
+                assert np.array_equal(got, want), (off, n, s.key_words)
+
+
 def test_repeatable(torch_mod, sorter):
     from cascade_amd import workloads
     T = workloads.generate(5, 1 << 18)
