@@ -76,6 +76,18 @@ constexpr int EVENT_POOL = 2 * CSA_MAX_GENERATIONS * MAX_PASSES * 2;
 #endif
 constexpr u32 XCD_CHUNK = 16;
 constexpr u32 DEFER_MIN = CSA_DEFER_MIN;
+// Later generations: when at least half of the sorted list changes its rank, and at least WINDOW_MIN_CHANGED
+// suffixes in all, the rank writes of the generation are bucketed into windows of 1 << WINDOW_LOG2 positions of
+// rank[] first. Partitions that fit one window never need it.
+#ifndef CSA_WINDOW_LOG2
+#define CSA_WINDOW_LOG2 23
+#endif
+#ifndef CSA_WINDOW_MIN_CHANGED
+#define CSA_WINDOW_MIN_CHANGED (1u << 22)
+#endif
+constexpr int WINDOW_LOG2 = CSA_WINDOW_LOG2;
+constexpr u32 WINDOW_MIN_CHANGED = CSA_WINDOW_MIN_CHANGED;
+
 
 int bit_length(u64 v)
 {
@@ -102,17 +114,19 @@ struct csa_handle {
     u64* lookback = nullptr;
     u64 lookback_words = 0;
     u64 lookback_tile_words = 0;
-    u32* tile_tables = nullptr; // rerank: [rank_tiles_cap][4] tile aggregates, the same of prefixes, [RERANK_SLABS][4] slab totals
+    u32* tile_tables = nullptr; // rerank: [rank_tiles_cap][4] tile aggregates, the same of prefixes, [rank_tiles_cap] splits,
+                                // [RERANK_SLABS][5] slab totals
     u64 rank_tiles_cap = 0;
     u32* ghist = nullptr;      // [MAX_PASSES][256]
     u32* digit_base = nullptr; // [MAX_PASSES][256]
     u32* tickets = nullptr;    // [TICKET_POOL]
     u32 ticket_next = 0;
-    u32* counts = nullptr; // [2] survivors, groups; [2] error flag; [3] verifier flag
+    u32* counts = nullptr; // [2] error flag; [3] verifier flag; [4] members of large groups
     u32* h_pinned = nullptr; // host mirror: [0..3] counts/err, [16 ..) histogram
     u32 epoch = 0;
     u32 xcd_chunk = 0;         // tiles of a radix pass that one XCD takes in a row (0: numbered by arrival)
     u32 defer_min = DEFER_MIN; // lists at least this long use the bucketed rank update (env CASCADE_DEFER_MIN overrides)
+    u32 window_min_changed = WINDOW_MIN_CHANGED; // env CASCADE_WINDOW_MIN_CHANGED overrides (0xFFFFFFFF: never)
     std::vector<hipEvent_t> events;
     hipEvent_t ev_gen[CSA_MAX_GENERATIONS + 2] = {};
     bool ev_gen_ready = false;
@@ -311,8 +325,8 @@ int ensure_events(csa_handle* h, bool kernel_timing)
     return CSA_OK;
 }
 
-// counts: [0] survivors, [1] their groups, [2] device error flag, [3] verifier flag, [4] members of large groups
-int read_counts(Launch& L, u32* survivors, u32* groups, u32* big)
+// counts: [2] device error flag, [3] verifier flag, [4] members of large groups. Waits for the stream.
+int read_counts(Launch& L, u32* big)
 {
     csa_handle* h = L.h;
     HIP_TRY(hipMemcpyAsync(h->h_pinned, h->counts, 8 * sizeof(u32), hipMemcpyDeviceToHost, L.stream));
@@ -325,10 +339,6 @@ int read_counts(Launch& L, u32* survivors, u32* groups, u32* big)
         const u32 code = h->h_pinned[2];
         return fail(CSA_ERR_INTERNAL, "device invariant %u failed: %s", code, code < 5 ? what[code] : "unknown");
     }
-    if (survivors)
-        *survivors = h->h_pinned[0];
-    if (groups)
-        *groups = h->h_pinned[1];
     if (big)
         *big = h->h_pinned[4];
     return CSA_OK;
@@ -428,44 +438,103 @@ int deferred_rank_update(Launch& L, const u32* pos, const DeferBuffers& buf, u32
     return CSA_OK;
 }
 
-int launch_rerank(Launch& L, RerankArgs& a)
+// Bucketed rank update of a later generation: rank[pos[c]] = vals[c] wherever vals[c] != NO_RANK, c < m.
+// One radix pass on the position bits above the window size, then a plain scatter that stays inside one window
+// of rank[] at a time.
+int windowed_rank_update(Launch& L, const u32* pos, const DeferBuffers& buf, u32 m, u32 n)
 {
     csa_handle* h = L.h;
-    const u32 tiles = (u32)(((u64)a.m + RANK_TILE - 1) / RANK_TILE);
-    a.tile_agg = h->tile_tables;
-    a.tile_prefix = h->tile_tables + (u64)h->rank_tiles_cap * 4;
-    a.slab_total = h->tile_tables + (u64)h->rank_tiles_cap * 8;
-    a.slab = (tiles + RERANK_SLABS - 1) / RERANK_SLABS;
-    a.err = h->counts + 2;
-    a.counts = h->counts;
-    const u32 slabs = (tiles + a.slab - 1) / a.slab;
-    hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS, false>), dim3(tiles), dim3(RANK_BLOCK), 0, L.stream, a);
-    hipLaunchKernelGGL(rerank_scan_kernel, dim3(slabs), dim3(1024), 0, L.stream, a.tile_agg, a.tile_prefix, tiles, a.slab,
-                       a.slab_total);
-    hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS, true>), dim3(tiles), dim3(RANK_BLOCK), 0, L.stream, a);
+    hipStream_t s = L.stream;
+    const int nb = bit_length(n - 1);
+    int top = nb - WINDOW_LOG2;
+    if (top > 8)
+        top = 8;
+    const u32* in_pos = pos;
+    const u32* in_val = buf.vals;
+    if (top > 0) {
+        const int shift = nb - top;
+        HIP_TRY(hipMemsetAsync(h->ghist, 0, RADIX_BINS * sizeof(u32), s));
+        hipLaunchKernelGGL(position_hist_kernel, dim3(hist_blocks(256 * 16, m)), dim3(256), 0, s, pos, m, shift, top, h->ghist);
+        hipLaunchKernelGGL(radix_scan_hist_kernel, dim3(1), dim3(256), 0, s, h->ghist, h->digit_base, 1);
+        OnesweepArgs a;
+        a.keys_in = pos;
+        a.vals_in = buf.vals;
+        a.keys_out = buf.t1_pos;
+        a.vals_out = buf.t1_val;
+        a.text = nullptr;
+        a.n = m;
+        a.text_n = n;
+        a.tail = 0;
+        a.word = 0;
+        a.shift = shift;
+        a.bits = top;
+        a.digit_base = h->digit_base;
+        a.lookback = h->lookback;
+        a.lookback_groups = h->lookback + h->lookback_tile_words;
+        a.epoch = next_epoch(h);
+        a.err = h->counts + 2;
+        a.xcd_chunk = h->xcd_chunk;
+        int rc = next_ticket(L, &a.ticket);
+        if (rc)
+            return rc;
+        launch_onesweep32(a, s);
+        in_pos = buf.t1_pos;
+        in_val = buf.t1_val;
+    }
+    hipLaunchKernelGGL(scatter_ranks_kernel, dim3((u32)(((u64)m + 1023) / 1024)), dim3(256), 0, s, in_pos, in_val, m, n, h->rank,
+                       h->counts + 2);
     HIP_TRY(hipGetLastError());
     return CSA_OK;
 }
 
-// Ranks the sorted list described by `ra`, reads back the survivor counts and brings rank[] up to date
-// (directly from the kernel for short lists, through the bucketed update for long ones).
-int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivors, u32* groups)
+// Ranks the sorted list described by `ra`: counts per tile, scans the counts, reads the totals back (the one
+// host round trip of the step: the next list's size decides the launches that follow), then applies them and
+// brings rank[] up to date, directly from the kernel or through one of the bucketed updates.
+int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivors, u32* groups, int* rank_update)
 {
     csa_handle* h = L.h;
-    (void)h;
-    // generation 0 ranks every suffix of the partition: on large partitions the n scattered writes go through
-    // the bucketed update instead
-    const bool defer = ra.gen0 && ra.m >= h->defer_min;
-    if (defer)
+    hipStream_t s = L.stream;
+    const u32 tiles = (u32)(((u64)ra.m + RANK_TILE - 1) / RANK_TILE);
+    ra.tile_agg = h->tile_tables;
+    ra.tile_prefix = h->tile_tables + (u64)h->rank_tiles_cap * 4;
+    ra.tile_splits = h->tile_tables + (u64)h->rank_tiles_cap * 8;
+    ra.slab_total = h->tile_tables + (u64)h->rank_tiles_cap * 9;
+    ra.slab = (tiles + RERANK_SLABS - 1) / RERANK_SLABS;
+    ra.err = h->counts + 2;
+    ra.rank_vals = nullptr;
+    const u32 slabs = (tiles + ra.slab - 1) / ra.slab;
+    hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS, false>), dim3(tiles), dim3(RANK_BLOCK), 0, s, ra);
+    hipLaunchKernelGGL(rerank_scan_kernel, dim3(slabs), dim3(1024), 0, s, ra.tile_agg, ra.tile_prefix, tiles, ra.slab,
+                       ra.slab_total, ra.tile_splits);
+    HIP_TRY(hipGetLastError());
+    u32* h_slabs = h->h_pinned + 16;
+    HIP_TRY(hipMemcpyAsync(h_slabs, ra.slab_total, slabs * 5 * sizeof(u32), hipMemcpyDeviceToHost, s));
+    int rc = read_counts(L, nullptr);
+    if (rc)
+        return rc;
+    u64 surv = 0, heads = 0, changed = 0;
+    for (u32 sl = 0; sl < slabs; ++sl) {
+        surv += h_slabs[sl * 5 + 2];
+        heads += h_slabs[sl * 5 + 3];
+        changed += h_slabs[sl * 5 + 4];
+    }
+    *survivors = (u32)surv;
+    *groups = (u32)heads;
+    // Generation 0 ranks every suffix of the partition: on large partitions the n scattered writes go through the
+    // two-pass bucketed update. Later generations write only the ranks that changed; when those are many and the
+    // partition is larger than one window, they go through the one-pass bucketed update.
+    const bool defer0 = ra.gen0 && ra.m >= h->defer_min;
+    const bool windowed = !ra.gen0 && bit_length(ra.n - 1) > WINDOW_LOG2 && changed >= h->window_min_changed &&
+                          changed >= ra.m / 2;
+    if (defer0 || windowed)
         ra.rank_vals = buf.vals;
-    int rc = launch_rerank(L, ra);
-    if (rc)
-        return rc;
-    rc = read_counts(L, survivors, groups, nullptr);
-    if (rc)
-        return rc;
-    if (defer)
+    *rank_update = defer0 ? 1 : windowed ? 2 : 0;
+    hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS, true>), dim3(tiles), dim3(RANK_BLOCK), 0, s, ra);
+    HIP_TRY(hipGetLastError());
+    if (defer0)
         return deferred_rank_update(L, ra.sufs, buf, ra.n);
+    if (windowed)
+        return windowed_rank_update(L, ra.sufs, buf, ra.m, ra.n);
     return CSA_OK;
 }
 
@@ -539,7 +608,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     const DeferBuffers defer_buf = {bx[0], bx[1], reinterpret_cast<u32*>(bkey[0]), reinterpret_cast<u32*>(bkey[1]),
                                     reinterpret_cast<u32*>(bkey[1]) + h->cap};
     u32 m = 0, groups = 0, big = 0;
-    rc = rerank_step(L, ra, defer_buf, &m, &groups);
+    rc = rerank_step(L, ra, defer_buf, &m, &groups, &st->rank_update[0]);
     if (rc)
         return rc;
     st->passes[0] = passes;
@@ -578,7 +647,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
         hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG>),
                            dim3((m + SMALL_TILE - 1) / SMALL_TILE), dim3(SMALL_BLOCK), 0, s, sa);
         HIP_TRY(hipGetLastError());
-        rc = read_counts(L, nullptr, nullptr, &big);
+        rc = read_counts(L, &big);
         if (rc)
             return rc;
         st->big[gen] = big;
@@ -627,7 +696,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
         ra.gids_out = agid;
         ra.gprim_out = h->gprim[gp ^ 1];
         ra.gstart_out = h->gstart[gp ^ 1];
-        rc = rerank_step(L, ra, defer_buf, &m, &groups);
+        rc = rerank_step(L, ra, defer_buf, &m, &groups, &st->rank_update[gen]);
         if (rc)
             return rc;
         gp ^= 1;
@@ -645,7 +714,9 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
                        aligned4);
     HIP_TRY(hipGetLastError());
     HIP_TRY(hipEventRecord(h->ev_gen[gen + 1], s));
-    HIP_TRY(hipStreamSynchronize(s));
+    rc = read_counts(L, nullptr); // waits for the stream; the last apply pass may still have raised the error word
+    if (rc)
+        return rc;
 
     for (int g = 0; g < gen; ++g)
         HIP_TRY(hipEventElapsedTime(&st->ms[g], h->ev_gen[g], h->ev_gen[g + 1]));
@@ -689,6 +760,8 @@ int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
     h->key_words = key_words;
     if (const char* e = getenv("CASCADE_DEFER_MIN"))
         h->defer_min = (u32)strtoul(e, nullptr, 10);
+    if (const char* e = getenv("CASCADE_WINDOW_MIN_CHANGED"))
+        h->window_min_changed = (u32)strtoul(e, nullptr, 10);
     const u64 cap = h->cap;
     const u64 sort_tiles = (cap + SORT_TILE - 1) / SORT_TILE;
     const u64 rank_tiles = (cap + RANK_TILE - 1) / RANK_TILE;
@@ -721,7 +794,7 @@ int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
     alloc((void**)&h->gstart[1], (cap / 2 + 2) * 4);
     alloc((void**)&h->lookback, h->lookback_words * 8);
     h->rank_tiles_cap = rank_tiles + 1;
-    alloc((void**)&h->tile_tables, (h->rank_tiles_cap * 4 * 2 + RERANK_SLABS * 4) * sizeof(u32));
+    alloc((void**)&h->tile_tables, (h->rank_tiles_cap * 9 + RERANK_SLABS * 5) * sizeof(u32));
     alloc((void**)&h->ghist, (MAX_PASSES + 2) * RADIX_BINS * 4);
     alloc((void**)&h->digit_base, MAX_PASSES * RADIX_BINS * 4);
     alloc((void**)&h->tickets, TICKET_POOL * 4);
@@ -891,7 +964,7 @@ int csa_radix_sort_pairs_dev(csa_handle* h, uint64_t* d_keys, uint32_t* d_vals, 
         HIP_TRY(hipMemcpyAsync(d_keys, h->key[0], n * 8, hipMemcpyDeviceToDevice, L.stream));
         HIP_TRY(hipMemcpyAsync(d_vals, h->idx[0], n * 4, hipMemcpyDeviceToDevice, L.stream));
     }
-    return read_counts(L, nullptr, nullptr, nullptr);
+    return read_counts(L, nullptr);
 }
 
 int csa_verify_sa40_dev(csa_handle* h, const uint16_t* d_text, uint64_t n, uint64_t index_base,

@@ -25,6 +25,8 @@ namespace csa {
 // src/GPU_SACA.cu:1253-1261,1917-1925), each with the dense id of its new group.
 // ---------------------------------------------------------------------------------------------
 
+constexpr u32 NO_RANK = 0xFFFFFFFFu; // ranks are below 2^31
+
 struct RerankArgs {
     const u64* keys;
     const u32* sufs;
@@ -38,20 +40,20 @@ struct RerankArgs {
     const u32* gprim_in; // generation t: first rank of each incoming group
     u32 groups_in;       // generation t: number of incoming groups
     u32* rank;           // [n] by text position
-    // Deferred rank update (generation 0 of large partitions): instead of the scattered write rank[x] = r,
-    // the new rank of the suffix at sorted index c is stored at rank_vals[c] (a coalesced stream; the suffix
-    // itself is sufs[c]). The (x, r) pairs then go through two radix passes on the high bits of x before they
-    // are written to rank[], so that those writes fall into one small window of rank[] at a time.
+    // Deferred rank update: instead of the scattered write rank[x] = r, the new rank of the suffix at sorted
+    // index c is stored at rank_vals[c] (a coalesced stream; the suffix itself is sufs[c]; NO_RANK where the rank
+    // did not change). The (x, r) pairs then go through one or two radix passes on the high bits of x before
+    // they are written to rank[], so that those writes fall into one window of rank[] at a time.
     u32* rank_vals; // null: write rank[x] directly
     u32* sa32;           // [n] suffix array under construction
     u32* sufs_out;       // next active list
     u32* gids_out;
     u32* gprim_out;
     u32* gstart_out; // index in the next active list where each new group starts; [groups] = survivors
-    u32* counts; // [0] = survivors, [1] = their groups (written by the last tile)
     u32* tile_agg;    // [tiles][4]: last key-run head, last group head, survivors, new groups of each tile
+    u32* tile_splits; // [tiles]: elements whose rank changes | elements that change if the tile starts inside a split group << 16
     u32* tile_prefix; // [tiles][4]: the same, combined over the earlier tiles of the tile's slab (max, max, sum, sum)
-    u32* slab_total;  // [RERANK_SLABS][4]: combination over each slab of tiles
+    u32* slab_total;  // [RERANK_SLABS][5]: combination over each slab of tiles (max, max, sum, sum; changed ranks)
     u32 slab;         // tiles per slab
     u32* err;
 };
@@ -63,6 +65,7 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
 {
     constexpr int TILE = BLOCK * ITEMS;
     constexpr int WAVES = BLOCK / WAVE;
+    static_assert(TILE < 65536, "two per-tile counts are packed into one 32-bit word");
     // The tile is read from and written to HBM in striped order (consecutive lanes, consecutive elements) and
     // exchanged through LDS with the blocked order (each thread, ITEMS consecutive elements) the scans want.
     // One pad slot per ITEMS elements keeps the blocked LDS accesses off a single bank.
@@ -132,6 +135,7 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
     }
 
     // thread-local aggregates
+    // head positions are kept 1-based (c + 1), so that 0 means "no head so far"
     u32 la = 0, lb = 0, lcnt = 0, lheads = 0;
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
@@ -141,9 +145,9 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
             const bool pb = !pq[k];
             const bool single = ka && !eq[k + 1];
             if (ka)
-                la = (u32)c;
+                la = (u32)c + 1u;
             if (pb)
-                lb = (u32)c;
+                lb = (u32)c + 1u;
             lcnt += single ? 0u : 1u;
             lheads += (ka && !single) ? 1u : 0u;
         }
@@ -174,6 +178,35 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
                 agg = t < 2 ? (agg > s_wagg[ww][t] ? agg : s_wagg[ww][t]) : agg + s_wagg[ww][t];
             a.tile_agg[(u64)tile * 4 + t] = agg;
         }
+        // Elements whose rank will change (key-run head behind the group head), for the host's choice of how to
+        // write the ranks: those the tile can tell by itself, and those before its first head, which change if
+        // the tiles before end inside a split group. Packed as changed | undecided << 16.
+        u32 ra = xa, rb = xb, lchg = 0, lund = 0;
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            const u64 c = base + k;
+            if (c < m) {
+                if (!eq[k])
+                    ra = (u32)c + 1u;
+                if (!pq[k])
+                    rb = (u32)c + 1u;
+                if (ra == 0)
+                    lund++;
+                else if (ra != rb)
+                    lchg++;
+            }
+        }
+        const u32 wpacked = wave_reduce_sum(lchg | (lund << 16)); // at most TILE <= 65535 each: no carry between the halves
+        __syncthreads(); // s_wagg has been read: reuse its first column
+        if (lane == 0)
+            s_wagg[w][0] = wpacked;
+        __syncthreads();
+        if (t == 0) {
+            u32 sp = 0;
+            for (int ww = 0; ww < WAVES; ++ww)
+                sp += s_wagg[ww][0];
+            a.tile_splits[tile] = sp;
+        }
         return;
     }
     u32 tile_total_surv = 0, tile_total_heads = 0;
@@ -185,17 +218,14 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
     u32 pre_a = a.tile_prefix[(u64)tile * 4 + 0], pre_b = a.tile_prefix[(u64)tile * 4 + 1];
     u32 tile_rc = a.tile_prefix[(u64)tile * 4 + 2], tile_rh = a.tile_prefix[(u64)tile * 4 + 3];
     for (u32 sl = 0; sl < tile / a.slab; ++sl) {
-        const u32 sa_ = a.slab_total[sl * 4 + 0], sb_ = a.slab_total[sl * 4 + 1];
+        const u32 sa_ = a.slab_total[sl * 5 + 0], sb_ = a.slab_total[sl * 5 + 1];
         pre_a = pre_a > sa_ ? pre_a : sa_;
         pre_b = pre_b > sb_ ? pre_b : sb_;
-        tile_rc += a.slab_total[sl * 4 + 2];
-        tile_rh += a.slab_total[sl * 4 + 3];
+        tile_rc += a.slab_total[sl * 5 + 2];
+        tile_rh += a.slab_total[sl * 5 + 3];
     }
-    if (t == 0 && tile_base + TILE >= m) { // the last tile knows the totals
-        a.counts[0] = tile_rc + tile_total_surv;
-        a.counts[1] = tile_rh + tile_total_heads;
+    if (t == 0 && tile_base + TILE >= m) // the last tile knows the totals
         a.gstart_out[tile_rh + tile_total_heads] = tile_rc + tile_total_surv; // gstart[groups] = survivors
-    }
     u32 ra = xa > pre_a ? xa : pre_a;
     u32 rb = xb > pre_b ? xb : pre_b;
     u32 rc = xc; // tile-local from here on
@@ -214,9 +244,9 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
             const bool pb = !pq[k];
             const bool single = ka && !eq[k + 1];
             if (ka)
-                ra = (u32)c;
+                ra = (u32)c + 1u;
             if (pb)
-                rb = (u32)c;
+                rb = (u32)c + 1u;
             const u32 x = suf[k + 1];
             u32 prim = 0;
             if (!a.gen0) {
@@ -228,9 +258,10 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
                 atomicExch(a.err, DEV_ERR_RERANK_RANGE);
                 continue;
             }
+            const bool changed = a.gen0 || ra != rb;
             if (a.rank_vals) {
-                s_rv[t * ITEMS + k] = nr;
-            } else if (a.gen0 || ra != rb) {
+                s_rv[t * ITEMS + k] = changed ? nr : NO_RANK;
+            } else if (changed) {
                 a.rank[x] = nr;
             }
             if (single) {
@@ -271,9 +302,11 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
 constexpr u32 RERANK_SLABS = 64;
 
 __global__ __launch_bounds__(1024) void rerank_scan_kernel(const u32* __restrict__ tile_agg, u32* __restrict__ tile_prefix,
-                                                           u32 tiles, u32 slab, u32* __restrict__ slab_total)
+                                                           u32 tiles, u32 slab, u32* __restrict__ slab_total,
+                                                           const u32* __restrict__ tile_splits)
 {
     __shared__ u32 s_w[16][4];
+    __shared__ u32 s_sp[16];
     const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
     const u32 slab_first = blockIdx.x * slab;
     const u32 slab_last = slab_first + slab < tiles ? slab_first + slab : tiles;
@@ -282,7 +315,7 @@ __global__ __launch_bounds__(1024) void rerank_scan_kernel(const u32* __restrict
     const u32 last = first + per < slab_last ? first + per : slab_last;
     const uint4* agg4 = reinterpret_cast<const uint4*>(tile_agg);
     uint4* pre4 = reinterpret_cast<uint4*>(tile_prefix);
-    u32 ra = 0, rb = 0, rc = 0, rh = 0;
+    u32 ra = 0, rb = 0, rc = 0, rh = 0, sp = 0;
     for (u32 i = first; i < last; ++i) {
         const uint4 v = agg4[i];
         ra = ra > v.x ? ra : v.x;
@@ -317,16 +350,28 @@ __global__ __launch_bounds__(1024) void rerank_scan_kernel(const u32* __restrict
     for (u32 i = first; i < last; ++i) {
         const uint4 v = agg4[i];
         pre4[i] = make_uint4(xa, xb, xc, xh);
+        // changed ranks of the tile; its undecided elements change if the slab so far ends inside a split group
+        // (what the slabs before left open is ignored: the sum only steers a choice between two correct paths)
+        const u32 packed = tile_splits[i];
+        sp += (packed & 0xFFFFu) + (xa > xb ? packed >> 16 : 0u);
         xa = xa > v.x ? xa : v.x;
         xb = xb > v.y ? xb : v.y;
         xc += v.z;
         xh += v.w;
     }
+    const u32 wsp = wave_reduce_sum(sp);
+    if (lane == 0)
+        s_sp[w] = wsp;
+    __syncthreads();
     if (t == 0) {
-        slab_total[blockIdx.x * 4 + 0] = ta;
-        slab_total[blockIdx.x * 4 + 1] = tb;
-        slab_total[blockIdx.x * 4 + 2] = tc;
-        slab_total[blockIdx.x * 4 + 3] = th;
+        u32 tsp = 0;
+        for (u32 ww = 0; ww < 16; ++ww)
+            tsp += s_sp[ww];
+        slab_total[blockIdx.x * 5 + 0] = ta;
+        slab_total[blockIdx.x * 5 + 1] = tb;
+        slab_total[blockIdx.x * 5 + 2] = tc;
+        slab_total[blockIdx.x * 5 + 3] = th;
+        slab_total[blockIdx.x * 5 + 4] = tsp;
     }
 }
 
@@ -351,6 +396,56 @@ __global__ __launch_bounds__(1024) void place_ranks_kernel(const u32* __restrict
     __syncthreads();
     for (u32 i = threadIdx.x; i < count; i += 1024)
         rank[first + i] = s_win[i];
+}
+
+// Bucketed rank update of a later generation. The changed ranks of a generation are few or many: when they are
+// many, the (text position, rank) pairs of the whole sorted list go through ONE radix pass on the position bits
+// above the window size, after which consecutive workgroups scatter into one window of rank[] at a time. Random
+// 4-byte writes into a window that the last-level cache holds (here 128 MB) run about four times faster than
+// writes spread over a multi-GB array.
+constexpr int POS_BINS = 256; // digits of the one bucket pass are at most 8 bits wide
+
+__global__ __launch_bounds__(256) void position_hist_kernel(const u32* __restrict__ pos, u32 m, int shift, int bits,
+                                                            u32* ghist)
+{
+    __shared__ u32 s_hist[POS_BINS * 8];
+    for (int i = threadIdx.x; i < POS_BINS * 8; i += 256)
+        s_hist[i] = 0;
+    __syncthreads();
+    const u32 copy = threadIdx.x & 7u;
+    const u32 mask = (1u << bits) - 1u;
+    const u64 stride = (u64)gridDim.x * 256;
+    for (u64 i = (u64)blockIdx.x * 256 + threadIdx.x; i < m; i += stride)
+        atomicAdd(&s_hist[((pos[i] >> shift) & mask) * 8 + copy], 1u);
+    __syncthreads();
+    for (int i = threadIdx.x; i < POS_BINS; i += 256) {
+        u32 v = 0;
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+            v += s_hist[i * 8 + c];
+        if (v)
+            atomicAdd(&ghist[i], v);
+    }
+}
+
+__global__ __launch_bounds__(256) void scatter_ranks_kernel(const u32* __restrict__ pos, const u32* __restrict__ val, u32 m,
+                                                            u32 n, u32* __restrict__ rank, u32* err)
+{
+    const u64 i0 = ((u64)blockIdx.x * 256 + threadIdx.x) * 4;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const u64 i = i0 + k;
+        if (i < m) {
+            const u32 v = val[i];
+            if (v != NO_RANK) {
+                const u32 x = pos[i];
+                if (x < n && v < n)
+                    rank[x] = v;
+                else
+                    atomicExch(err, DEV_ERR_RERANK_RANGE);
+            }
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------------------------

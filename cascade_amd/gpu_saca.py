@@ -24,6 +24,7 @@ def stats_to_dict(st):
         "groups": [int(st.groups[i]) for i in range(g)],
         "big": [int(st.big[i]) for i in range(g)],
         "passes": [int(st.passes[i]) for i in range(g)],
+        "rank_update": [int(st.rank_update[i]) for i in range(g)],
         "ms": [float(st.ms[i]) for i in range(g)],
         "ms_output": float(st.ms_output),
         "ms_total": float(st.ms_total),

@@ -46,6 +46,9 @@ typedef struct csa_stats {
     uint64_t groups[CSA_MAX_GENERATIONS]; /* unresolved groups entering generation g (0 for g = 0) */
     uint64_t big[CSA_MAX_GENERATIONS];    /* of active[g], members of groups too large for the in-tile sort */
     int32_t passes[CSA_MAX_GENERATIONS];  /* radix passes run in generation g (over the large groups for g > 0) */
+    int32_t rank_update[CSA_MAX_GENERATIONS]; /* how generation g wrote its ranks: 0 scattered from the rank pass,
+                                                 1 bucketed by two passes into LDS-sized windows (generation 0),
+                                                 2 bucketed by one pass into cache-sized windows */
     float ms[CSA_MAX_GENERATIONS];        /* device time of generation g */
     float ms_output;                      /* sa40 emission */
     float ms_total;                       /* first kernel to last kernel, on the stream */

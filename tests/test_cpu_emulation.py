@@ -40,6 +40,7 @@ def emu_sort(lib, T, key_words):
     rc = lib.csa_sort_partition_u16_dev(h, T.ctypes.data, n, 0, out.ctypes.data, None, 0, C.byref(st))
     lib.csa_destroy(h)
     assert rc == 0, lib.csa_last_error()
+    emu_sort.rank_update = [int(st.rank_update[i]) for i in range(st.generations)]
     return out[:5 * n], [int(st.active[i]) for i in range(st.generations)], [int(st.big[i]) for i in range(st.generations)]
 
 
@@ -80,6 +81,9 @@ def test_small_and_large_groups_take_both_paths(emu):
     got, active, big = emu_sort(emu, T, 1)
     assert np.array_equal(got, oracle_lib.build_sa40(T))
     assert big[1] > 0 and any(b == 0 and a > 0 for a, b in zip(active[2:], big[2:]))
+    # generation 0 takes the two-pass bucketed rank update here and later ones the one-pass kind (the emulation
+    # library is built with tiny thresholds for both); the short fixtures above write their ranks directly
+    assert emu_sort.rank_update[0] == 1 and 2 in emu_sort.rank_update[1:]
 
 
 def test_emulated_radix_sort_matches_stable_sort(emu):
