@@ -53,7 +53,7 @@ static_assert(SORT32_ITEMS >= SORT_ITEMS, "the look-back words are sized for til
 #define CSA_RANK_BLOCK 256
 #endif
 #ifndef CSA_RANK_ITEMS
-#define CSA_RANK_ITEMS 8
+#define CSA_RANK_ITEMS 4
 #endif
 constexpr int RANK_BLOCK = CSA_RANK_BLOCK;
 constexpr int RANK_ITEMS = CSA_RANK_ITEMS;
@@ -62,8 +62,14 @@ constexpr int RANK_TILE = RANK_BLOCK * RANK_ITEMS;
 #ifndef CSA_SMALL_MAXG
 #define CSA_SMALL_MAXG 64
 #endif
-constexpr int SMALL_BLOCK = 256;
-constexpr int SMALL_ITEMS = 8;
+#ifndef CSA_SMALL_BLOCK
+#define CSA_SMALL_BLOCK 256
+#endif
+#ifndef CSA_SMALL_ITEMS
+#define CSA_SMALL_ITEMS 8
+#endif
+constexpr int SMALL_BLOCK = CSA_SMALL_BLOCK;
+constexpr int SMALL_ITEMS = CSA_SMALL_ITEMS;
 constexpr int SMALL_TILE = SMALL_BLOCK * SMALL_ITEMS;
 constexpr int SMALL_MAXG = CSA_SMALL_MAXG;
 constexpr u32 TICKET_POOL = 4096;
