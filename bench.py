@@ -67,6 +67,64 @@ def cpu_baseline(config, sample_n):
     }
 
 
+def bench_partition_ids(args):
+    """The step before the partition sort: partition id of every suffix of the workload's text against p - 1 pivots
+    (packed map + partition sizes out). One step = one pass over the text resident in HBM."""
+    import numpy as np
+    import torch
+    import oracle_lib
+    from cascade_amd import _native, partition_ids, workloads
+    dev = torch.device("cuda:0")
+    n = args.n if args.n is not None else workloads.default_n(args.config)
+    p, words = args.partitions, 2  # the reference's default pivot width: 2 words = 8 symbols (include/Packed_Prefix.hpp:30-34)
+    T = workloads.generate(args.config, n)
+    rng = np.random.default_rng(1)
+    pivots = oracle_lib.sample_pivots(T[:1 << 22], p, words, rng)
+    d_text = torch.from_numpy(T.view(np.int16)).to(dev)
+    d_piv = torch.from_numpy(pivots.view(np.int64)).to(dev).reshape(-1, words)
+    bits = int(_native.load().csa_partition_id_bits(p))
+    for _ in range(args.warmup):
+        partition_ids(d_text, d_piv, p, want_ids=False)
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    t0 = time.perf_counter()
+    ev[0].record()
+    for _ in range(args.steps):
+        _, packed, sizes = partition_ids(d_text, d_piv, p, want_ids=False)
+    ev[1].record()
+    torch.cuda.synchronize()
+    ms = 1e3 * (time.perf_counter() - t0) / args.steps
+    kernel_ms = ev[0].elapsed_time(ev[1]) / args.steps  # includes the zero fill of the outputs made by the wrapper
+    alg_bytes = n * (2 + bits / 8.0)  # symbols in, packed entries out
+    sample = min(n, 1 << 22)
+    want_ids, _ = oracle_lib.partition_ids(T[:sample], pivots, p, words, text_len=sample)
+    got = packed.cpu().numpy().view(np.uint64)
+    ok = bool(np.array_equal(got[:oracle_lib.packed_words(sample - sample % 64, bits)],
+                             oracle_lib.pack_partition_ids(want_ids[:sample - sample % 64], bits)[:oracle_lib.packed_words(sample - sample % 64, bits)]))
+    ok = ok and int(sizes.sum().item()) == n
+    t1 = time.perf_counter()
+    cs = min(n, max(args.cpu_sample, 1) // 4) if args.cpu_sample else 0
+    result = {
+        "metric": "suffixes assigned to partitions/sec at 1 GPU", "value": n / (ms * 1e-3), "unit": "suffixes/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u64 keys", "data": "synthetic",
+        "config": {"workload": workloads.NAMES[args.config], "n": n, "partitions": p, "pivot_words": words,
+                   "checked_against_oracle": ok},
+        "roofline": {"bound": "hbm", "kernel": "partition_ids_kernel<2>", "achieved": round(alg_bytes / (kernel_ms * 1e-3) / 1e9, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(alg_bytes / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "traffic": None, "avg_launch_ms": round(kernel_ms, 4), "algorithmic_bytes_per_launch": round(alg_bytes)},
+    }
+    if cs:
+        t1 = time.perf_counter()
+        oracle_lib.partition_ids(T[:cs], pivots, p, words, text_len=cs)
+        dt = time.perf_counter() - t1
+        result["cpu_baseline"] = {"value": cs / dt, "unit": "suffixes/s", "cores": 1, "kind": "port",
+                                  "sample": f"first {cs} symbols of the same text, C restatement of the reference's validator loop, {dt:.1f} s"}
+    print(json.dumps(result), flush=True)
+    if not ok:
+        sys.exit(1)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -78,6 +136,9 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=1 << 26, help="symbols of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--generations", action="store_true", help="print the per-generation table to stderr")
+    ap.add_argument("--row", default="sort", choices=["sort", "partition_ids"],
+                    help="which step to measure: the partition sort (the headline) or the partition-id step before it")
+    ap.add_argument("--partitions", type=int, default=256, help="partitions of --row partition_ids")
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -90,6 +151,8 @@ def main():
     from cascade_amd import PartitionSorter, _native, workloads
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.row == "partition_ids":
+        return bench_partition_ids(args)
     dev = torch.device("cuda:0")
     n = args.n if args.n is not None else workloads.default_n(args.config)
 

@@ -18,6 +18,7 @@ CSA_FLAG_KERNEL_TIMING = 1
 EXPORTS = (
     "csa_bytes_per_suffix", "csa_create", "csa_destroy", "csa_sort_partition_u16_dev", "csa_sort_partition_u16",
     "csa_pack_keys_u16_dev", "csa_radix_sort_pairs_dev", "csa_verify_sa40_dev", "csa_last_error",
+    "csa_partition_id_bits", "csa_partition_ids_u16_dev",
 )
 
 
@@ -79,6 +80,10 @@ def load():
     lib.csa_verify_sa40_dev.argtypes = [vp, vp, u64, u64, vp, vp, C.POINTER(i32)]
     lib.csa_last_error.restype = C.c_char_p
     lib.csa_last_error.argtypes = []
+    lib.csa_partition_id_bits.restype = u32
+    lib.csa_partition_id_bits.argtypes = [u32]
+    lib.csa_partition_ids_u16_dev.restype = i32
+    lib.csa_partition_ids_u16_dev.argtypes = [vp, u64, u64, vp, i32, u32, vp, vp, vp, vp]
     _lib = lib
     return lib
 

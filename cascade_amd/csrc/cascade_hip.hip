@@ -4,6 +4,7 @@
 
 #include "device_utils.hpp"
 #include "doubling.hpp"
+#include "partition_ids.hpp"
 #include "radix_sort.hpp"
 
 #include <cstdarg>
@@ -741,6 +742,59 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
 } // namespace
 
 extern "C" {
+
+uint32_t csa_partition_id_bits(uint32_t p)
+{
+    const int id_bits = p <= 1 ? 0 : bit_length((u64)p - 1);
+    return (u32)(id_bits < 1 ? 1 : id_bits) + 1u;
+}
+
+int csa_partition_ids_u16_dev(const uint16_t* d_text, uint64_t n, uint64_t text_len, const uint64_t* d_pivots,
+                              int pivot_words, uint32_t p, uint16_t* d_pid, uint64_t* d_packed, uint64_t* d_psz,
+                              void* stream)
+{
+    if (p < 1 || p > 65536u)
+        return fail(CSA_ERR_ARG, "csa_partition_ids_u16_dev: p = %u is outside [1, 65536]", p);
+    if (pivot_words < 1 || pivot_words > 4)
+        return fail(CSA_ERR_ARG, "csa_partition_ids_u16_dev: pivot_words = %d is outside [1, 4]", pivot_words);
+    if (n == 0)
+        return CSA_OK;
+    if (!d_text || (p > 1 && !d_pivots) || text_len < n)
+        return fail(CSA_ERR_ARG, "csa_partition_ids_u16_dev: null text or pivots, or text_len < n");
+    const u64 tiles64 = (n + PID_TILE - 1) / PID_TILE;
+    if (tiles64 > 0xFFFFFFFFull)
+        return fail(CSA_ERR_TOO_LARGE, "csa_partition_ids_u16_dev: %llu suffixes in one call", (unsigned long long)n);
+    PartitionIdArgs a;
+    a.text = d_text;
+    a.n = n;
+    a.text_len = text_len;
+    a.pivots = d_pivots;
+    a.p = p;
+    a.bits = csa_partition_id_bits(p);
+    a.pid = d_pid;
+    a.packed = d_packed;
+    a.psz = reinterpret_cast<unsigned long long*>(d_psz);
+    a.tiles = (u32)tiles64;
+    const u32 grid = a.tiles < 2048u ? a.tiles : 2048u;
+    hipStream_t s = (hipStream_t)stream;
+    const bool piv_lds = (u64)(p - 1) * (u64)pivot_words <= PID_LDS_PIVOT_WORDS;
+#define CSA_LAUNCH_PID(W)                                                                                  \
+    do {                                                                                                   \
+        if (piv_lds)                                                                                       \
+            hipLaunchKernelGGL((partition_ids_kernel<W, true>), dim3(grid), dim3(PID_BLOCK), 0, s, a);    \
+        else                                                                                               \
+            hipLaunchKernelGGL((partition_ids_kernel<W, false>), dim3(grid), dim3(PID_BLOCK), 0, s, a);   \
+    } while (0)
+    switch (pivot_words) {
+    case 1: CSA_LAUNCH_PID(1); break;
+    case 2: CSA_LAUNCH_PID(2); break;
+    case 3: CSA_LAUNCH_PID(3); break;
+    default: CSA_LAUNCH_PID(4); break;
+    }
+#undef CSA_LAUNCH_PID
+    HIP_TRY(hipGetLastError());
+    return CSA_OK;
+}
 
 const char* csa_last_error(void) { return g_err; }
 

@@ -335,4 +335,45 @@ __device__ __forceinline__ u64 load_kgram(const u16* __restrict__ T, u32 n, u32 
     return k;
 }
 
+// ---- a stretch of the text in LDS ----
+//
+// Consecutive suffixes share all but one symbol of their K-grams, and the text is only 2-byte aligned, so kernels
+// that build the keys of a run of consecutive positions stage the stretch once: symbols [p0, p0 + count) of the text
+// (zero past its end, the key padding) are copied into s_words with aligned 8-byte loads by the `block` threads of the
+// workgroup. Returns sym_off: after a __syncthreads(), symbol p0 + i is 16-bit element sym_off + i of s_words.
+// s_words needs room for (count + 6) / 4 + 1 words.
+__device__ __forceinline__ u32 stage_text(const u16* __restrict__ text, u64 text_len, u64 p0, u32 count, u64* s_words, u32 t,
+                                          u32 block)
+{
+    const u32 sym_off = (u32)(((uintptr_t)(text + p0) & 7u) >> 1); // symbols between the aligned word boundary and p0
+    const long long first_pos = (long long)p0 - (long long)sym_off;
+    const u32 nw = (sym_off + count + 3u) / 4u;
+    for (u32 i = t; i < nw; i += block) {
+        const long long q0 = first_pos + 4ll * i;
+        u64 wv = 0;
+        if (q0 >= 0 && q0 + 4 <= (long long)text_len) {
+            wv = *reinterpret_cast<const u64*>(text + q0); // 8-byte aligned by construction, wholly inside the text
+        } else {
+#pragma unroll
+            for (int sy = 0; sy < 4; ++sy) {
+                const long long q = q0 + sy;
+                if (q >= 0 && q < (long long)text_len)
+                    wv |= (u64)text[q] << (16 * sy);
+            }
+        }
+        s_words[i] = wv;
+    }
+    return sym_off;
+}
+
+// K-gram word (four symbols, the first most significant) that starts at 16-bit element sidx of a staged stretch.
+// Reads three 32-bit LDS words; the stretch must extend one word past the last symbol used.
+__device__ __forceinline__ u64 staged_kgram(const u32* s_dw, u32 sidx)
+{
+    const u32 dw = sidx >> 1;
+    const u64 lo = (u64)s_dw[dw] | ((u64)s_dw[dw + 1] << 32);
+    const u64 raw = (sidx & 1u) ? (lo >> 16) | ((u64)s_dw[dw + 2] << 48) : lo; // s0 | s1 << 16 | s2 << 32 | s3 << 48
+    return (raw << 48) | ((raw & 0xFFFF0000ull) << 16) | ((raw >> 16) & 0xFFFF0000ull) | (raw >> 48);
+}
+
 } // namespace csa

@@ -1,0 +1,157 @@
+// Partition ids of the suffixes of a text against sorted pivots, their bit-packed map and the partition sizes, in
+// one pass over the text. The reference does this with two kernels and one global atomic per suffix
+// (include/GPU_SACA.cuh:23-74 compute_partition_IDs_kernel, :82-91 pack_partition_IDs_kernel; host loop
+// src/GPU_SACA.cu:854-1000); the packed layout is that of include/Partition_ID_Map.hpp:158-177.
+#pragma once
+
+#include "device_utils.hpp"
+
+namespace csa {
+
+struct PartitionIdArgs {
+    const u16* text;
+    u64 n;        // suffixes: text positions [0, n)
+    u64 text_len; // symbols readable at `text` (>= n); the text reads as zero beyond them
+    const u64* pivots; // [p - 1][W] packed K-grams, first symbols most significant, ascending; inclusive upper bounds
+    u32 p;        // partitions
+    u32 bits;     // bits per entry of the packed map (the id, then a clear retirement flag)
+    u16* pid;     // [n] partition id of every suffix, or null
+    u64* packed;  // the packed map (`bits` words per 64 suffixes), or null
+    unsigned long long* psz; // [p] partition sizes, added to; or null
+    u32 tiles;
+};
+
+constexpr int PID_BLOCK = 256;
+constexpr int PID_ITEMS = 8; // groups of 64 suffixes per wave and tile
+constexpr int PID_TILE = PID_BLOCK * PID_ITEMS;
+constexpr u32 PID_LDS_PIVOT_WORDS = 4096; // pivots are searched in LDS when they fit
+constexpr u32 PID_LDS_BINS = 4096;        // partition sizes are counted in LDS when they fit
+
+// W: 64-bit words per pivot (the reference's K_WORDS, include/Packed_Prefix.hpp:26-34). PIV_LDS: the pivots fit in LDS.
+// A wave handles 64 consecutive suffixes at a time: exactly one group of the packed map, whose `bits` words the
+// wave assembles with one shuffle and one ballot per word. The searches of a thread's PID_ITEMS suffixes advance
+// together, one pivot probe each per step, so that their LDS (or cache) latencies overlap. Workgroups stride over
+// the tiles so that the LDS histogram is flushed once per workgroup, not once per tile; it is replicated so that
+// the lanes of a wave that meet in one hot partition spread over several counters.
+template <int W, bool PIV_LDS>
+__global__ __launch_bounds__(PID_BLOCK) void partition_ids_kernel(PartitionIdArgs a)
+{
+    __shared__ u64 s_text[(PID_TILE + 4 * W + 6) / 4 + 2];
+    __shared__ u64 s_piv[PIV_LDS ? PID_LDS_PIVOT_WORDS : 1];
+    __shared__ u32 s_hist[PID_LDS_BINS];
+    const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
+    const u32 np = a.p - 1u; // pivots
+    const bool hist_lds = a.psz != nullptr && a.p <= PID_LDS_BINS;
+    u32 copies_log2 = 0; // counters per partition in the LDS histogram
+    while (copies_log2 < 4 && (a.p << (copies_log2 + 1)) <= PID_LDS_BINS)
+        ++copies_log2;
+    if (PIV_LDS)
+        for (u32 i = t; i < np * (u32)W; i += PID_BLOCK)
+            s_piv[i] = a.pivots[i];
+    if (hist_lds)
+        for (u32 i = t; i < (a.p << copies_log2); i += PID_BLOCK)
+            s_hist[i] = 0;
+    int steps = 0; // bits of the pivot count: probes per search
+    while ((np >> steps) != 0)
+        ++steps;
+    // entry and bit inside the entry that this lane contributes to word 0 of a group; +64 bits per further word
+    const u32 ent0 = lane / a.bits, sh0 = lane % a.bits;
+    const u32 dq = 64u / a.bits, dr = 64u % a.bits;
+    __syncthreads();
+
+    for (u32 tile = blockIdx.x; tile < a.tiles; tile += gridDim.x) {
+        const u64 tile_base = (u64)tile * PID_TILE;
+        const u32 count = (u32)(a.n - tile_base < (u64)PID_TILE ? a.n - tile_base : (u64)PID_TILE);
+        const u32 sym_off = stage_text(a.text, a.text_len, tile_base, count + 4u * W - 1u, s_text, t, PID_BLOCK);
+        __syncthreads();
+        const u32* s_dw = reinterpret_cast<const u32*>(s_text);
+
+        // keys of this thread's suffixes (zero for lanes past the end: never used)
+        u64 key[PID_ITEMS][W];
+        u32 id[PID_ITEMS];
+#pragma unroll
+        for (int k = 0; k < PID_ITEMS; ++k) {
+            const u32 local = (w * PID_ITEMS + (u32)k) * 64u + lane;
+            id[k] = 0;
+#pragma unroll
+            for (int j = 0; j < W; ++j)
+                key[k][j] = local < count ? staged_kgram(s_dw, sym_off + local + 4u * j) : 0ull;
+        }
+        // id = number of pivots below the key = the smallest id with key <= pivots[id], p - 1 if there is none
+        // (test/partitioning.cpp:21-31), found by fixing the bits of the answer from the top
+        for (int b = steps - 1; b >= 0; --b) {
+#pragma unroll
+            for (int k = 0; k < PID_ITEMS; ++k) {
+                const u32 cand = id[k] + (1u << b);
+                if (cand <= np) {
+                    const u64* pv = (PIV_LDS ? s_piv : a.pivots) + (u64)(cand - 1u) * W;
+                    bool below = false; // pivot < key
+#pragma unroll
+                    for (int j = 0; j < W; ++j) {
+                        const u64 x = pv[j];
+                        if (x != key[k][j]) {
+                            below = x < key[k][j];
+                            break;
+                        }
+                    }
+                    if (below)
+                        id[k] = cand;
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < PID_ITEMS; ++k) {
+            const u32 group_local = (w * PID_ITEMS + (u32)k) * 64u; // wave-uniform
+            if (group_local >= count)
+                break;
+            const u32 local = group_local + lane;
+            if (local < count) {
+                if (a.pid)
+                    a.pid[tile_base + local] = (u16)id[k];
+                if (a.psz) {
+                    if (hist_lds)
+                        atomicAdd(&s_hist[(id[k] << copies_log2) + (lane & ((1u << copies_log2) - 1u))], 1u);
+                    else
+                        atomicAdd(&a.psz[id[k]], 1ull);
+                }
+            } else {
+                id[k] = 0;
+            }
+            if (a.packed) {
+                // Entries fill the words least significant bits first (include/Partition_ID_Map.hpp:158-177): bit b of
+                // word ww of the group is bit (64 ww + b) % bits of entry (64 ww + b) / bits. Lanes past the end of
+                // the text hold id 0, which is what the reference's partial last word carries there.
+                u32 ent = ent0, sh = sh0;
+                u64 mine = 0;
+                for (u32 ww = 0; ww < a.bits; ++ww) {
+                    const u32 v = __shfl(id[k], ent & 63u);
+                    const u64 m = __ballot(((v >> sh) & 1u) != 0);
+                    if (lane == ww)
+                        mine = m;
+                    ent += dq;
+                    sh += dr;
+                    if (sh >= a.bits) {
+                        sh -= a.bits;
+                        ent++;
+                    }
+                }
+                const u32 sz = count - group_local < 64u ? count - group_local : 64u;
+                const u32 nwords = (sz * a.bits + 63u) / 64u; // the reference writes no more for a partial last group
+                if (lane < nwords)
+                    a.packed[((tile_base + group_local) / 64u) * a.bits + lane] = mine;
+            }
+        }
+        __syncthreads(); // the staged text is replaced in the next round
+    }
+    if (hist_lds) {
+        for (u32 i = t; i < a.p; i += PID_BLOCK) {
+            u32 v = 0;
+            for (u32 c = 0; c < (1u << copies_log2); ++c)
+                v += s_hist[(i << copies_log2) + c];
+            if (v)
+                atomicAdd(&a.psz[i], (unsigned long long)v);
+        }
+    }
+}
+
+} // namespace csa

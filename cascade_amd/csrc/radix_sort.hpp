@@ -259,46 +259,21 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
 #endif
     // ---- first pass of generation 0: stage the tile's stretch of the text in LDS ----
     // The tile covers consecutive virtual positions, i.e. (after the few tail suffixes of tile 0) consecutive text
-    // positions j0, j0 + 1, ...; their keys overlap in three of four symbols. The stretch is read once with aligned
-    // 8-byte loads into the (still unused) reorder buffer, and each key is assembled from three LDS words; per-key
-    // loads from the text would be 2-byte aligned, four narrow global loads per key.
+    // positions j0, j0 + 1, ...; the (still unused) reorder buffer holds the stretch, and each key is assembled
+    // from three LDS words instead of four narrow global loads.
     u32 j0 = 0, sym_off = 0;
     if constexpr (SRC == SRC_TEXT) {
         const u32 first_virtual = (u32)base > a.tail ? (u32)base : a.tail;
         j0 = first_virtual - a.tail;
-        const u64 p0 = (u64)j0 + 4ull * a.word; // first text position staged
-        sym_off = (u32)(((uintptr_t)(a.text + p0) & 7u) >> 1); // symbols between the aligned word boundary and p0
-        const long long first_pos = (long long)p0 - (long long)sym_off;
-        const u32 count = (u32)TILE - (first_virtual - (u32)base);
-        const u32 nw = (sym_off + count + 3u + 3u) / 4u; // 64-bit words that cover symbols [p0 - sym_off, p0 + count + 3)
-        u64* s_words = reinterpret_cast<u64*>(s_keys);
-        static_assert(sizeof(KeyT) * TILE >= 8 * ((3 + TILE + 3 + 3) / 4 + 1), "the staged text must fit the reorder buffer");
-        for (u32 i = t; i < nw; i += BLOCK) {
-            const long long q0 = first_pos + 4ll * i;
-            u64 wv = 0;
-            if (q0 >= 0 && q0 + 4 <= (long long)a.text_n) {
-                wv = *reinterpret_cast<const u64*>(a.text + q0); // 8-byte aligned by construction, wholly inside the text
-            } else {
-#pragma unroll
-                for (int sy = 0; sy < 4; ++sy) {
-                    const long long q = q0 + sy;
-                    if (q >= 0 && q < (long long)a.text_n)
-                        wv |= (u64)a.text[q] << (16 * sy); // symbols past the end stay zero: the key padding
-                }
-            }
-            s_words[i] = wv;
-        }
+        const u32 count = (u32)TILE - (first_virtual - (u32)base) + 3u; // the last key reaches 3 symbols further
+        static_assert(sizeof(KeyT) * TILE >= 8 * ((TILE + 3 + 6) / 4 + 2), "the staged text must fit the reorder buffer");
+        sym_off = stage_text(a.text, a.text_n, (u64)j0 + 4ull * a.word, count, reinterpret_cast<u64*>(s_keys), t, BLOCK);
         __syncthreads();
     }
     auto text_key = [&](u32 i) -> u64 { // key of virtual position i of this tile (SRC_TEXT)
         if (i < a.tail)
             return load_kgram(a.text, a.text_n, a.text_n - 1u - i, a.word);
-        const u32* s_dw = reinterpret_cast<const u32*>(s_keys);
-        const u32 sidx = (i - a.tail) - j0 + sym_off; // symbol index in the staged stretch
-        const u32 dw = sidx >> 1;
-        const u64 lo = (u64)s_dw[dw] | ((u64)s_dw[dw + 1] << 32);
-        const u64 raw = (sidx & 1u) ? (lo >> 16) | ((u64)s_dw[dw + 2] << 48) : lo; // s0 | s1 << 16 | s2 << 32 | s3 << 48
-        return (raw << 48) | ((raw & 0xFFFF0000ull) << 16) | ((raw >> 16) & 0xFFFF0000ull) | (raw >> 48);
+        return staged_kgram(reinterpret_cast<const u32*>(s_keys), (i - a.tail) - j0 + sym_off);
     };
 
     // ---- load: wave-striped, so that consecutive lanes read consecutive pairs ----

@@ -116,6 +116,34 @@ def pack_keys(text, key_words=1):
     return keys
 
 
+def partition_ids(text, pivots, p, n=None, text_len=None, want_ids=True, want_packed=True, want_sizes=True, sizes=None):
+    """Partition id of every suffix against sorted pivots (csa_partition_ids_u16_dev; the reference's
+    GPU_SACA::compute_partition_IDs, src/GPU_SACA.cu:854-1000, for a text chunk resident in HBM).
+    text: uint16 device tensor; pivots: (p - 1, pivot_words) int64/uint64 device tensor, ascending.
+    Returns (ids int16 tensor or None, packed int64 tensor or None, sizes int64 tensor or None); `sizes` is added to
+    when given (chunked use)."""
+    import torch
+    lib = _native.load()
+    assert text.is_cuda and text.element_size() == 2 and text.is_contiguous()
+    n = text.numel() if n is None else int(n)
+    text_len = text.numel() if text_len is None else int(text_len)
+    assert pivots.dim() == 2, "pivots: one row of pivot_words 64-bit words per pivot"
+    words = int(pivots.shape[1])
+    assert pivots.element_size() == 8 and pivots.is_contiguous() and pivots.numel() == (p - 1) * words
+    bits = int(lib.csa_partition_id_bits(p))
+    dev = text.device
+    ids = torch.empty(max(n, 1), dtype=torch.int16, device=dev) if want_ids else None
+    packed = torch.zeros(((n + 63) // 64) * bits + 1, dtype=torch.int64, device=dev) if want_packed else None
+    if want_sizes and sizes is None:
+        sizes = torch.zeros(p, dtype=torch.int64, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    _native.check(lib.csa_partition_ids_u16_dev(text.data_ptr(), n, text_len, pivots.data_ptr() if pivots.numel() else None,
+                                                words, int(p), ids.data_ptr() if want_ids else None,
+                                                packed.data_ptr() if want_packed else None,
+                                                sizes.data_ptr() if sizes is not None else None, stream or None))
+    return (ids[:n] if want_ids else None), packed, sizes
+
+
 def sort_partition(text, key_words=1):
     """Host arrays in and out: uint16 numpy text -> uint8 numpy sa40 of 5*n bytes, plus statistics
     (csa_sort_partition_u16: device memory is allocated and released inside the call)."""

@@ -108,6 +108,30 @@ int csa_radix_sort_pairs_dev(csa_handle* h, uint64_t* d_keys, uint32_t* d_vals, 
 int csa_verify_sa40_dev(csa_handle* h, const uint16_t* d_text, uint64_t n, uint64_t index_base,
                         const uint8_t* d_sa40, void* stream, int* ok);
 
+/* ---- the step before the partition sort: which partition does every suffix belong to ---- */
+
+/* Bits per entry of the packed partition-id map for p partitions: the id's bits, then one retirement flag
+ * (reference: Partition_ID_Map::bits_for, include/Partition_ID_Map.hpp:79). */
+uint32_t csa_partition_id_bits(uint32_t p);
+
+/* For every suffix i in [0, n) of d_text: id(i) = the smallest q with K-gram(i) <= pivot[q], or p - 1 if there is
+ * none, where K-gram(i) is the first 4 * pivot_words symbols of the suffix, zero padded past d_text[text_len).
+ * d_pivots: (p - 1) * pivot_words 64-bit words, most significant symbols first, ascending (the reference's Pivot_Key,
+ * include/Packed_Prefix.hpp:26-34,88); pivot_words 1..4; p <= 65536.
+ * Any of the three outputs may be NULL:
+ *   d_pid    : n uint16 ids;
+ *   d_packed : the ids bit-packed like Partition_ID_Map::pack (include/Partition_ID_Map.hpp:158-177),
+ *              csa_partition_id_bits(p) words per 64 suffixes, ceil(n * bits / 64) words for a trailing partial group;
+ *   d_psz    : p counters to which the partition sizes are ADDED (zero them before the first chunk of a text).
+ * A chunk in the middle of a text passes text_len = n + 4 * pivot_words - 1 so that its last suffixes see the
+ * symbols that follow; n must then be a multiple of 64.
+ * Replaces compute_partition_IDs_kernel + pack_partition_IDs_kernel (include/GPU_SACA.cuh:23-91) as launched per
+ * chunk by GPU_SACA::compute_partition_IDs (src/GPU_SACA.cu:854-1000); same answers as
+ * test::validate_partition_IDs (test/partitioning.cpp:12-39). */
+int csa_partition_ids_u16_dev(const uint16_t* d_text, uint64_t n, uint64_t text_len, const uint64_t* d_pivots,
+                              int pivot_words, uint32_t p, uint16_t* d_pid, uint64_t* d_packed, uint64_t* d_psz,
+                              void* stream);
+
 /* Message of the calling thread's last failed call ("" if none). */
 const char* csa_last_error(void);
 

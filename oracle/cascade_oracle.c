@@ -367,3 +367,76 @@ void orc_stable_sort_pairs_u64_u32(uint64_t* keys, uint32_t* vals, uint64_t n, i
     }
     free(k2), free(v2);
 }
+
+/* ---------- partition ids ---------- */
+
+uint32_t orc_partition_id_bits(uint32_t p)
+{
+    /* util::math::bits_for(x) = ceil(log2 x), 0 for x <= 1 (include/utility.hpp:118-121) */
+    uint32_t id_bits = 0;
+    while (id_bits < 32 && ((uint64_t)1 << id_bits) < (uint64_t)p)
+        ++id_bits;
+    return (id_bits < 1 ? 1 : id_bits) + 1; /* max(1, bits) + the retirement flag: include/Partition_ID_Map.hpp:79 */
+}
+
+/* include/Packed_Prefix.hpp:122-135: a <= b, most significant word first */
+static int prefix_le(const uint64_t* a, const uint64_t* b, int words)
+{
+    for (int w = 0; w < words; ++w)
+        if (a[w] != b[w])
+            return a[w] < b[w];
+    return 1;
+}
+
+void orc_partition_ids_u16(const uint16_t* T, uint64_t n, uint64_t text_len, const uint64_t* pivots, int words, uint32_t p,
+                           uint16_t* pid, uint64_t* psz)
+{
+    uint64_t key[64];
+    for (uint64_t i = 0; i < n; ++i) {
+        orc_pack_prefix_u16(T, text_len, i, words, key);
+        /* test/partitioning.cpp:21-31 */
+        uint32_t low = 0, high = p - 1;
+        while (low < high) {
+            const uint32_t mid = low + (high - low) / 2;
+            if (prefix_le(key, pivots + (uint64_t)mid * words, words))
+                high = mid;
+            else
+                low = mid + 1;
+        }
+        pid[i] = (uint16_t)low;
+        if (psz)
+            psz[low]++;
+    }
+}
+
+void orc_pack_partition_ids(const uint16_t* pid, uint64_t n, uint32_t bits, uint64_t* out)
+{
+    for (uint64_t off = 0; off < n; off += 64) { /* one "thread" per group: include/GPU_SACA.cuh:86-90 */
+        const uint64_t sz = n - off < 64 ? n - off : 64;
+        uint64_t* dst = out + (off / 64) * bits;
+        /* include/Partition_ID_Map.hpp:160-176 */
+        uint64_t acc = 0;
+        uint32_t fill = 0;
+        for (uint64_t i = 0; i < sz; ++i) {
+            const uint64_t id = pid[off + i];
+            acc |= id << fill;
+            fill += bits;
+            if (fill >= 64) {
+                *dst++ = acc;
+                fill -= 64;
+                acc = fill > 0 ? id >> (bits - fill) : 0;
+            }
+        }
+        if (fill > 0)
+            *dst = acc;
+    }
+}
+
+uint16_t orc_partition_id_map_get(const uint64_t* words, uint32_t bits, uint64_t i)
+{
+    const uint64_t mask = ((uint64_t)1 << (bits - 1)) - 1; /* the id's bits; the flag is the entry's top bit */
+    const uint64_t bit = i * bits, off = bit % 64;
+    const uint64_t lo = words[bit / 64] >> off;
+    const uint64_t hi = off + bits - 1 > 64 ? words[bit / 64 + 1] << (64 - off) : 0;
+    return (uint16_t)((lo | hi) & mask);
+}

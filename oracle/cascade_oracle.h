@@ -82,6 +82,23 @@ void orc_retire_generations_u16(const uint16_t* T, uint64_t n, const uint64_t* s
  * (the CUB contracts the reference relies on, src/GPU_SACA.cu:1175-1210,1241-1261). */
 void orc_stable_sort_pairs_u64_u32(uint64_t* keys, uint32_t* vals, uint64_t n, int begin_bit, int end_bit);
 
+/* ---- partition ids (the step before the partition sort) ---- */
+
+/* include/Partition_ID_Map.hpp:79 with util::math::bits_for (include/utility.hpp:118-121): bits per map entry. */
+uint32_t orc_partition_id_bits(uint32_t p);
+/* test/partitioning.cpp:12-39 (= the search of include/GPU_SACA.cuh:52-66) over a zero-padded text: pid[i] = the smallest
+ * q with key(i) <= pivots[q] (word-wise, include/Packed_Prefix.hpp:122-135), p - 1 if none; key(i) = `words` packed words
+ * of suffix i, positions >= text_len read as 0. psz[q] (p counters, may be NULL) is incremented per suffix
+ * (include/GPU_SACA.cuh:69). */
+void orc_partition_ids_u16(const uint16_t* T, uint64_t n, uint64_t text_len, const uint64_t* pivots, int words, uint32_t p,
+                           uint16_t* pid, uint64_t* psz);
+/* include/Partition_ID_Map.hpp:158-177 applied to each group of 64 suffixes as include/GPU_SACA.cuh:82-91 does:
+ * group g fills words [g * bits, ...), least significant bits first; a trailing partial group writes
+ * ceil(sz * bits / 64) words. `out` must hold ceil(n / 64) * bits words; words not written are left alone. */
+void orc_pack_partition_ids(const uint16_t* pid, uint64_t n, uint32_t bits, uint64_t* out);
+/* include/Partition_ID_Map.hpp:180-189: the id of suffix i read back from the packed words. */
+uint16_t orc_partition_id_map_get(const uint64_t* words, uint32_t bits, uint64_t i);
+
 #ifdef __cplusplus
 }
 #endif

@@ -8,6 +8,7 @@
 #include "Packed_Prefix.hpp"  // gpu_saca::Packed_Prefix         (include/Packed_Prefix.hpp:91-104)
 #include "bit-layout.hpp"     // gpu_saca::bit_layout::fwd_tag   (include/bit-layout.hpp:99-100)
 #include "utility.hpp"        // gpu_saca::util::pack_word       (include/utility.hpp:147-162)
+#include "Partition_ID_Map.hpp" // gpu_saca::Partition_ID_Map::pack, bits_for (include/Partition_ID_Map.hpp:79,158-177)
 
 #include <cstring>
 #include <vector>
@@ -40,6 +41,33 @@ uint64_t ref_pack_word_u16(const uint16_t* T)
 uint64_t ref_fwd_tag_single_partition(uint64_t tgt, uint64_t n, uint64_t ell)
 {
     return gpu_saca::bit_layout::fwd_tag([](const uint64_t) { return 0; }, tgt, n, ell);
+}
+
+// Width of the reference's pivots in 64-bit words, as this library was compiled (include/Packed_Prefix.hpp:26-34).
+int ref_pivot_words(void)
+{
+    return (int)gpu_saca::K_WORDS;
+}
+
+// key(T) <= pivot with the reference's own packing and comparison (include/Packed_Prefix.hpp:91-104,122-135).
+// T must be readable for 4 * ref_pivot_words() symbols.
+int ref_pivot_key_le_u16(const uint16_t* T, const uint64_t* pivot_words)
+{
+    gpu_saca::Pivot_Key piv;
+    for(gpu_saca::idx_t w = 0; w < gpu_saca::K_WORDS; ++w)
+        piv.word[w] = pivot_words[w];
+    return gpu_saca::Pivot_Key::pack_prefix(T) <= piv ? 1 : 0;
+}
+
+uint32_t ref_partition_id_bits(uint32_t p)
+{
+    return gpu_saca::Partition_ID_Map::bits_for(static_cast<gpu_saca::p_id_t>(p));
+}
+
+// One group (or a trailing partial group) of the packed map (include/Partition_ID_Map.hpp:158-177).
+void ref_partition_id_pack(const uint16_t* src, uint64_t sz, uint32_t bits, uint64_t* dst)
+{
+    gpu_saca::Partition_ID_Map::pack(src, sz, bits, dst);
 }
 
 }

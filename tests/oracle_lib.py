@@ -49,6 +49,15 @@ def oracle():
         lib.orc_retire_generations_u16.argtypes = [vp, u64, vp, u64, vp]
         lib.orc_stable_sort_pairs_u64_u32.restype = None
         lib.orc_stable_sort_pairs_u64_u32.argtypes = [vp, vp, u64, i32, i32]
+        u32 = C.c_uint32
+        lib.orc_partition_id_bits.restype = u32
+        lib.orc_partition_id_bits.argtypes = [u32]
+        lib.orc_partition_ids_u16.restype = None
+        lib.orc_partition_ids_u16.argtypes = [vp, u64, u64, vp, i32, u32, vp, vp]
+        lib.orc_pack_partition_ids.restype = None
+        lib.orc_pack_partition_ids.argtypes = [vp, u64, u32, vp]
+        lib.orc_partition_id_map_get.restype = C.c_uint16
+        lib.orc_partition_id_map_get.argtypes = [vp, u32, u64]
         _oracle = lib
     return _oracle
 
@@ -69,6 +78,15 @@ def ref():
         lib.ref_pack_word_u16.argtypes = [vp]
         lib.ref_fwd_tag_single_partition.restype = u64
         lib.ref_fwd_tag_single_partition.argtypes = [u64, u64, u64]
+        u32 = C.c_uint32
+        lib.ref_pivot_words.restype = i32
+        lib.ref_pivot_words.argtypes = []
+        lib.ref_pivot_key_le_u16.restype = i32
+        lib.ref_pivot_key_le_u16.argtypes = [vp, vp]
+        lib.ref_partition_id_bits.restype = u32
+        lib.ref_partition_id_bits.argtypes = [u32]
+        lib.ref_partition_id_pack.restype = None
+        lib.ref_partition_id_pack.argtypes = [vp, u64, u32, vp]
         _ref = lib
     return _ref
 
@@ -169,3 +187,46 @@ def stable_sort_pairs(keys, vals, begin_bit=0, end_bit=64):
     vals = np.array(vals, dtype=np.uint32, copy=True)
     oracle().orc_stable_sort_pairs_u64_u32(_ptr(keys), _ptr(vals), keys.size, begin_bit, end_bit)
     return keys, vals
+
+
+def partition_id_bits(p):
+    return int(oracle().orc_partition_id_bits(int(p)))
+
+
+def partition_ids(T, pivots, p, words, text_len=None, n=None):
+    """(pid uint16[n], psz uint64[p]) of the suffixes [0, n) of T (default: all); pivots is a (p - 1, words) uint64 array."""
+    T = _text(T)
+    n = T.size if n is None else int(n)
+    text_len = T.size if text_len is None else int(text_len)
+    pivots = np.ascontiguousarray(pivots, dtype=np.uint64).reshape(-1)
+    assert pivots.size == (p - 1) * words
+    pid = np.zeros(max(n, 1), dtype=np.uint16)
+    psz = np.zeros(p, dtype=np.uint64)
+    oracle().orc_partition_ids_u16(_ptr(T), n, text_len, _ptr(pivots) if pivots.size else None, int(words), int(p), _ptr(pid),
+                                   _ptr(psz))
+    return pid[:n], psz
+
+
+def packed_words(n, bits):
+    """Words the packed map of n suffixes occupies up to and including a trailing partial group."""
+    return (n // 64) * bits + ((n % 64) * bits + 63) // 64
+
+
+def pack_partition_ids(pid, bits, fill=0):
+    pid = np.ascontiguousarray(pid, dtype=np.uint16)
+    out = np.full(((pid.size + 63) // 64) * bits + 1, fill, dtype=np.uint64)
+    oracle().orc_pack_partition_ids(_ptr(pid), pid.size, int(bits), _ptr(out))
+    return out
+
+
+def sample_pivots(T, p, words, rng, duplicates=False):
+    """p - 1 ascending pivots drawn from the K-grams of T (what the reference's sampler hands over, include/GPU_SACA.hpp:76)."""
+    T = _text(T)
+    if p <= 1:
+        return np.zeros((0, words), dtype=np.uint64)
+    pos = rng.integers(0, T.size, p - 1)
+    if duplicates and p > 3:
+        pos[1::3] = pos[0:-1:3][:pos[1::3].size]
+    keys = pack_prefix_np(T, words).reshape(T.size, words)[pos]
+    order = np.lexsort(tuple(keys[:, w] for w in reversed(range(words))))
+    return np.ascontiguousarray(keys[order])

@@ -27,6 +27,7 @@ def emu():
     lib.csa_sort_partition_u16_dev.argtypes = [vp, vp, u64, u64, vp, vp, u32, C.POINTER(_native.CsaStats)]
     lib.csa_radix_sort_pairs_dev.argtypes = [vp, vp, vp, u64, i32, i32, vp]
     lib.csa_last_error.restype = C.c_char_p
+    lib.csa_partition_ids_u16_dev.argtypes = [vp, u64, u64, vp, i32, u32, vp, vp, vp, vp]
     return lib
 
 
@@ -98,3 +99,22 @@ def test_emulated_radix_sort_matches_stable_sort(emu):
     assert emu.csa_radix_sort_pairs_dev(h, k.ctypes.data, v.ctypes.data, n, 3, 37, None) == 0
     emu.csa_destroy(h)
     assert np.array_equal(k, wk) and np.array_equal(v, wv)
+
+
+@pytest.mark.parametrize("words,p", [(1, 1), (1, 3), (2, 17), (3, 300), (4, 5)])
+def test_emulated_partition_ids_match_the_oracle(emu, words, p):
+    rng = np.random.default_rng(words * 1000 + p)
+    for n in (1, 64, 65, 2049, 4500):
+        T = texts.random_text(n, 3, n + p, sep_every=0)
+        pivots = oracle_lib.sample_pivots(T, p, words, rng, duplicates=True)
+        bits = oracle_lib.partition_id_bits(p)
+        ids = np.zeros(n, dtype=np.uint16)
+        packed = np.zeros(((n + 63) // 64) * bits + 1, dtype=np.uint64)
+        sizes = np.zeros(p, dtype=np.uint64)
+        rc = emu.csa_partition_ids_u16_dev(T.ctypes.data, n, n, pivots.ctypes.data if p > 1 else None, words, p, ids.ctypes.data,
+                                           packed.ctypes.data, sizes.ctypes.data, None)
+        assert rc == 0, emu.csa_last_error()
+        want_ids, want_sizes = oracle_lib.partition_ids(T, pivots, p, words)
+        assert np.array_equal(ids, want_ids) and np.array_equal(sizes, want_sizes), n
+        nw = oracle_lib.packed_words(n, bits)
+        assert np.array_equal(packed[:nw], oracle_lib.pack_partition_ids(want_ids, bits)[:nw]) and not packed[nw:].any(), n
