@@ -796,6 +796,53 @@ int csa_partition_ids_u16_dev(const uint16_t* d_text, uint64_t n, uint64_t text_
     return CSA_OK;
 }
 
+int csa_scatter_to_rank_order_dev(csa_handle* h, const uint8_t* d_suf, const uint32_t* d_rank, uint64_t part_sz,
+                                  uint8_t* d_sa40, void* stream)
+{
+    if (!h)
+        return fail(CSA_ERR_ARG, "csa_scatter_to_rank_order_dev: null handle");
+    if (part_sz == 0)
+        return CSA_OK;
+    if (!d_suf || !d_rank || !d_sa40)
+        return fail(CSA_ERR_ARG, "csa_scatter_to_rank_order_dev: null buffer");
+    if (part_sz > CSA_MAX_PART_SZ)
+        return fail(CSA_ERR_TOO_LARGE, "csa_scatter_to_rank_order_dev: %llu suffixes exceed a partition", (unsigned long long)part_sz);
+    hipStream_t s = (hipStream_t)stream;
+    HIP_TRY(hipMemsetAsync(h->counts + 3, 0, sizeof(u32), s));
+    hipLaunchKernelGGL(scatter_lanes_kernel, dim3((u32)((part_sz + 255) / 256)), dim3(256), 0, s, d_suf, d_rank, part_sz, d_sa40,
+                       h->counts + 3);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpyAsync(h->h_pinned + 3, h->counts + 3, sizeof(u32), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    if (h->h_pinned[3])
+        return fail(CSA_ERR_ARG, "csa_scatter_to_rank_order_dev: a rank lies outside [0, %llu)", (unsigned long long)part_sz);
+    return CSA_OK;
+}
+
+void csa_output_cut(uint64_t lo, uint64_t hi, uint64_t chunk_bytes, uint64_t c, uint64_t chunk_c, uint64_t out[6])
+{
+    constexpr u64 BLK = 4096; // the O_DIRECT granularity of the output file (include/Direct_File.hpp:27)
+    auto clamp = [](u64 v, u64 a, u64 b) { return v < a ? a : (v > b ? b : v); };
+    const u64 first_block = lo & ~(BLK - 1);       // chunks are laid out from the block that holds the range's start
+    const u64 aligned_lo = (lo + BLK - 1) & ~(BLK - 1);
+    u64 aligned_hi = hi & ~(BLK - 1);              // [aligned_lo, aligned_hi): the whole blocks of the range
+    if (aligned_hi < aligned_lo)
+        aligned_hi = aligned_lo;                   // the range lies inside one block
+    // the chunk's piece: its window of chunk_bytes, clipped to the whole blocks
+    out[0] = clamp(first_block + c * chunk_bytes, aligned_lo, aligned_hi);
+    out[1] = clamp(first_block + (c + 1) * chunk_bytes, out[0], aligned_hi);
+    // the first chunk also carries what precedes the whole blocks, the last one what follows them
+    out[2] = out[3] = out[4] = out[5] = 0;
+    if (c == 0) {
+        out[2] = lo;
+        out[3] = hi < aligned_lo ? hi : aligned_lo;
+    }
+    if (c + 1 == chunk_c) {
+        out[4] = aligned_hi;
+        out[5] = hi > aligned_hi ? hi : aligned_hi;
+    }
+}
+
 const char* csa_last_error(void) { return g_err; }
 
 uint64_t csa_bytes_per_suffix(int key_words)

@@ -693,6 +693,29 @@ __global__ __launch_bounds__(256) void emit_sa40_kernel(const u32* __restrict__ 
     }
 }
 
+__device__ __forceinline__ u64 load_sa40(const u8* sa, u64 r);
+
+// Rank-order scatter of a partition that arrives as (suffix lane, local rank) pairs in any order:
+// out lane[rank[i]] = lane[i]. The reference scatters into 8-byte words and packs the lanes in a second kernel
+// (include/GPU_SACA.cuh:167-182 and :126-133, src/GPU_SACA.cu:2133-2143); here the 5 bytes go straight to their place.
+// `bad` is set if a rank is out of range (the reference traps under -DTESTS).
+__global__ __launch_bounds__(256) void scatter_lanes_kernel(const u8* __restrict__ suf, const u32* __restrict__ rank, u64 n,
+                                                           u8* __restrict__ out, u32* bad)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n)
+        return;
+    const u64 r = rank[i];
+    if (r >= n) {
+        atomicExch(bad, 1u);
+        return;
+    }
+    const u64 v = load_sa40(suf, i);
+#pragma unroll
+    for (int b = 0; b < 5; ++b)
+        out[5 * r + b] = (u8)(v >> (8 * b));
+}
+
 // Standalone K-gram packing (reference: include/utility.hpp:147-162, include/Packed_Prefix.hpp:91-104).
 __global__ __launch_bounds__(256) void pack_keys_kernel(const u16* __restrict__ text, u32 n, int key_words,
                                                         u64* __restrict__ keys)

@@ -95,6 +95,20 @@ class PartitionSorter:
         _native.check(self._lib.csa_radix_sort_pairs_dev(self._h, keys.data_ptr(), vals.data_ptr(), keys.numel(),
                                                          int(begin_bit), int(end_bit), stream or None))
 
+    def scatter_to_rank_order(self, suf40, rank, out=None):
+        """out lane[rank[i]] = lane i of suf40 (csa_scatter_to_rank_order_dev): uint8 tensor of 5 * m bytes, int32/uint32
+        tensor of m ranks (a permutation of [0, m)). Returns the uint8 tensor of 5 * m bytes in rank order."""
+        import torch
+        m = rank.numel()
+        assert suf40.is_cuda and rank.is_cuda and suf40.dtype == torch.uint8 and rank.element_size() == 4
+        assert suf40.numel() >= SA_WIDTH * m
+        if out is None:
+            out = torch.empty(SA_WIDTH * m + 128, dtype=torch.uint8, device=rank.device)
+        stream = torch.cuda.current_stream(rank.device).cuda_stream
+        _native.check(self._lib.csa_scatter_to_rank_order_dev(self._h, suf40.data_ptr(), rank.data_ptr(), m, out.data_ptr(),
+                                                              stream or None))
+        return out[:SA_WIDTH * m]
+
     def verify(self, text, sa40, index_base=0):
         """Device-side O(n) suffix-array check (csa_verify_sa40_dev). Returns True if sa40 is the suffix array."""
         import torch
@@ -142,6 +156,14 @@ def partition_ids(text, pivots, p, n=None, text_len=None, want_ids=True, want_pa
                                                 packed.data_ptr() if want_packed else None,
                                                 sizes.data_ptr() if sizes is not None else None, stream or None))
     return (ids[:n] if want_ids else None), packed, sizes
+
+
+def output_cut(lo, hi, chunk_bytes, c, chunk_c):
+    """(piece_lo, piece_hi, head_lo, head_hi, tail_lo, tail_hi) of chunk c's share of the output byte range [lo, hi)
+    (csa_output_cut; the reference's Output_File::cut, src/Output_File.cpp:18-35)."""
+    out = (C.c_uint64 * 6)()
+    _native.load().csa_output_cut(int(lo), int(hi), int(chunk_bytes), int(c), int(chunk_c), C.byref(out))
+    return tuple(int(v) for v in out)
 
 
 def sort_partition(text, key_words=1):

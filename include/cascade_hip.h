@@ -132,6 +132,24 @@ int csa_partition_ids_u16_dev(const uint16_t* d_text, uint64_t n, uint64_t text_
                               int pivot_words, uint32_t p, uint16_t* d_pid, uint64_t* d_packed, uint64_t* d_psz,
                               void* stream);
 
+/* ---- the step after the partition sort, for partitions that come back as (suffix, local rank) pairs ---- */
+
+/* d_sa40 entry rank[i] = d_suf entry i for i in [0, part_sz): 5-byte little-endian lanes in, lanes in rank order out.
+ * d_rank must be a permutation of [0, part_sz); an entry out of range fails the call with CSA_ERR_ARG (checked on the
+ * device; the reference traps under -DTESTS). The handle lends its error word only; any capacity will do.
+ * Replaces scatter_suffixes_to_rank_kernel + pack_lanes_kernel (include/GPU_SACA.cuh:167-182,126-133) of
+ * GPU_SACA::scatter_to_rank_order (src/GPU_SACA.cu:2107-2143). The call returns after the stream has finished. */
+int csa_scatter_to_rank_order_dev(csa_handle* h, const uint8_t* d_suf, const uint32_t* d_rank, uint64_t part_sz,
+                                  uint8_t* d_sa40, void* stream);
+
+/* The byte ranges of a partition's output that chunk c of chunk_c carries to the output file, so that every write
+ * but the first and the last of the file is a whole number of 4 KiB disk blocks: [lo, hi) is the partition's byte
+ * range in the file, chunk_bytes the bytes of a full chunk.
+ * out[0..1] = the chunk's block-aligned piece, out[2..3] = the range's unaligned head (first chunk only),
+ * out[4..5] = its unaligned tail (last chunk only); absent parts are empty intervals.
+ * Pure host arithmetic: Output_File::cut (src/Output_File.cpp:18-35; struct at include/Output_File.hpp:29-37). */
+void csa_output_cut(uint64_t lo, uint64_t hi, uint64_t chunk_bytes, uint64_t c, uint64_t chunk_c, uint64_t out[6]);
+
 /* Message of the calling thread's last failed call ("" if none). */
 const char* csa_last_error(void);
 

@@ -440,3 +440,36 @@ uint16_t orc_partition_id_map_get(const uint64_t* words, uint32_t bits, uint64_t
     const uint64_t hi = off + bits - 1 > 64 ? words[bit / 64 + 1] << (64 - off) : 0;
     return (uint16_t)((lo | hi) & mask);
 }
+
+/* ---------- after the partition sort ---------- */
+
+int orc_scatter_to_rank_order(const uint8_t* suf, const uint32_t* rank, uint64_t n, uint8_t* out)
+{
+    for (uint64_t i = 0; i < n; ++i) {
+        if (rank[i] >= n)
+            return -1; /* include/GPU_SACA.cuh:176-179 */
+        orc_sa40_store(out, rank[i], orc_sa40_load(suf, i)); /* SA[rank[i]] = suffix; then lane::store of each word */
+    }
+    return 0;
+}
+
+static uint64_t u64_min(uint64_t a, uint64_t b) { return a < b ? a : b; }
+static uint64_t u64_max(uint64_t a, uint64_t b) { return a > b ? a : b; }
+
+void orc_output_cut(uint64_t lo, uint64_t hi, uint64_t chunk_bytes, uint64_t c, uint64_t chunk_c, uint64_t out[6])
+{
+    const uint64_t B = 4096; /* Direct_File::DISK_BLOCK, include/Direct_File.hpp:27 */
+    const uint64_t base = lo / B * B, mid_lo = (lo + B - 1) / B * B, mid_hi = u64_max(mid_lo, hi / B * B);
+    for (int i = 0; i < 6; ++i)
+        out[i] = 0;
+    out[0] = u64_min(u64_max(mid_lo, base + c * chunk_bytes), mid_hi);
+    out[1] = u64_max(out[0], u64_min(mid_hi, base + (c + 1) * chunk_bytes));
+    if (c == 0) {
+        out[2] = lo;
+        out[3] = u64_min(hi, mid_lo);
+    }
+    if (c + 1 == chunk_c) {
+        out[4] = u64_max(mid_lo, hi / B * B);
+        out[5] = u64_max(out[4], hi);
+    }
+}

@@ -99,6 +99,15 @@ void orc_pack_partition_ids(const uint16_t* pid, uint64_t n, uint32_t bits, uint
 /* include/Partition_ID_Map.hpp:180-189: the id of suffix i read back from the packed words. */
 uint16_t orc_partition_id_map_get(const uint64_t* words, uint32_t bits, uint64_t i);
 
+/* ---- after the partition sort ---- */
+
+/* include/GPU_SACA.cuh:167-182 followed by :126-133: out lane[rank[i]] = lane i of suf (5-byte lanes, include/lane.hpp:51-79).
+ * Returns 0, or -1 if some rank[i] >= n (the reference traps there under -DTESTS). */
+int orc_scatter_to_rank_order(const uint8_t* suf, const uint32_t* rank, uint64_t n, uint8_t* out);
+/* src/Output_File.cpp:18-35: how the byte range [lo, hi) of a partition's output is shared out over chunk_c chunks of
+ * chunk_bytes so that all but the edges are whole 4 KiB blocks. out = {piece lo, hi, head lo, hi, tail lo, hi}. */
+void orc_output_cut(uint64_t lo, uint64_t hi, uint64_t chunk_bytes, uint64_t c, uint64_t chunk_c, uint64_t out[6]);
+
 #ifdef __cplusplus
 }
 #endif

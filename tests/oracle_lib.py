@@ -58,6 +58,10 @@ def oracle():
         lib.orc_pack_partition_ids.argtypes = [vp, u64, u32, vp]
         lib.orc_partition_id_map_get.restype = C.c_uint16
         lib.orc_partition_id_map_get.argtypes = [vp, u32, u64]
+        lib.orc_scatter_to_rank_order.restype = i32
+        lib.orc_scatter_to_rank_order.argtypes = [vp, vp, u64, vp]
+        lib.orc_output_cut.restype = None
+        lib.orc_output_cut.argtypes = [u64, u64, u64, u64, u64, vp]
         _oracle = lib
     return _oracle
 
@@ -230,3 +234,17 @@ def sample_pivots(T, p, words, rng, duplicates=False):
     keys = pack_prefix_np(T, words).reshape(T.size, words)[pos]
     order = np.lexsort(tuple(keys[:, w] for w in reversed(range(words))))
     return np.ascontiguousarray(keys[order])
+
+
+def scatter_to_rank_order(suf40, rank):
+    suf40 = np.ascontiguousarray(suf40, dtype=np.uint8)
+    rank = np.ascontiguousarray(rank, dtype=np.uint32)
+    out = np.zeros(5 * rank.size, dtype=np.uint8)
+    rc = oracle().orc_scatter_to_rank_order(_ptr(suf40), _ptr(rank), rank.size, _ptr(out))
+    return rc, out
+
+
+def output_cut(lo, hi, chunk_bytes, c, chunk_c):
+    out = np.zeros(6, dtype=np.uint64)
+    oracle().orc_output_cut(int(lo), int(hi), int(chunk_bytes), int(c), int(chunk_c), _ptr(out))
+    return [int(v) for v in out]
