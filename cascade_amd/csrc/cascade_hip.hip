@@ -796,6 +796,48 @@ int csa_partition_ids_u16_dev(const uint16_t* d_text, uint64_t n, uint64_t text_
     return CSA_OK;
 }
 
+int csa_stage_slab_u16_dev(const uint16_t* d_text, uint64_t n, const uint8_t* d_suf40, uint64_t count, int key_words,
+                           const uint64_t* d_pid_map, uint32_t p, uint64_t ctx, int generation0, uint64_t* d_keys,
+                           uint32_t* d_beta, void* stream)
+{
+    if (key_words < 1 || key_words > 4)
+        return fail(CSA_ERR_ARG, "csa_stage_slab_u16_dev: key_words = %d is outside [1, 4]", key_words);
+    if (p < 1 || p > 32768u)
+        return fail(CSA_ERR_ARG, "csa_stage_slab_u16_dev: p = %u is outside [1, 32768] (bit 15 of a route is the retirement flag)", p);
+    if (generation0 && ctx != 4ull * (u64)key_words)
+        return fail(CSA_ERR_ARG, "csa_stage_slab_u16_dev: generation 0 runs at ctx = ell = %d", 4 * key_words);
+    if (count == 0)
+        return CSA_OK;
+    if (!d_text || !d_suf40 || !d_pid_map || !d_beta)
+        return fail(CSA_ERR_ARG, "csa_stage_slab_u16_dev: null buffer");
+    if (n > CSA_MAX_INDEX)
+        return fail(CSA_ERR_TOO_LARGE, "csa_stage_slab_u16_dev: text of %llu symbols", (unsigned long long)n);
+    StageArgs a;
+    a.text = d_text;
+    a.n = n;
+    a.suf40 = d_suf40;
+    a.count = count;
+    a.pid_map = d_pid_map;
+    a.bits = csa_partition_id_bits(p);
+    a.ctx = ctx;
+    a.ell = 4u * (u32)key_words;
+    a.gen0 = generation0 ? 1 : 0;
+    a.keys = d_keys;
+    a.beta = d_beta;
+    const u64 blocks = (count + 255) / 256;
+    if (blocks > 0x7FFFFFFFull)
+        return fail(CSA_ERR_TOO_LARGE, "csa_stage_slab_u16_dev: %llu suffixes in one call", (unsigned long long)count);
+    hipStream_t s = (hipStream_t)stream;
+    switch (key_words) {
+    case 1: hipLaunchKernelGGL(stage_slab_kernel<1>, dim3((u32)blocks), dim3(256), 0, s, a); break;
+    case 2: hipLaunchKernelGGL(stage_slab_kernel<2>, dim3((u32)blocks), dim3(256), 0, s, a); break;
+    case 3: hipLaunchKernelGGL(stage_slab_kernel<3>, dim3((u32)blocks), dim3(256), 0, s, a); break;
+    default: hipLaunchKernelGGL(stage_slab_kernel<4>, dim3((u32)blocks), dim3(256), 0, s, a); break;
+    }
+    HIP_TRY(hipGetLastError());
+    return CSA_OK;
+}
+
 int csa_scatter_to_rank_order_dev(csa_handle* h, const uint8_t* d_suf, const uint32_t* d_rank, uint64_t part_sz,
                                   uint8_t* d_sa40, void* stream)
 {

@@ -154,4 +154,82 @@ __global__ __launch_bounds__(PID_BLOCK) void partition_ids_kernel(PartitionIdArg
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Staging of a partition's suffixes on the device: what the reference's host threads do per slab before every
+// upload (GPU_SACA::stage_slab, src/GPU_SACA.cu:1611-1692). For the suffix j of every 5-byte lane:
+//   generation 0 : key = its packed K-gram (W words) gathered from the text in HBM;
+//                  beta = (route of j - ell) | forward tag of j + ell << 16
+//   generation t : beta = (route of j - ctx) | route of j - ctx / 2 << 16
+// route(x) = partition id of x, with bit 15 set if x has retired; 0 where x would lie before the text
+// (include/bit-layout.hpp:137-152). Forward tag: id + ell, or n + ell - 1 - tgt past the end of the text (:99-100).
+// Ids and retirement flags are read from the packed partition-id map.
+// ---------------------------------------------------------------------------------------------
+
+struct StageArgs {
+    const u16* text;
+    u64 n; // symbols in the text
+    const u8* suf40;
+    u64 count;
+    const u64* pid_map; // packed map of the whole text
+    u32 bits;           // bits per map entry
+    u64 ctx;            // context of the generation (ell at generation 0)
+    u32 ell;
+    int gen0;
+    u64* keys; // [count][W], generation 0 only; may be null
+    u32* beta; // [count]
+};
+
+// entry i of the packed map: id in the low bits - 1 bits, retirement flag on top (include/Partition_ID_Map.hpp:180-196)
+__device__ __forceinline__ u32 pid_map_entry(const u64* __restrict__ map, u32 bits, u64 i)
+{
+    const u64 bit = i * bits, off = bit & 63u;
+    u64 v = map[bit >> 6] >> off;
+    if (off + bits > 64)
+        v |= map[(bit >> 6) + 1] << (64 - off);
+    return (u32)(v & ((1ull << bits) - 1ull));
+}
+
+__device__ __forceinline__ u32 pid_route(const u64* __restrict__ map, u32 bits, u64 x)
+{
+    const u32 e = pid_map_entry(map, bits, x);
+    const u32 id = e & ((1u << (bits - 1)) - 1u);
+    return (e >> (bits - 1)) ? (id | 0x8000u) : id; // BETA_RETIRED, include/bit-layout.hpp:135
+}
+
+template <int W>
+__global__ __launch_bounds__(256) void stage_slab_kernel(StageArgs a)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= a.count)
+        return;
+    u64 j = 0;
+#pragma unroll
+    for (int b = 0; b < 5; ++b)
+        j |= (u64)a.suf40[5 * i + b] << (8 * b);
+    if (a.gen0 && a.keys) {
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+            u64 k = 0;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const u64 pos = j + 4ull * w + q;
+                k = (k << 16) | (pos < a.n ? (u64)a.text[pos] : 0ull);
+            }
+            a.keys[i * W + w] = k;
+        }
+    }
+    const u32 cur = j < a.ctx ? 0u : pid_route(a.pid_map, a.bits, j - a.ctx);
+    u32 prev;
+    if (a.gen0) {
+        const u64 tgt = j + a.ell;
+        const u64 tag = tgt < a.n ? (u64)(pid_map_entry(a.pid_map, a.bits, tgt) & ((1u << (a.bits - 1)) - 1u)) + a.ell
+                                  : a.n + a.ell - 1 - tgt;
+        prev = (u32)tag & 0xFFFFu; // the tag travels in a 16-bit half (include/bit-layout.hpp:137)
+    } else {
+        const u64 stride = a.ctx / 2;
+        prev = j < stride ? 0u : pid_route(a.pid_map, a.bits, j - stride);
+    }
+    a.beta[i] = (prev << 16) | cur;
+}
+
 } // namespace csa

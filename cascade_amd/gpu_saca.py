@@ -158,6 +158,24 @@ def partition_ids(text, pivots, p, n=None, text_len=None, want_ids=True, want_pa
     return (ids[:n] if want_ids else None), packed, sizes
 
 
+def stage_slab(text, suf40, key_words, pid_map, p, ctx, generation0):
+    """Keys (generation 0) and routing-tag pairs of a partition's suffixes, computed on the device from the text and the
+    packed partition-id map (csa_stage_slab_u16_dev; the reference's host loop GPU_SACA::stage_slab,
+    src/GPU_SACA.cu:1674-1691). suf40: uint8 tensor of 5-byte lanes. Returns (keys int64 [count, key_words] or None,
+    beta int32 [count])."""
+    import torch
+    lib = _native.load()
+    count = suf40.numel() // SA_WIDTH
+    dev = text.device
+    keys = torch.empty((max(count, 1), key_words), dtype=torch.int64, device=dev) if generation0 else None
+    beta = torch.empty(max(count, 1), dtype=torch.int32, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    _native.check(lib.csa_stage_slab_u16_dev(text.data_ptr(), text.numel(), suf40.data_ptr(), count, int(key_words),
+                                             pid_map.data_ptr(), int(p), int(ctx), 1 if generation0 else 0,
+                                             keys.data_ptr() if generation0 else None, beta.data_ptr(), stream or None))
+    return (keys[:count] if generation0 else None), beta[:count]
+
+
 def output_cut(lo, hi, chunk_bytes, c, chunk_c):
     """(piece_lo, piece_hi, head_lo, head_hi, tail_lo, tail_hi) of chunk c's share of the output byte range [lo, hi)
     (csa_output_cut; the reference's Output_File::cut, src/Output_File.cpp:18-35)."""

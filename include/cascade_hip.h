@@ -132,6 +132,19 @@ int csa_partition_ids_u16_dev(const uint16_t* d_text, uint64_t n, uint64_t text_
                               int pivot_words, uint32_t p, uint16_t* d_pid, uint64_t* d_packed, uint64_t* d_psz,
                               void* stream);
 
+/* Staging of `count` suffixes of a partition (5-byte lanes d_suf40, any order) on the device, for a text and its packed
+ * partition-id map (as csa_partition_ids_u16_dev writes it, retirement flags included) resident in HBM:
+ *   generation0 != 0 : d_keys[i * key_words + w] = K-gram word w of suffix i (may be NULL to skip), and
+ *                      d_beta[i] = route(j - ell) | forward tag(j + ell) << 16, with ell = 4 * key_words = ctx;
+ *   generation0 == 0 : d_beta[i] = route(j - ctx) | route(j - ctx / 2) << 16.
+ * route(x) = id of x's partition, bit 15 set if x has retired, 0 if x would lie before the text; forward tag = id + ell, or
+ * n + ell - 1 - (j + ell) when j + ell is past the end (include/bit-layout.hpp:99-100,137-152).
+ * Replaces the host loop of GPU_SACA::stage_slab (src/GPU_SACA.cu:1674-1691) and the upload of 8 * key_words bytes
+ * per suffix that follows it (src/GPU_SACA.cu:1129). */
+int csa_stage_slab_u16_dev(const uint16_t* d_text, uint64_t n, const uint8_t* d_suf40, uint64_t count, int key_words,
+                           const uint64_t* d_pid_map, uint32_t p, uint64_t ctx, int generation0, uint64_t* d_keys,
+                           uint32_t* d_beta, void* stream);
+
 /* ---- the step after the partition sort, for partitions that come back as (suffix, local rank) pairs ---- */
 
 /* d_sa40 entry rank[i] = d_suf entry i for i in [0, part_sz): 5-byte little-endian lanes in, lanes in rank order out.

@@ -473,3 +473,32 @@ void orc_output_cut(uint64_t lo, uint64_t hi, uint64_t chunk_bytes, uint64_t c, 
         out[5] = u64_max(out[4], hi);
     }
 }
+
+/* ---------- slab staging ---------- */
+
+static uint16_t orc_route(uint16_t p_id, int retired)
+{
+    return retired ? (uint16_t)(p_id | 0x8000u) : p_id; /* include/bit-layout.hpp:135,152 */
+}
+
+void orc_stage_slab_u16(const uint16_t* T, uint64_t n, const uint8_t* suf40, uint64_t count, int key_words,
+                        const uint16_t* pid, const uint8_t* retired, uint64_t ctx, int generation0, uint64_t* keys,
+                        uint32_t* beta)
+{
+    const uint64_t ell = 4 * (uint64_t)key_words, stride = ctx / 2;
+    for (uint64_t i = 0; i < count; ++i) {
+        const uint64_t j = orc_sa40_load(suf40, i);
+        if (generation0 && keys)
+            orc_pack_prefix_u16(T, n, j, key_words, keys + i * key_words); /* src/GPU_SACA.cu:1683 */
+        /* src/GPU_SACA.cu:1688-1690 */
+        const uint16_t cur = j < ctx ? 0 : orc_route(pid[j - ctx], retired[j - ctx]);
+        uint16_t prev;
+        if (generation0) {
+            const uint64_t tgt = j + ell;
+            prev = (uint16_t)(tgt < n ? (uint64_t)pid[tgt] + ell : n + ell - 1 - tgt); /* include/bit-layout.hpp:100 */
+        } else {
+            prev = j < stride ? 0 : orc_route(pid[j - stride], retired[j - stride]);
+        }
+        beta[i] = ((uint32_t)prev << 16) | cur; /* include/bit-layout.hpp:137 */
+    }
+}

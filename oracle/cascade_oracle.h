@@ -99,6 +99,13 @@ void orc_pack_partition_ids(const uint16_t* pid, uint64_t n, uint32_t bits, uint
 /* include/Partition_ID_Map.hpp:180-189: the id of suffix i read back from the packed words. */
 uint16_t orc_partition_id_map_get(const uint64_t* words, uint32_t bits, uint64_t i);
 
+/* src/GPU_SACA.cu:1674-1691 (GPU_SACA::stage_slab without the spilled-map branch) with include/bit-layout.hpp:99-100,
+ * 137-152: keys (generation 0, may be NULL) and routing-tag pairs of `count` suffix lanes. pid[x] and retired[x]
+ * (one byte each, 0/1) describe every text position x in [0, n). */
+void orc_stage_slab_u16(const uint16_t* T, uint64_t n, const uint8_t* suf40, uint64_t count, int key_words,
+                        const uint16_t* pid, const uint8_t* retired, uint64_t ctx, int generation0, uint64_t* keys,
+                        uint32_t* beta);
+
 /* ---- after the partition sort ---- */
 
 /* include/GPU_SACA.cuh:167-182 followed by :126-133: out lane[rank[i]] = lane i of suf (5-byte lanes, include/lane.hpp:51-79).

@@ -70,4 +70,16 @@ void ref_partition_id_pack(const uint16_t* src, uint64_t sz, uint32_t bits, uint
     gpu_saca::Partition_ID_Map::pack(src, sz, bits, dst);
 }
 
+// The routing-tag pair of suffix j, put together with the reference's own helpers (include/bit-layout.hpp:99-100,137,152)
+// the way GPU_SACA::stage_slab does (src/GPU_SACA.cu:1688-1690); ids and retirement flags come as plain arrays.
+uint32_t ref_beta_u16(uint64_t j, uint64_t n, uint64_t ell, uint64_t ctx, int generation0, const uint16_t* pid, const uint8_t* retired)
+{
+    namespace bl = gpu_saca::bit_layout;
+    const uint64_t stride = ctx / 2;
+    const auto id = [pid](const uint64_t x) { return pid[x]; };
+    return bl::beta_pair(j < ctx ? 0 : bl::route(pid[j - ctx], retired[j - ctx] != 0),
+                         generation0 ? bl::fwd_tag(id, j + ell, n, ell)
+                                     : (j < stride ? 0 : bl::route(pid[j - stride], retired[j - stride] != 0)));
+}
+
 }

@@ -58,6 +58,8 @@ def oracle():
         lib.orc_pack_partition_ids.argtypes = [vp, u64, u32, vp]
         lib.orc_partition_id_map_get.restype = C.c_uint16
         lib.orc_partition_id_map_get.argtypes = [vp, u32, u64]
+        lib.orc_stage_slab_u16.restype = None
+        lib.orc_stage_slab_u16.argtypes = [vp, u64, vp, u64, i32, vp, vp, u64, i32, vp, vp]
         lib.orc_scatter_to_rank_order.restype = i32
         lib.orc_scatter_to_rank_order.argtypes = [vp, vp, u64, vp]
         lib.orc_output_cut.restype = None
@@ -91,6 +93,8 @@ def ref():
         lib.ref_partition_id_bits.argtypes = [u32]
         lib.ref_partition_id_pack.restype = None
         lib.ref_partition_id_pack.argtypes = [vp, u64, u32, vp]
+        lib.ref_beta_u16.restype = u32
+        lib.ref_beta_u16.argtypes = [u64, u64, u64, u64, i32, vp, vp]
         _ref = lib
     return _ref
 
@@ -248,3 +252,24 @@ def output_cut(lo, hi, chunk_bytes, c, chunk_c):
     out = np.zeros(6, dtype=np.uint64)
     oracle().orc_output_cut(int(lo), int(hi), int(chunk_bytes), int(c), int(chunk_c), _ptr(out))
     return [int(v) for v in out]
+
+
+def stage_slab(T, suf, key_words, pid, retired, ctx, generation0):
+    """(keys uint64[count, key_words] or None, beta uint32[count]) for the suffixes `suf` (uint64 array)."""
+    T = _text(T)
+    suf = np.ascontiguousarray(suf, dtype=np.uint64)
+    lanes = u64_to_sa40(suf)
+    pid = np.ascontiguousarray(pid, dtype=np.uint16)
+    retired = np.ascontiguousarray(retired, dtype=np.uint8)
+    keys = np.zeros((suf.size, key_words), dtype=np.uint64) if generation0 else None
+    beta = np.zeros(suf.size, dtype=np.uint32)
+    oracle().orc_stage_slab_u16(_ptr(T), T.size, _ptr(lanes), suf.size, int(key_words), _ptr(pid), _ptr(retired), int(ctx),
+                                1 if generation0 else 0, _ptr(keys) if generation0 else None, _ptr(beta))
+    return keys, beta
+
+
+def set_retired(words, bits, positions):
+    """Marks text positions retired in a packed map: the top bit of their entries (include/Partition_ID_Map.hpp:55,198-202)."""
+    for x in positions:
+        bit = int(x) * bits + bits - 1
+        words[bit // 64] |= np.uint64(1) << np.uint64(bit % 64)

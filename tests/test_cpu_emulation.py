@@ -28,6 +28,8 @@ def emu():
     lib.csa_radix_sort_pairs_dev.argtypes = [vp, vp, vp, u64, i32, i32, vp]
     lib.csa_last_error.restype = C.c_char_p
     lib.csa_partition_ids_u16_dev.argtypes = [vp, u64, u64, vp, i32, u32, vp, vp, vp, vp]
+    lib.csa_stage_slab_u16_dev.argtypes = [vp, u64, vp, u64, i32, vp, u32, u64, i32, vp, vp, vp]
+    lib.csa_scatter_to_rank_order_dev.argtypes = [vp, vp, vp, u64, vp, vp]
     return lib
 
 
@@ -118,3 +120,34 @@ def test_emulated_partition_ids_match_the_oracle(emu, words, p):
         assert np.array_equal(ids, want_ids) and np.array_equal(sizes, want_sizes), n
         nw = oracle_lib.packed_words(n, bits)
         assert np.array_equal(packed[:nw], oracle_lib.pack_partition_ids(want_ids, bits)[:nw]) and not packed[nw:].any(), n
+
+
+@pytest.mark.parametrize("generation0,ctx,key_words", [(True, 4, 1), (False, 16, 2)])
+def test_emulated_slab_staging_and_rank_order_scatter(emu, generation0, ctx, key_words):
+    rng = np.random.default_rng(ctx)
+    n, p = 3000, 11
+    T = texts.random_text(n, 4, 2, sep_every=0)
+    pid = rng.integers(0, p, n).astype(np.uint16)
+    retired = (rng.random(n) < 0.3).astype(np.uint8)
+    bits = oracle_lib.partition_id_bits(p)
+    words = oracle_lib.pack_partition_ids(pid, bits)
+    oracle_lib.set_retired(words, bits, np.flatnonzero(retired))
+    suf = rng.permutation(n)[:1000].astype(np.uint64)
+    lanes = oracle_lib.u64_to_sa40(suf)
+    keys = np.zeros((suf.size, key_words), dtype=np.uint64)
+    beta = np.zeros(suf.size, dtype=np.uint32)
+    rc = emu.csa_stage_slab_u16_dev(T.ctypes.data, n, lanes.ctypes.data, suf.size, key_words, words.ctypes.data, p, ctx,
+                                    1 if generation0 else 0, keys.ctypes.data if generation0 else None, beta.ctypes.data, None)
+    assert rc == 0, emu.csa_last_error()
+    want_keys, want_beta = oracle_lib.stage_slab(T, suf, key_words, pid, retired, ctx, generation0)
+    assert np.array_equal(beta, want_beta)
+    if generation0:
+        assert np.array_equal(keys, want_keys)
+    # and the way back: the same lanes scattered to a random rank order
+    rank = rng.permutation(suf.size).astype(np.uint32)
+    out = np.zeros(5 * suf.size, dtype=np.uint8)
+    h = C.c_void_p()
+    assert emu.csa_create(16, 1, C.byref(h)) == 0
+    rc = emu.csa_scatter_to_rank_order_dev(h, lanes.ctypes.data, rank.ctypes.data, suf.size, out.ctypes.data, None)
+    emu.csa_destroy(h)
+    assert rc == 0 and np.array_equal(out, oracle_lib.scatter_to_rank_order(lanes, rank)[1])

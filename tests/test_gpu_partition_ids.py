@@ -108,3 +108,30 @@ def test_bad_arguments_are_refused(torch_mod):
     assert lib.csa_partition_ids_u16_dev(None, 10, 10, None, 5, 3, None, None, None, None) == _native.CSA_ERR_ARG
     assert lib.csa_partition_ids_u16_dev(None, 10, 5, None, 2, 1, None, None, None, None) == _native.CSA_ERR_ARG
     assert lib.csa_partition_ids_u16_dev(None, 0, 0, None, 2, 3, None, None, None, None) == _native.CSA_OK
+
+
+@pytest.mark.parametrize("generation0,ctx,key_words", [(True, 4, 1), (True, 8, 2), (False, 8, 1), (False, 4096, 2)])
+def test_slab_staging_on_the_device_matches_the_oracle(torch_mod, generation0, ctx, key_words):
+    # the packed map comes from the partition-id kernel itself; some suffixes are then marked retired
+    from cascade_amd import partition_ids, stage_slab
+    torch = torch_mod
+    rng = np.random.default_rng(ctx)
+    n, p = 300000, 29
+    T = texts.random_text(n, 6, 1, sep_every=0)
+    pivots = oracle_lib.sample_pivots(T, p, 2, rng)
+    d_T = dev16(torch, T)
+    ids, packed, _ = partition_ids(d_T, dev64(torch, pivots).reshape(-1, 2), p)
+    pid = ids.cpu().numpy().view(np.uint16)
+    bits = oracle_lib.partition_id_bits(p)
+    words = packed.cpu().numpy().view(np.uint64).copy()
+    retired = (rng.random(n) < 0.25).astype(np.uint8)
+    oracle_lib.set_retired(words, bits, np.flatnonzero(retired))
+    suf = rng.permutation(n)[:100000].astype(np.uint64)
+    suf[:6] = [0, 1, n - 1, n - 2, ctx, max(ctx // 2 - 1, 0)]
+    lanes = oracle_lib.u64_to_sa40(suf)
+    print(f"  stage n={n} count={suf.size} ctx={ctx} gen0={generation0}", flush=True)
+    keys, beta = stage_slab(d_T, torch.from_numpy(lanes).cuda(), key_words, dev64(torch, words), p, ctx, generation0)
+    want_keys, want_beta = oracle_lib.stage_slab(T, suf, key_words, pid, retired, ctx, generation0)
+    assert np.array_equal(beta.cpu().numpy().view(np.uint32), want_beta)
+    if generation0:
+        assert np.array_equal(keys.cpu().numpy().view(np.uint64), want_keys)

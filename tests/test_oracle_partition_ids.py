@@ -92,3 +92,29 @@ def test_a_chunk_in_the_middle_of_the_text_sees_the_symbols_after_it():
     off, n = 128, 512
     chunk, _ = oracle_lib.partition_ids(T[off:], pivots, p, words, text_len=n + 4 * words - 1, n=n)
     assert np.array_equal(chunk, whole[off:off + n])
+
+
+@pytest.mark.parametrize("generation0,ctx,key_words", [(True, 4, 1), (True, 8, 2), (False, 8, 1), (False, 64, 2)])
+def test_staging_matches_the_references_tag_helpers(generation0, ctx, key_words):
+    rng = np.random.default_rng(ctx + key_words)
+    n, p = 700, 37
+    T = texts.random_text(n, 5, 3, sep_every=0)
+    pid = rng.integers(0, p, n).astype(np.uint16)
+    retired = (rng.random(n) < 0.3).astype(np.uint8)
+    suf = rng.permutation(n)[:300].astype(np.uint64)
+    suf[:4] = [0, n - 1, ctx, max(ctx // 2 - 1, 0)]
+    keys, beta = oracle_lib.stage_slab(T, suf, key_words, pid, retired, ctx, generation0)
+    ell = 4 * key_words
+    for i, j in enumerate(suf.tolist()):
+        cur = 0 if j < ctx else int(pid[j - ctx]) | (0x8000 if retired[j - ctx] else 0)
+        if generation0:
+            prev = (int(pid[j + ell]) + ell) if j + ell < n else n + ell - 1 - (j + ell)
+        else:
+            prev = 0 if j < ctx // 2 else int(pid[j - ctx // 2]) | (0x8000 if retired[j - ctx // 2] else 0)
+        assert beta[i] == ((prev & 0xFFFF) << 16 | cur), (i, j)
+    if generation0:
+        assert np.array_equal(keys, oracle_lib.pack_prefix_np(T, key_words)[suf.astype(np.int64)])
+    ref = oracle_lib.ref()
+    if ref is not None:
+        for i, j in enumerate(suf.tolist()):
+            assert beta[i] == ref.ref_beta_u16(j, n, ell, ctx, 1 if generation0 else 0, pid.ctypes.data, retired.ctypes.data), (i, j)
