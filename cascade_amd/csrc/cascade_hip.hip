@@ -4,6 +4,7 @@
 
 #include "device_utils.hpp"
 #include "doubling.hpp"
+#include "messages.hpp"
 #include "partition_ids.hpp"
 #include "radix_sort.hpp"
 
@@ -792,6 +793,92 @@ int csa_partition_ids_u16_dev(const uint16_t* d_text, uint64_t n, uint64_t text_
     default: CSA_LAUNCH_PID(4); break;
     }
 #undef CSA_LAUNCH_PID
+    HIP_TRY(hipGetLastError());
+    return CSA_OK;
+}
+
+namespace {
+int fill_message_args(MessageArgs& a, const char* who, const uint64_t* d_sa, const uint64_t* d_keys, const uint32_t* d_beta,
+                      uint64_t n, uint64_t ctx, int packed_keys, uint32_t p)
+{
+    if (p < 1 || p > 32768u)
+        return fail(CSA_ERR_ARG, "%s: p = %u is outside [1, 32768]", who, p);
+    if (n > CSA_MAX_PART_SZ)
+        return fail(CSA_ERR_TOO_LARGE, "%s: %llu suffixes exceed a partition", who, (unsigned long long)n);
+    if (n && (!d_sa || !d_keys || !d_beta))
+        return fail(CSA_ERR_ARG, "%s: null buffer", who);
+    a.sa = d_sa;
+    a.keys = d_keys;
+    a.beta = d_beta;
+    a.n = n;
+    a.ctx = ctx;
+    a.packed = packed_keys ? 1 : 0;
+    a.active_sz = nullptr;
+    a.p = p;
+    a.msg_target = nullptr;
+    a.msg_rank = nullptr;
+    a.msg_off = nullptr;
+    a.tiles = (u32)((n + MSG_TILE - 1) / MSG_TILE);
+    return CSA_OK;
+}
+} // namespace
+
+int csa_count_messages_dev(const uint64_t* d_sa, const uint64_t* d_keys, const uint32_t* d_beta, uint64_t n, uint64_t ctx,
+                           int packed_keys, uint32_t p, uint32_t* d_msg_count, void* stream)
+{
+    MessageArgs a;
+    const int rc = fill_message_args(a, "csa_count_messages_dev", d_sa, d_keys, d_beta, n, ctx, packed_keys, p);
+    if (rc || n == 0)
+        return rc;
+    if (!d_msg_count)
+        return fail(CSA_ERR_ARG, "csa_count_messages_dev: null counters");
+    a.msg_off = d_msg_count;
+    hipLaunchKernelGGL(count_messages_kernel, dim3(a.tiles < 4096u ? a.tiles : 4096u), dim3(MSG_BLOCK), 0, (hipStream_t)stream, a);
+    HIP_TRY(hipGetLastError());
+    return CSA_OK;
+}
+
+int csa_message_offsets_dev(uint32_t* d_msg_off, uint32_t count, void* stream)
+{
+    if (count == 0)
+        return CSA_OK;
+    if (!d_msg_off || count > 32769u)
+        return fail(CSA_ERR_ARG, "csa_message_offsets_dev: null counters or more than 32769 of them");
+    hipLaunchKernelGGL(message_offsets_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, d_msg_off, count);
+    HIP_TRY(hipGetLastError());
+    return CSA_OK;
+}
+
+int csa_emit_messages_dev(const uint64_t* d_sa, const uint64_t* d_keys, const uint32_t* d_beta, uint64_t n, uint64_t ctx,
+                          int packed_keys, const uint64_t* d_active_sz, uint32_t p, uint8_t* d_msg_target,
+                          uint32_t* d_msg_rank, uint32_t* d_msg_off, void* stream)
+{
+    MessageArgs a;
+    const int rc = fill_message_args(a, "csa_emit_messages_dev", d_sa, d_keys, d_beta, n, ctx, packed_keys, p);
+    if (rc || n == 0)
+        return rc;
+    if (!d_active_sz || !d_msg_target || !d_msg_rank || !d_msg_off)
+        return fail(CSA_ERR_ARG, "csa_emit_messages_dev: null buffer");
+    a.active_sz = reinterpret_cast<const unsigned long long*>(d_active_sz);
+    a.msg_target = d_msg_target;
+    a.msg_rank = d_msg_rank;
+    a.msg_off = d_msg_off;
+    hipLaunchKernelGGL(emit_messages_kernel, dim3(a.tiles < 4096u ? a.tiles : 4096u), dim3(MSG_BLOCK), 0, (hipStream_t)stream, a);
+    HIP_TRY(hipGetLastError());
+    return CSA_OK;
+}
+
+int csa_join_messages_dev(const uint8_t* d_msg_target, const uint32_t* d_msg_rank, uint32_t msg_c, const uint64_t* d_sa,
+                          const uint32_t* d_primary, uint64_t* d_keys, uint64_t n, void* stream)
+{
+    if (msg_c == 0)
+        return CSA_OK;
+    if (!d_msg_target || !d_msg_rank || (n && (!d_sa || !d_primary || !d_keys)))
+        return fail(CSA_ERR_ARG, "csa_join_messages_dev: null buffer");
+    if (n > CSA_MAX_PART_SZ)
+        return fail(CSA_ERR_TOO_LARGE, "csa_join_messages_dev: %llu suffixes exceed a partition", (unsigned long long)n);
+    hipLaunchKernelGGL(join_messages_kernel, dim3((msg_c + 255u) / 256u), dim3(256), 0, (hipStream_t)stream, d_msg_target,
+                       d_msg_rank, msg_c, d_sa, d_primary, d_keys, n);
     HIP_TRY(hipGetLastError());
     return CSA_OK;
 }

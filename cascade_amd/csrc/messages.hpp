@@ -1,0 +1,211 @@
+// Rank-propagation messages between partitions, for partitions that are sorted one at a time and exchange ranks
+// through the host (the reference's scheme, README.md:26; kernels include/GPU_SACA.cuh:283-389). A partition whose
+// text and ranks are resident in HBM does not need them (it gathers rank[x + h] by text position); these kernels
+// serve the per-generation entry points that keep the reference's slab interface.
+//
+// At the end of a generation that resolved `ctx` symbols, every cohort member j (sorted list SA, keys K, routing
+// tags beta) sends
+//   its rank to j - ctx, via the partition in the low half of beta, unless j < ctx or the recipient has retired;
+//     the rank carries the poison-pill bit if j itself retired in this generation (list index >= *active_sz);
+//   and, if its own key had received a pill, the secondary of that key as a pill to j - ctx / 2, via the high half.
+// Messages are collated by destination: msg_off[q] must hold, before the emission, the exclusive prefix sum of the
+// per-destination counts, and holds the exclusive END of q's group afterwards. The order inside a group is arbitrary.
+#pragma once
+
+#include "device_utils.hpp"
+
+namespace csa {
+
+constexpr u64 MSG_VAL_MASK = (1ull << 48) - 1ull;    // suffix in a word (include/bit-layout.hpp:44,109)
+constexpr u64 MSG_PILL_RECEIPT = 1ull << 62;         // a key that received a pill (include/bit-layout.hpp:57)
+constexpr u32 MSG_PILL_BIT = 1u << 31;               // finality of a message's rank (include/message.hpp:22)
+constexpr u32 MSG_RETIRED = 0x8000u;                 // recipient retired, in a half of beta (include/bit-layout.hpp:135)
+constexpr int MSG_BLOCK = 256;
+constexpr int MSG_ITEMS = 4;
+constexpr int MSG_TILE = MSG_BLOCK * MSG_ITEMS;
+constexpr u32 MSG_LDS_PARTS = 2048; // destinations counted in LDS (more: one global atomic per message, as the reference)
+
+struct MessageArgs {
+    const u64* sa;
+    const u64* keys;
+    const u32* beta;
+    u64 n;
+    u64 ctx;
+    int packed; // keys are composite (primary << 31 | secondary, pill receipt in bit 62), not plain ranks
+    const unsigned long long* active_sz;
+    u32 p;
+    u8* msg_target;
+    u32* msg_rank;
+    u32* msg_off; // count kernel: per-destination counters to add to
+    u32 tiles;
+};
+
+struct Message {
+    u32 dest;   // 0xFFFFFFFF: none
+    u64 target;
+    u32 rank;
+};
+
+// the (at most) two messages of list element i (include/GPU_SACA.cuh:300-307, 334-352)
+__device__ __forceinline__ void messages_of(const MessageArgs& a, u64 i, u64 active_sz, Message& pay, Message& fwd)
+{
+    pay.dest = fwd.dest = 0xFFFFFFFFu;
+    const u64 j = a.sa[i] & MSG_VAL_MASK;
+    const u64 k = a.keys[i];
+    const u32 beta = a.beta[i];
+    if (j >= a.ctx && !(beta & MSG_RETIRED)) {
+        const u32 primary = a.packed ? (u32)((k >> 31) & 0x7FFFFFFFull) : (u32)k;
+        pay.dest = beta & 0xFFFFu;
+        pay.target = j - a.ctx;
+        pay.rank = i < active_sz ? primary : (primary | MSG_PILL_BIT);
+    }
+    if (a.packed && (k & MSG_PILL_RECEIPT) && j >= (a.ctx >> 1) && !((beta >> 16) & MSG_RETIRED)) {
+        fwd.dest = beta >> 16;
+        fwd.target = j - (a.ctx >> 1);
+        fwd.rank = (u32)(k & 0x7FFFFFFFull) | MSG_PILL_BIT;
+    }
+}
+
+// msg_off[q] += messages bound for partition q. Workgroups stride over the tiles and flush their LDS counters once.
+__global__ __launch_bounds__(MSG_BLOCK) void count_messages_kernel(MessageArgs a)
+{
+    __shared__ u32 s_cnt[MSG_LDS_PARTS];
+    const u32 t = threadIdx.x;
+    const bool lds = a.p <= MSG_LDS_PARTS;
+    if (lds)
+        for (u32 q = t; q < a.p; q += MSG_BLOCK)
+            s_cnt[q] = 0;
+    __syncthreads();
+    for (u32 tile = blockIdx.x; tile < a.tiles; tile += gridDim.x) {
+#pragma unroll
+        for (int k = 0; k < MSG_ITEMS; ++k) {
+            const u64 i = (u64)tile * MSG_TILE + (u64)k * MSG_BLOCK + t;
+            if (i >= a.n)
+                continue;
+            Message pay, fwd;
+            messages_of(a, i, ~0ull, pay, fwd); // the destinations do not depend on the active size
+            // a destination outside [0, p) would be a corrupt routing tag: not counted (and not emitted either)
+            if (pay.dest < a.p)
+                atomicAdd(lds ? &s_cnt[pay.dest] : &a.msg_off[pay.dest], 1u);
+            if (fwd.dest < a.p)
+                atomicAdd(lds ? &s_cnt[fwd.dest] : &a.msg_off[fwd.dest], 1u);
+        }
+    }
+    if (lds) {
+        __syncthreads();
+        for (u32 q = t; q < a.p; q += MSG_BLOCK)
+            if (s_cnt[q])
+                atomicAdd(&a.msg_off[q], s_cnt[q]);
+    }
+}
+
+// Writes the messages: a tile counts its messages per destination in LDS, reserves one range per destination with
+// a single global atomic, and its messages take consecutive slots of that range.
+__global__ __launch_bounds__(MSG_BLOCK) void emit_messages_kernel(MessageArgs a)
+{
+    __shared__ u32 s_cnt[MSG_LDS_PARTS];
+    __shared__ u32 s_base[MSG_LDS_PARTS];
+    const u32 t = threadIdx.x;
+    const bool lds = a.p <= MSG_LDS_PARTS;
+    const u64 active_sz = *a.active_sz;
+    for (u32 tile = blockIdx.x; tile < a.tiles; tile += gridDim.x) {
+        if (lds)
+            for (u32 q = t; q < a.p; q += MSG_BLOCK)
+                s_cnt[q] = 0;
+        __syncthreads();
+        Message m[2 * MSG_ITEMS];
+        u32 slot[2 * MSG_ITEMS];
+#pragma unroll
+        for (int k = 0; k < MSG_ITEMS; ++k) {
+            const u64 i = (u64)tile * MSG_TILE + (u64)k * MSG_BLOCK + t;
+            m[2 * k].dest = m[2 * k + 1].dest = 0xFFFFFFFFu;
+            if (i < a.n)
+                messages_of(a, i, active_sz, m[2 * k], m[2 * k + 1]);
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                Message& mm = m[2 * k + e];
+                if (mm.dest >= a.p)
+                    mm.dest = 0xFFFFFFFFu;
+                else
+                    slot[2 * k + e] = atomicAdd(lds ? &s_cnt[mm.dest] : &a.msg_off[mm.dest], 1u);
+            }
+        }
+        if (lds) {
+            __syncthreads();
+            for (u32 q = t; q < a.p; q += MSG_BLOCK)
+                if (s_cnt[q])
+                    s_base[q] = atomicAdd(&a.msg_off[q], s_cnt[q]);
+            __syncthreads();
+        }
+#pragma unroll
+        for (int e = 0; e < 2 * MSG_ITEMS; ++e) {
+            if (m[e].dest == 0xFFFFFFFFu)
+                continue;
+            const u64 s = (u64)slot[e] + (lds ? s_base[m[e].dest] : 0u);
+#pragma unroll
+            for (int b = 0; b < 5; ++b)
+                a.msg_target[5 * s + b] = (u8)(m[e].target >> (8 * b));
+            a.msg_rank[s] = m[e].rank;
+        }
+        __syncthreads(); // the counters are cleared for the next tile
+    }
+}
+
+// In-place exclusive prefix sum of `count` counters (count <= 32769: one per partition and one more), one workgroup.
+// Replaces cub::DeviceScan::ExclusiveSum over the p + 1 message counters (src/GPU_SACA.cu:1278-1283).
+__global__ __launch_bounds__(1024) void message_offsets_kernel(u32* v, u32 count)
+{
+    __shared__ u32 s_w[16];
+    const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
+    const u32 per = (count + 1023u) / 1024u;
+    const u32 first = t * per < count ? t * per : count;
+    const u32 last = first + per < count ? first + per : count;
+    u32 sum = 0;
+    for (u32 i = first; i < last; ++i)
+        sum += v[i];
+    const u32 incl = wave_incl_sum(sum);
+    if (lane == 63u)
+        s_w[w] = incl;
+    __syncthreads();
+    u32 run = incl - sum;
+    for (u32 ww = 0; ww < w; ++ww)
+        run += s_w[ww];
+    for (u32 i = first; i < last; ++i) {
+        const u32 c = v[i];
+        v[i] = run;
+        run += c;
+    }
+}
+
+// Delivers every message to its recipient in the suffix-ordered cohort SA[0, n): K[pos] = primary[pos] << 31 |
+// received rank, marked if the message is a pill; a recipient that is not in the cohort has retired and the
+// message is dropped (include/GPU_SACA.cuh:362-389).
+__global__ __launch_bounds__(256) void join_messages_kernel(const u8* __restrict__ msg_target, const u32* __restrict__ msg_rank,
+                                                            u32 msg_c, const u64* __restrict__ sa,
+                                                            const u32* __restrict__ primary, u64* keys, u64 n)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= msg_c)
+        return;
+    u64 tgt = 0;
+#pragma unroll
+    for (int b = 0; b < 5; ++b)
+        tgt |= (u64)msg_target[5 * i + b] << (8 * b);
+    u64 low = 0, high = n;
+    while (low < high) {
+        const u64 mid = low + (high - low) / 2;
+        if ((sa[mid] & MSG_VAL_MASK) < tgt)
+            low = mid + 1;
+        else
+            high = mid;
+    }
+    if (low == n || (sa[low] & MSG_VAL_MASK) != tgt)
+        return;
+    const u32 r = msg_rank[i];
+    u64 key = ((u64)primary[low] << 31) | (u64)(r & ~MSG_PILL_BIT);
+    if (r & MSG_PILL_BIT)
+        key |= MSG_PILL_RECEIPT;
+    keys[low] = key;
+}
+
+} // namespace csa

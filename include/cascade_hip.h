@@ -145,6 +145,36 @@ int csa_stage_slab_u16_dev(const uint16_t* d_text, uint64_t n, const uint8_t* d_
                            const uint64_t* d_pid_map, uint32_t p, uint64_t ctx, int generation0, uint64_t* d_keys,
                            uint32_t* d_beta, void* stream);
 
+/* ---- rank messages between partitions (for partitions sorted one at a time behind the reference's slab interface) ---- */
+
+/* At the end of a generation that resolved ctx symbols, cohort member i (suffix = low 48 bits of d_sa[i], key d_keys[i],
+ * routing tags d_beta[i]) sends its rank to suffix - ctx through the partition in the low half of beta, and forwards a
+ * received poison pill to suffix - ctx / 2 through the high half; packed_keys = 0: keys are plain ranks (generation 0),
+ * 1: primary << 31 | secondary with the pill receipt in bit 62.
+ * d_msg_count[q] += messages bound for partition q, q < p.
+ * Replaces count_message_destination_distribution_kernel (include/GPU_SACA.cuh:291-308; src/GPU_SACA.cu:1272-1276). */
+int csa_count_messages_dev(const uint64_t* d_sa, const uint64_t* d_keys, const uint32_t* d_beta, uint64_t n, uint64_t ctx,
+                           int packed_keys, uint32_t p, uint32_t* d_msg_count, void* stream);
+
+/* In-place exclusive prefix sum of `count` <= 32769 counters: the message counts become the groups' start offsets.
+ * Replaces the cub::DeviceScan::ExclusiveSum over p + 1 counters (src/GPU_SACA.cu:1278-1283). */
+int csa_message_offsets_dev(uint32_t* d_msg_off, uint32_t count, void* stream);
+
+/* Writes those messages, collated by destination: 5-byte target lanes to d_msg_target and ranks to d_msg_rank (MSB =
+ * the sender retired in this generation, i.e. its list index is >= *d_active_sz, or the message is a forwarded pill).
+ * d_msg_off[q] must hold the exclusive prefix sum of the counts on entry and holds the exclusive end of q's group on
+ * return; the order of messages inside a group is arbitrary.
+ * Replaces emit_messages_kernel (include/GPU_SACA.cuh:321-353; src/GPU_SACA.cu:1285-1287,1949-1951). */
+int csa_emit_messages_dev(const uint64_t* d_sa, const uint64_t* d_keys, const uint32_t* d_beta, uint64_t n, uint64_t ctx,
+                          int packed_keys, const uint64_t* d_active_sz, uint32_t p, uint8_t* d_msg_target,
+                          uint32_t* d_msg_rank, uint32_t* d_msg_off, void* stream);
+
+/* Delivers msg_c messages to the cohort d_sa[0, n), which is sorted by suffix: for the position pos of each target,
+ * d_keys[pos] = d_primary[pos] << 31 | rank, with bit 62 set for a pill; messages whose target is not in the cohort are
+ * dropped (the recipient has retired). Replaces join_messages_kernel (include/GPU_SACA.cuh:362-389; src/GPU_SACA.cu:1826-1833). */
+int csa_join_messages_dev(const uint8_t* d_msg_target, const uint32_t* d_msg_rank, uint32_t msg_c, const uint64_t* d_sa,
+                          const uint32_t* d_primary, uint64_t* d_keys, uint64_t n, void* stream);
+
 /* ---- the step after the partition sort, for partitions that come back as (suffix, local rank) pairs ---- */
 
 /* d_sa40 entry rank[i] = d_suf entry i for i in [0, part_sz): 5-byte little-endian lanes in, lanes in rank order out.

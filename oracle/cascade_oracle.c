@@ -502,3 +502,81 @@ void orc_stage_slab_u16(const uint16_t* T, uint64_t n, const uint8_t* suf40, uin
         beta[i] = ((uint32_t)prev << 16) | cur; /* include/bit-layout.hpp:137 */
     }
 }
+
+/* ---------- rank messages ---------- */
+
+#define ORC_VAL_MASK (((uint64_t)1 << 48) - 1)       /* include/bit-layout.hpp:44 */
+#define ORC_PILL_RECEIPT ((uint64_t)1 << 62)         /* include/bit-layout.hpp:57 */
+#define ORC_MSG_PILL ((uint32_t)1 << 31)             /* include/message.hpp:22 */
+#define ORC_BETA_RETIRED 0x8000u                     /* include/bit-layout.hpp:135 */
+
+void orc_messages_of(uint64_t sa_word, uint64_t key, uint32_t beta, uint64_t i, uint64_t active_sz, uint64_t ctx, int packed,
+                     uint64_t out[6])
+{
+    const uint64_t j = sa_word & ORC_VAL_MASK;
+    out[0] = out[3] = 0xFFFFFFFFu;
+    out[1] = out[2] = out[4] = out[5] = 0;
+    if (j >= ctx && !(beta & ORC_BETA_RETIRED)) { /* include/GPU_SACA.cuh:334 */
+        const uint32_t primary = packed ? (uint32_t)((key >> 31) & 0x7FFFFFFFu) : (uint32_t)key;
+        out[0] = beta & 0xFFFFu;
+        out[1] = j - ctx;
+        out[2] = i < active_sz ? primary : (primary | ORC_MSG_PILL); /* :342 */
+    }
+    if (packed && (key & ORC_PILL_RECEIPT) && j >= (ctx >> 1) && !((beta >> 16) & ORC_BETA_RETIRED)) { /* :345 */
+        out[3] = beta >> 16;
+        out[4] = j - (ctx >> 1);
+        out[5] = (uint32_t)(key & 0x7FFFFFFFu) | ORC_MSG_PILL; /* :349-351 */
+    }
+}
+
+void orc_count_messages(const uint64_t* sa, const uint64_t* keys, const uint32_t* beta, uint64_t n, uint64_t ctx, int packed,
+                        uint32_t* msg_count)
+{
+    uint64_t m[6];
+    for (uint64_t i = 0; i < n; ++i) {
+        /* the count kernel tests the pill receipt whatever the key kind (include/GPU_SACA.cuh:306); plain ranks never
+         * carry bit 62, so this is the same set of messages */
+        orc_messages_of(sa[i], keys[i], beta[i], i, ~(uint64_t)0, ctx, packed, m);
+        if (m[0] != 0xFFFFFFFFu)
+            msg_count[m[0]]++;
+        if (m[3] != 0xFFFFFFFFu)
+            msg_count[m[3]]++;
+    }
+}
+
+void orc_emit_messages(const uint64_t* sa, const uint64_t* keys, const uint32_t* beta, uint64_t n, uint64_t ctx, int packed,
+                       uint64_t active_sz, uint8_t* msg_target, uint32_t* msg_rank, uint32_t* msg_off)
+{
+    uint64_t m[6];
+    for (uint64_t i = 0; i < n; ++i) {
+        orc_messages_of(sa[i], keys[i], beta[i], i, active_sz, ctx, packed, m);
+        for (int e = 0; e < 2; ++e)
+            if (m[3 * e] != 0xFFFFFFFFu) {
+                const uint32_t slot = msg_off[m[3 * e]]++;
+                orc_sa40_store(msg_target, slot, m[3 * e + 1]);
+                msg_rank[slot] = (uint32_t)m[3 * e + 2];
+            }
+    }
+}
+
+void orc_join_messages(const uint8_t* msg_target, const uint32_t* msg_rank, uint32_t msg_c, const uint64_t* sa,
+                       const uint32_t* primary, uint64_t* keys, uint64_t n)
+{
+    for (uint32_t i = 0; i < msg_c; ++i) {
+        const uint64_t tgt = orc_sa40_load(msg_target, i) & ORC_VAL_MASK;
+        uint64_t low = 0, high = n;
+        while (low < high) { /* include/GPU_SACA.cuh:373-381 */
+            const uint64_t mid = low + (high - low) / 2;
+            if ((sa[mid] & ORC_VAL_MASK) < tgt)
+                low = mid + 1;
+            else
+                high = mid;
+        }
+        if (low == n || (sa[low] & ORC_VAL_MASK) != tgt)
+            continue; /* the recipient has retired */
+        uint64_t key = ((uint64_t)primary[low] << 31) | (msg_rank[i] & ~ORC_MSG_PILL);
+        if (msg_rank[i] & ORC_MSG_PILL)
+            key |= ORC_PILL_RECEIPT;
+        keys[low] = key;
+    }
+}

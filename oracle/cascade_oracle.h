@@ -106,6 +106,22 @@ void orc_stage_slab_u16(const uint16_t* T, uint64_t n, const uint8_t* suf40, uin
                         const uint16_t* pid, const uint8_t* retired, uint64_t ctx, int generation0, uint64_t* keys,
                         uint32_t* beta);
 
+/* ---- rank messages (include/GPU_SACA.cuh:283-389, include/message.hpp:20-52, include/bit-layout.hpp:57,115-152) ---- */
+
+/* The up to two messages of cohort member i: out = {dest, target, rank} of the payload, then of the forwarded pill;
+ * dest = 0xFFFFFFFF where there is none (include/GPU_SACA.cuh:334-352). */
+void orc_messages_of(uint64_t sa_word, uint64_t key, uint32_t beta, uint64_t i, uint64_t active_sz, uint64_t ctx, int packed,
+                     uint64_t out[6]);
+/* include/GPU_SACA.cuh:291-308: msg_count[q] += messages to partition q. */
+void orc_count_messages(const uint64_t* sa, const uint64_t* keys, const uint32_t* beta, uint64_t n, uint64_t ctx, int packed,
+                        uint32_t* msg_count);
+/* include/GPU_SACA.cuh:321-353, run sequentially: slot = msg_off[dest]++ in list order (payload before pill). */
+void orc_emit_messages(const uint64_t* sa, const uint64_t* keys, const uint32_t* beta, uint64_t n, uint64_t ctx, int packed,
+                       uint64_t active_sz, uint8_t* msg_target, uint32_t* msg_rank, uint32_t* msg_off);
+/* include/GPU_SACA.cuh:362-389. */
+void orc_join_messages(const uint8_t* msg_target, const uint32_t* msg_rank, uint32_t msg_c, const uint64_t* sa,
+                       const uint32_t* primary, uint64_t* keys, uint64_t n);
+
 /* ---- after the partition sort ---- */
 
 /* include/GPU_SACA.cuh:167-182 followed by :126-133: out lane[rank[i]] = lane i of suf (5-byte lanes, include/lane.hpp:51-79).

@@ -8,6 +8,7 @@
 #include "Packed_Prefix.hpp"  // gpu_saca::Packed_Prefix         (include/Packed_Prefix.hpp:91-104)
 #include "bit-layout.hpp"     // gpu_saca::bit_layout::fwd_tag   (include/bit-layout.hpp:99-100)
 #include "utility.hpp"        // gpu_saca::util::pack_word       (include/utility.hpp:147-162)
+#include "message.hpp"        // gpu_saca::poison_pill, extract_rank, is_poison_pill (include/message.hpp:40-52)
 #include "Partition_ID_Map.hpp" // gpu_saca::Partition_ID_Map::pack, bits_for (include/Partition_ID_Map.hpp:79,158-177)
 
 #include <cstring>
@@ -80,6 +81,39 @@ uint32_t ref_beta_u16(uint64_t j, uint64_t n, uint64_t ell, uint64_t ctx, int ge
     return bl::beta_pair(j < ctx ? 0 : bl::route(pid[j - ctx], retired[j - ctx] != 0),
                          generation0 ? bl::fwd_tag(id, j + ell, n, ell)
                                      : (j < stride ? 0 : bl::route(pid[j - stride], retired[j - stride] != 0)));
+}
+
+// The messages of one cohort member, put together with the reference's own bit helpers in the order of the emission
+// kernel (include/GPU_SACA.cuh:334-352): out = {dest, target, rank} of the payload, then of the forwarded pill;
+// dest = 0xFFFFFFFF where there is none.
+void ref_messages_of(uint64_t sa_word, uint64_t key, uint32_t beta, uint64_t i, uint64_t active_sz, uint64_t ctx, int packed,
+                     uint64_t* out)
+{
+    namespace bl = gpu_saca::bit_layout;
+    out[0] = out[3] = 0xFFFFFFFFu;
+    out[1] = out[2] = out[4] = out[5] = 0;
+    const auto j = bl::suffix_of(sa_word);
+    if(j >= ctx && !bl::beta_cur_retired(beta))
+    {
+        const gpu_saca::msg_rank_t primary = packed ? bl::primary_of(key) : key;
+        out[0] = bl::beta_cur_gen(beta);
+        out[1] = j - ctx;
+        out[2] = i < active_sz ? primary : gpu_saca::poison_pill(primary);
+    }
+    if(packed && bl::received_poison_pill(key) && j >= (ctx >> 1) && !bl::beta_prev_retired(beta))
+    {
+        out[3] = bl::beta_prev_gen(beta);
+        out[4] = j - (ctx >> 1);
+        out[5] = gpu_saca::poison_pill(static_cast<gpu_saca::msg_rank_t>(bl::secondary_of(key)));
+    }
+}
+
+// The key a delivered message leaves at its recipient (include/GPU_SACA.cuh:386-388).
+uint64_t ref_joined_key(uint32_t primary, uint32_t msg_rank)
+{
+    namespace bl = gpu_saca::bit_layout;
+    const auto key = bl::key(primary, gpu_saca::extract_rank(msg_rank));
+    return gpu_saca::is_poison_pill(msg_rank) ? bl::mark_poison_pill_receipt(key) : key;
 }
 
 }

@@ -60,6 +60,14 @@ def oracle():
         lib.orc_partition_id_map_get.argtypes = [vp, u32, u64]
         lib.orc_stage_slab_u16.restype = None
         lib.orc_stage_slab_u16.argtypes = [vp, u64, vp, u64, i32, vp, vp, u64, i32, vp, vp]
+        lib.orc_messages_of.restype = None
+        lib.orc_messages_of.argtypes = [u64, u64, u32, u64, u64, u64, i32, vp]
+        lib.orc_count_messages.restype = None
+        lib.orc_count_messages.argtypes = [vp, vp, vp, u64, u64, i32, vp]
+        lib.orc_emit_messages.restype = None
+        lib.orc_emit_messages.argtypes = [vp, vp, vp, u64, u64, i32, u64, vp, vp, vp]
+        lib.orc_join_messages.restype = None
+        lib.orc_join_messages.argtypes = [vp, vp, u32, vp, vp, vp, u64]
         lib.orc_scatter_to_rank_order.restype = i32
         lib.orc_scatter_to_rank_order.argtypes = [vp, vp, u64, vp]
         lib.orc_output_cut.restype = None
@@ -93,6 +101,10 @@ def ref():
         lib.ref_partition_id_bits.argtypes = [u32]
         lib.ref_partition_id_pack.restype = None
         lib.ref_partition_id_pack.argtypes = [vp, u64, u32, vp]
+        lib.ref_messages_of.restype = None
+        lib.ref_messages_of.argtypes = [u64, u64, u32, u64, u64, u64, i32, vp]
+        lib.ref_joined_key.restype = u64
+        lib.ref_joined_key.argtypes = [u32, u32]
         lib.ref_beta_u16.restype = u32
         lib.ref_beta_u16.argtypes = [u64, u64, u64, u64, i32, vp, vp]
         _ref = lib
@@ -273,3 +285,36 @@ def set_retired(words, bits, positions):
     for x in positions:
         bit = int(x) * bits + bits - 1
         words[bit // 64] |= np.uint64(1) << np.uint64(bit % 64)
+
+
+def count_messages(sa, keys, beta, ctx, packed, p):
+    sa, keys = np.ascontiguousarray(sa, dtype=np.uint64), np.ascontiguousarray(keys, dtype=np.uint64)
+    beta = np.ascontiguousarray(beta, dtype=np.uint32)
+    cnt = np.zeros(p + 1, dtype=np.uint32)
+    oracle().orc_count_messages(_ptr(sa), _ptr(keys), _ptr(beta), sa.size, int(ctx), 1 if packed else 0, _ptr(cnt))
+    return cnt
+
+
+def emit_messages(sa, keys, beta, ctx, packed, active_sz, p):
+    """(target uint64[total], rank uint32[total], end offsets uint32[p + 1]) with the groups in list order."""
+    sa, keys = np.ascontiguousarray(sa, dtype=np.uint64), np.ascontiguousarray(keys, dtype=np.uint64)
+    beta = np.ascontiguousarray(beta, dtype=np.uint32)
+    cnt = count_messages(sa, keys, beta, ctx, packed, p)
+    off = np.zeros(p + 1, dtype=np.uint32)
+    off[1:] = np.cumsum(cnt[:-1])
+    total = int(cnt.sum())
+    tgt = np.zeros(5 * max(total, 1), dtype=np.uint8)
+    rank = np.zeros(max(total, 1), dtype=np.uint32)
+    oracle().orc_emit_messages(_ptr(sa), _ptr(keys), _ptr(beta), sa.size, int(ctx), 1 if packed else 0, int(active_sz), _ptr(tgt),
+                               _ptr(rank), _ptr(off))
+    return sa40_to_u64(tgt)[:total], rank[:total], off
+
+
+def join_messages(msg_target, msg_rank, sa, primary, keys):
+    lanes = u64_to_sa40(np.ascontiguousarray(msg_target, dtype=np.uint64))
+    msg_rank = np.ascontiguousarray(msg_rank, dtype=np.uint32)
+    sa = np.ascontiguousarray(sa, dtype=np.uint64)
+    primary = np.ascontiguousarray(primary, dtype=np.uint32)
+    keys = np.array(keys, dtype=np.uint64, copy=True)
+    oracle().orc_join_messages(_ptr(lanes), _ptr(msg_rank), msg_rank.size, _ptr(sa), _ptr(primary), _ptr(keys), sa.size)
+    return keys

@@ -30,6 +30,10 @@ def emu():
     lib.csa_partition_ids_u16_dev.argtypes = [vp, u64, u64, vp, i32, u32, vp, vp, vp, vp]
     lib.csa_stage_slab_u16_dev.argtypes = [vp, u64, vp, u64, i32, vp, u32, u64, i32, vp, vp, vp]
     lib.csa_scatter_to_rank_order_dev.argtypes = [vp, vp, vp, u64, vp, vp]
+    lib.csa_count_messages_dev.argtypes = [vp, vp, vp, u64, u64, i32, u32, vp, vp]
+    lib.csa_message_offsets_dev.argtypes = [vp, u32, vp]
+    lib.csa_emit_messages_dev.argtypes = [vp, vp, vp, u64, u64, i32, vp, u32, vp, vp, vp, vp]
+    lib.csa_join_messages_dev.argtypes = [vp, vp, u32, vp, vp, vp, u64, vp]
     return lib
 
 
@@ -151,3 +155,34 @@ def test_emulated_slab_staging_and_rank_order_scatter(emu, generation0, ctx, key
     rc = emu.csa_scatter_to_rank_order_dev(h, lanes.ctypes.data, rank.ctypes.data, suf.size, out.ctypes.data, None)
     emu.csa_destroy(h)
     assert rc == 0 and np.array_equal(out, oracle_lib.scatter_to_rank_order(lanes, rank)[1])
+
+
+class HostArray:
+    """In the emulation "device" memory is host memory: the arrays stand for themselves."""
+
+    def __init__(self, a):
+        self.a = a
+        self.ptr = a.ctypes.data
+
+
+@pytest.mark.parametrize("packed,ctx,n,p", [(False, 4, 3000, 5), (True, 8, 3000, 300), (True, 64, 1500, 2049)])
+def test_emulated_message_kernels_match_the_oracle(emu, packed, ctx, n, p):
+    import test_gpu_messages
+    test_gpu_messages.check_messages(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a.copy(), n, p, ctx, packed,
+                                     seed=n + p)
+
+
+def test_emulated_join_matches_the_oracle(emu):
+    rng = np.random.default_rng(4)
+    n = 2000
+    suf = np.sort(rng.choice(1 << 20, n, replace=False)).astype(np.uint64)
+    sa = suf | (rng.integers(0, 1 << 16, n).astype(np.uint64) << np.uint64(48))
+    primary = rng.integers(0, 1 << 31, n).astype(np.uint32)
+    tgt = np.concatenate([suf[rng.choice(n, 700, replace=False)], np.setdiff1d(rng.integers(0, 1 << 20, 200).astype(np.uint64), suf)])
+    rank = rng.integers(0, 1 << 32, tgt.size, dtype=np.uint64).astype(np.uint32)
+    seed_keys = np.full(n, np.uint64(0xFFFFFFFFFFFFFFFF))
+    keys = seed_keys.copy()
+    lanes = oracle_lib.u64_to_sa40(tgt)
+    assert emu.csa_join_messages_dev(lanes.ctypes.data, rank.ctypes.data, tgt.size, sa.ctypes.data, primary.ctypes.data,
+                                     keys.ctypes.data, n, None) == 0
+    assert np.array_equal(keys, oracle_lib.join_messages(tgt, rank, sa, primary, seed_keys))
