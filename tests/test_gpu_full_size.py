@@ -1,0 +1,41 @@
+"""The benchmark configurations at their full sizes, through the C ABI, checked by properties that do not need the CPU
+oracle to finish: the device verifier (permutation + every adjacent pair in order, the reference's rule of
+test/end-to-end.cpp:46-80) accepts the result and rejects it after one swap; the entries sum to n (n - 1) / 2; the
+number of generations and the active counts are those of a second, independent run."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.timeout(300)
+@pytest.mark.parametrize("config", [2, 3, 5, 4])
+def test_full_size_configuration_sorts_to_a_verified_suffix_array(config):
+    import torch
+    from cascade_amd import PartitionSorter, workloads
+    n = workloads.default_n(config)
+    print(f"  full size C{config} n={n}", flush=True)
+    T = workloads.generate(config, n)
+    d_text = torch.from_numpy(T.view(np.int16)).cuda()
+    del T
+    s = PartitionSorter(n, key_words=1)
+    try:
+        out = s.sort(d_text)
+        stats = s.last_stats
+        assert s.verify(d_text, out)
+        # permutation by another route: 40-bit entries, little-endian, sum = n (n - 1) / 2
+        b = out.view(n, 5).to(torch.int64)
+        total = int(b[:, 0].sum()) + (int(b[:, 1].sum()) << 8) + (int(b[:, 2].sum()) << 16) + (int(b[:, 3].sum()) << 24) + (
+            int(b[:, 4].sum()) << 32)
+        del b
+        assert total == n * (n - 1) // 2
+        # one swap of two neighbouring entries (distinct suffixes, so the order breaks) must be caught
+        r = n // 3
+        e0, e1 = out[5 * r:5 * r + 5].clone(), out[5 * r + 5:5 * r + 10].clone()
+        out[5 * r:5 * r + 5], out[5 * r + 5:5 * r + 10] = e1, e0
+        assert not s.verify(d_text, out)
+        out2 = s.sort(d_text)
+        assert s.last_stats["active"] == stats["active"] and s.last_stats["generations"] == stats["generations"]
+        assert s.verify(d_text, out2)
+    finally:
+        s.close()
