@@ -125,6 +125,118 @@ def bench_partition_ids(args):
         sys.exit(1)
 
 
+def _row_result(metric, workload, n, ms, kernel, alg_bytes, extra, steps, warmup, ok):
+    return {
+        "metric": metric, "value": n / (ms * 1e-3), "unit": "suffixes/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u64 / u32 integers",
+        "data": "synthetic", "config": dict({"workload": workload, "n": n, "checked_against_oracle": ok}, **extra),
+        "roofline": {"bound": "hbm", "kernel": kernel, "achieved": round(alg_bytes / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(alg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                     "avg_launch_ms": round(ms, 4), "algorithmic_bytes_per_launch": round(alg_bytes)},
+    }
+
+
+def _timed(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    torch.cuda.synchronize()
+    ev[0].record()
+    for _ in range(steps):
+        out = fn()
+    ev[1].record()
+    torch.cuda.synchronize()
+    return ev[0].elapsed_time(ev[1]) / steps, out
+
+
+def bench_next_rows(args):
+    """The steps either side of the partition sort that exist for partitions exchanged with the host: slab staging
+    (keys + routing tags from the text and the packed partition-id map), message count / offsets / emission, the join,
+    and the rank-order scatter. One step = one launch sequence over a synthetic partition of n suffixes in HBM."""
+    import ctypes as C
+    import numpy as np
+    import torch
+    import oracle_lib
+    import message_cases
+    from cascade_amd import PartitionSorter, _native, partition_ids, stage_slab, workloads
+    lib = _native.load()
+    dev = torch.device("cuda:0")
+    n = args.n if args.n is not None else 1 << 28
+    p = args.partitions
+    rng = np.random.default_rng(2)
+    cs = 1 << 20  # the slice every row is checked on against the oracle
+    if args.row == "stage_slab":
+        T = workloads.generate(args.config, n)
+        pivots = oracle_lib.sample_pivots(T[:1 << 22], p, 2, rng)
+        d_text = torch.from_numpy(T.view(np.int16)).to(dev)
+        ids, packed, _ = partition_ids(d_text, torch.from_numpy(pivots.view(np.int64)).to(dev).reshape(-1, 2), p)
+        suf = torch.randperm(n, device=dev)  # a partition's suffixes arrive in no particular text order
+        lanes = torch.stack([(suf >> (8 * b)) & 0xFF for b in range(5)], dim=1).to(torch.uint8).reshape(-1).contiguous()
+        ms, (keys, beta) = _timed(torch, lambda: stage_slab(d_text, lanes, 1, packed, p, 4, True), args.steps, args.warmup)
+        pid = ids[: n].cpu().numpy().view(np.uint16)
+        h_suf = suf[:cs].cpu().numpy().astype(np.uint64)
+        wk, wb = oracle_lib.stage_slab(T, h_suf, 1, pid, np.zeros(n, dtype=np.uint8), 4, True)
+        ok = bool(np.array_equal(keys[:cs].cpu().numpy().view(np.uint64), wk) and np.array_equal(beta[:cs].cpu().numpy().view(np.uint32), wb))
+        res = _row_result("suffixes staged/sec at 1 GPU", workloads.NAMES[args.config], n, ms, "stage_slab_kernel<1>",
+                          n * (5 + 8 + 8 + 4), {"partitions": p, "key_words": 1, "generation": 0}, args.steps, args.warmup, ok)
+    elif args.row == "messages":
+        ctx = 1 << 12
+        sa, keys, beta, active_sz = message_cases.cohort(n, p, ctx, True, seed=5)
+        d_sa, d_keys = torch.from_numpy(sa.view(np.int64)).to(dev), torch.from_numpy(keys.view(np.int64)).to(dev)
+        d_beta = torch.from_numpy(beta.view(np.int32)).to(dev)
+        d_act = torch.tensor([active_sz], dtype=torch.int64, device=dev)
+        d_off = torch.zeros(p + 1, dtype=torch.int32, device=dev)
+        d_tgt = torch.empty(5 * 2 * n, dtype=torch.uint8, device=dev)
+        d_rank = torch.empty(2 * n, dtype=torch.int32, device=dev)
+        st = torch.cuda.current_stream(dev).cuda_stream
+
+        def run():
+            d_off.zero_()
+            _native.check(lib.csa_count_messages_dev(d_sa.data_ptr(), d_keys.data_ptr(), d_beta.data_ptr(), n, ctx, 1, p, d_off.data_ptr(), st))
+            _native.check(lib.csa_message_offsets_dev(d_off.data_ptr(), p + 1, st))
+            _native.check(lib.csa_emit_messages_dev(d_sa.data_ptr(), d_keys.data_ptr(), d_beta.data_ptr(), n, ctx, 1, d_act.data_ptr(), p,
+                                                    d_tgt.data_ptr(), d_rank.data_ptr(), d_off.data_ptr(), st))
+        ms, _ = _timed(torch, run, args.steps, args.warmup)
+        end = d_off.cpu().numpy().view(np.uint32)
+        total = int(end[p - 1])
+        want = oracle_lib.count_messages(sa, keys, beta, ctx, True, p)
+        ok = bool(np.array_equal(np.diff(np.concatenate([[0], end[:p]])), want[:p]))
+        res = _row_result("cohort members whose messages are emitted/sec at 1 GPU", "random cohort, 20% retired recipients, 30% pill receipts",
+                          n, ms, "count_messages_kernel + emit_messages_kernel", 2 * n * 20 + total * 9,
+                          {"partitions": p, "messages": total}, args.steps, args.warmup, ok)
+    elif args.row == "join":
+        suf = torch.sort(torch.randperm(1 << 31, device=dev)[:n]).values if n <= (1 << 27) else torch.arange(n, device=dev) * 3
+        msg_c = n // 2
+        pick = torch.randperm(n, device=dev)[:msg_c]
+        tgt = suf[pick]
+        lanes = torch.stack([(tgt >> (8 * b)) & 0xFF for b in range(5)], dim=1).to(torch.uint8).reshape(-1).contiguous()
+        rank = torch.randint(0, 1 << 31, (msg_c,), dtype=torch.int32, device=dev)
+        primary = torch.randint(0, 1 << 31, (n,), dtype=torch.int32, device=dev)
+        keys = torch.full((n,), -1, dtype=torch.int64, device=dev)
+        st = torch.cuda.current_stream(dev).cuda_stream
+        ms, _ = _timed(torch, lambda: _native.check(lib.csa_join_messages_dev(lanes.data_ptr(), rank.data_ptr(), msg_c, suf.data_ptr(),
+                                                                               primary.data_ptr(), keys.data_ptr(), n, st)), args.steps, args.warmup)
+        want = (primary[pick].to(torch.int64) << 31) | rank.to(torch.int64)
+        ok = bool(torch.equal(keys[pick], want))
+        res = _row_result("messages joined/sec at 1 GPU", "messages for half of a suffix-ordered cohort", msg_c, ms, "join_messages_kernel",
+                          msg_c * (9 + 8 + 4 + 8), {"cohort": n}, args.steps, args.warmup, ok)
+    else:  # scatter
+        rank = torch.randperm(n, device=dev).to(torch.int32)
+        lanes = torch.randint(0, 256, (5 * n,), dtype=torch.uint8, device=dev)
+        s = PartitionSorter(16)
+        out = torch.empty(5 * n + 128, dtype=torch.uint8, device=dev)
+        ms, _ = _timed(torch, lambda: s.scatter_to_rank_order(lanes, rank, out=out), args.steps, args.warmup)
+        h_rank = rank[:cs].cpu().numpy().view(np.uint32).astype(np.int64)
+        got = out[:5 * n].view(n, 5)[torch.from_numpy(h_rank).to(dev)].cpu().numpy()
+        ok = bool(np.array_equal(got, lanes[:5 * cs].view(cs, 5).cpu().numpy()))
+        s.close()
+        res = _row_result("suffixes scattered to rank order/sec at 1 GPU", "random permutation of ranks", n, ms, "scatter_lanes_kernel",
+                          n * 14, {}, args.steps, args.warmup, ok)
+    print(json.dumps(res), flush=True)
+    if not res["config"]["checked_against_oracle"]:
+        sys.exit(1)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -136,8 +248,8 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=1 << 26, help="symbols of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--generations", action="store_true", help="print the per-generation table to stderr")
-    ap.add_argument("--row", default="sort", choices=["sort", "partition_ids"],
-                    help="which step to measure: the partition sort (the headline) or the partition-id step before it")
+    ap.add_argument("--row", default="sort", choices=["sort", "partition_ids", "stage_slab", "messages", "join", "scatter"],
+                    help="which step to measure: the partition sort (the headline, default) or one of the steps around it")
     ap.add_argument("--partitions", type=int, default=256, help="partitions of --row partition_ids")
     args = ap.parse_args()
 
@@ -153,6 +265,8 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     if args.row == "partition_ids":
         return bench_partition_ids(args)
+    if args.row != "sort":
+        return bench_next_rows(args)
     dev = torch.device("cuda:0")
     n = args.n if args.n is not None else workloads.default_n(args.config)
 
