@@ -498,7 +498,8 @@ int windowed_rank_update(Launch& L, const u32* pos, const DeferBuffers& buf, u32
 // Ranks the sorted list described by `ra`: counts per tile, scans the counts, reads the totals back (the one
 // host round trip of the step: the next list's size decides the launches that follow), then applies them and
 // brings rank[] up to date, directly from the kernel or through one of the bucketed updates.
-int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivors, u32* groups, int* rank_update)
+int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivors, u32* groups, int* rank_update,
+                bool expect_no_big)
 {
     csa_handle* h = L.h;
     hipStream_t s = L.stream;
@@ -517,9 +518,12 @@ int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivo
     HIP_TRY(hipGetLastError());
     u32* h_slabs = h->h_pinned + 16;
     HIP_TRY(hipMemcpyAsync(h_slabs, ra.slab_total, slabs * 5 * sizeof(u32), hipMemcpyDeviceToHost, s));
-    int rc = read_counts(L, nullptr);
+    u32 big_seen = 0;
+    int rc = read_counts(L, &big_seen);
     if (rc)
         return rc;
+    if (expect_no_big && big_seen != 0) // groups only split; a large group after an all-small generation is a corrupt list
+        return fail(CSA_ERR_INTERNAL, "%u members of large groups appeared after a generation without any", big_seen);
     u64 surv = 0, heads = 0, changed = 0;
     for (u32 sl = 0; sl < slabs; ++sl) {
         surv += h_slabs[sl * 5 + 2];
@@ -616,7 +620,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     const DeferBuffers defer_buf = {bx[0], bx[1], reinterpret_cast<u32*>(bkey[0]), reinterpret_cast<u32*>(bkey[1]),
                                     reinterpret_cast<u32*>(bkey[1]) + h->cap};
     u32 m = 0, groups = 0, big = 0;
-    rc = rerank_step(L, ra, defer_buf, &m, &groups, &st->rank_update[0]);
+    rc = rerank_step(L, ra, defer_buf, &m, &groups, &st->rank_update[0], false);
     if (rc)
         return rc;
     st->passes[0] = passes;
@@ -627,6 +631,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     // ---- generations t >= 1 (reference loop: src/GPU_SACA.cu:1999-2103) ----
     int gen = 1;
     int gp = 0; // gprim[gp] / gstart[gp] describe the current groups
+    bool all_small = false; // no group of the current list exceeds SMALL_MAXG members
     const int sec_bits = bit_length(n > 1 ? n - 1 : 1);
     u64 h_ctx = ell;
     while (m > 0) {
@@ -655,9 +660,14 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
         hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG>),
                            dim3((m + SMALL_TILE - 1) / SMALL_TILE), dim3(SMALL_BLOCK), 0, s, sa);
         HIP_TRY(hipGetLastError());
-        rc = read_counts(L, &big);
-        if (rc)
-            return rc;
+        // Groups only ever split: once a generation had no large group, none can appear again, and the host need
+        // not wait for the count (the error word is still read at the rank step's round trip).
+        if (!all_small) {
+            rc = read_counts(L, &big);
+            if (rc)
+                return rc;
+            all_small = big == 0;
+        }
         st->big[gen] = big;
         passes = 0;
         if (big > 0) {
@@ -704,7 +714,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
         ra.gids_out = agid;
         ra.gprim_out = h->gprim[gp ^ 1];
         ra.gstart_out = h->gstart[gp ^ 1];
-        rc = rerank_step(L, ra, defer_buf, &m, &groups, &st->rank_update[gen]);
+        rc = rerank_step(L, ra, defer_buf, &m, &groups, &st->rank_update[gen], all_small && big == 0);
         if (rc)
             return rc;
         gp ^= 1;
