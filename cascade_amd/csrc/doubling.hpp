@@ -501,10 +501,14 @@ __global__ __launch_bounds__(BLOCK) void smallsort_kernel(SmallSortArgs a)
             s_sec[MAXG + k * BLOCK + t] = sec[k];
         }
     }
+    // A halo element matters only if its group reaches into the tile, i.e. if it shares the group of the tile's
+    // first (left halo) or last (right halo) element; the others would be random reads for nothing.
+    const long long last_own = t0 + TILE - 1 < (long long)a.m - 1 ? t0 + TILE - 1 : (long long)a.m - 1;
+    const u32 gid_first = a.gids[t0], gid_last = a.gids[last_own];
     for (int i = t; i < 2 * MAXG; i += BLOCK) {
         const int slot = i < MAXG ? i : TILE + i; // [0, MAXG) and [MAXG + TILE, SPAN)
         const long long e = lo + slot;
-        if (e >= 0 && e < (long long)a.m) {
+        if (e >= 0 && e < (long long)a.m && a.gids[e] == (i < MAXG ? gid_first : gid_last)) {
             const u64 src = (u64)a.sufs[e] + a.h;
             s_sec[slot] = src < a.n ? a.rank[src] : 0u;
         }
