@@ -244,4 +244,28 @@ def test_sixteen_million_symbols_pass_the_oracle_verifier(torch_mod, config):
         torch_mod.cuda.synchronize()
         assert s.verify(d, out)
         got = out.cpu().numpy()
+        how = s.last_stats["rank_update"]
     assert oracle_lib.is_correct_sa40(got, T)
+    assert how[0] == 1  # generation 0 went through the two-pass bucketed rank update
+    if config == 4:     # four letters: nearly every rank changes in generation 1, which takes the one-pass kind
+        assert 2 in how[1:] and 0 in how[1:]
+
+
+def test_random_small_texts_against_the_oracle(torch_mod):
+    """Many short texts over tiny alphabets (long ties, groups that straddle tiles, tails of zeros), both key widths,
+    on exact-size handles: byte-equal to the oracle's comparison sort."""
+    from cascade_amd import PartitionSorter
+    rng = np.random.default_rng(2024)
+    for case in range(120):
+        n = int(rng.integers(1, 6000))
+        sigma = int(rng.integers(1, 5))
+        T = rng.integers(0, sigma, n).astype(np.uint16)
+        if case % 3 == 0:
+            T[-int(rng.integers(1, min(n, 40) + 1)):] = 0
+        if case % 4 == 1 and n > 600:
+            T[n // 2:n // 2 + 256] = T[:256]  # a long repeat
+        kw = 1 + case % 2
+        with PartitionSorter(n, key_words=kw) as s:
+            print(f"  random case={case} n={n} sigma={sigma} key_words={kw}", flush=True)
+            got = s.sort(to_dev(torch_mod, T)).cpu().numpy()
+        assert np.array_equal(got, oracle_lib.build_sa40(T)), (case, n, sigma, kw)
