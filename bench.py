@@ -318,7 +318,7 @@ def main():
     gen_table = []
     for g in range(st["generations"]):
         gbs = per_gen[g] / (st["ms"][g] * 1e-3) / 1e9 if st["ms"][g] > 0 else 0.0
-        gen_table.append({"g": g, "active": st["active"][g], "groups": st["groups"][g], "big": st["big"][g], "passes": st["passes"][g], "rank_update": st["rank_update"][g],
+        gen_table.append({"g": g, "active": st["active"][g], "groups": st["groups"][g], "big": st["big"][g], "passes": st["passes"][g], "rank_update": st["rank_update"][g], "small_only": st["small_only"][g],
                           "ms": round(st["ms"][g], 3), "alg_GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4)})
     if args.generations:
         for row in gen_table:

@@ -34,6 +34,7 @@ class CsaStats(C.Structure):
         ("big", C.c_uint64 * CSA_MAX_GENERATIONS),
         ("passes", C.c_int32 * CSA_MAX_GENERATIONS),
         ("rank_update", C.c_int32 * CSA_MAX_GENERATIONS),
+        ("small_only", C.c_int32 * CSA_MAX_GENERATIONS),
         ("ms", C.c_float * CSA_MAX_GENERATIONS),
         ("ms_output", C.c_float),
         ("ms_total", C.c_float),

@@ -343,9 +343,10 @@ int read_counts(Launch& L, u32* big)
         static const char* const what[] = {"", "a look-back wait ran into its spin limit",
                                            "an active suffix lies outside its group's range (small-group sort)",
                                            "a large-group member was sent outside the active list (place)",
-                                           "a rank or suffix index out of range in the sorted active list (rerank)"};
+                                           "a rank or suffix index out of range in the sorted active list (rerank)",
+                                           "a large group appeared in a list whose groups were all small"};
         const u32 code = h->h_pinned[2];
-        return fail(CSA_ERR_INTERNAL, "device invariant %u failed: %s", code, code < 5 ? what[code] : "unknown");
+        return fail(CSA_ERR_INTERNAL, "device invariant %u failed: %s", code, code < 6 ? what[code] : "unknown");
     }
     if (big)
         *big = h->h_pinned[4];
@@ -495,29 +496,38 @@ int windowed_rank_update(Launch& L, const u32* pos, const DeferBuffers& buf, u32
     return CSA_OK;
 }
 
-// Ranks the sorted list described by `ra`: counts per tile, scans the counts, reads the totals back (the one
-// host round trip of the step: the next list's size decides the launches that follow), then applies them and
-// brings rank[] up to date, directly from the kernel or through one of the bucketed updates.
-int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivors, u32* groups, int* rank_update,
-                bool expect_no_big)
+// Sizes of the rank step's tables for a list of m suffixes cut into tiles of `tile` elements.
+struct RankTables {
+    u32 tiles, slab, slabs;
+    u32 *tile_agg, *tile_prefix, *tile_splits, *slab_total;
+};
+
+RankTables rank_tables(csa_handle* h, u32 m, u32 tile)
+{
+    RankTables r;
+    r.tiles = (u32)(((u64)m + tile - 1) / tile);
+    r.slab = (r.tiles + RERANK_SLABS - 1) / RERANK_SLABS;
+    r.slabs = (r.tiles + r.slab - 1) / r.slab;
+    r.tile_agg = h->tile_tables;
+    r.tile_prefix = h->tile_tables + (u64)h->rank_tiles_cap * 4;
+    r.tile_splits = h->tile_tables + (u64)h->rank_tiles_cap * 8;
+    r.slab_total = h->tile_tables + (u64)h->rank_tiles_cap * 9;
+    return r;
+}
+
+// Scans the per-tile counts, reads the totals back (the one host round trip of the step: the next list's size
+// decides the launches that follow) and chooses how the ranks are written: 0 scattered by the applying kernel,
+// 1 two-pass bucketed (generation 0 of large partitions), 2 one-pass bucketed (most of a later list changed).
+int rank_totals(Launch& L, const RankTables& r, bool gen0, u32 m, u32 n, bool expect_no_big, u32* survivors, u32* groups,
+                int* rank_update)
 {
     csa_handle* h = L.h;
     hipStream_t s = L.stream;
-    const u32 tiles = (u32)(((u64)ra.m + RANK_TILE - 1) / RANK_TILE);
-    ra.tile_agg = h->tile_tables;
-    ra.tile_prefix = h->tile_tables + (u64)h->rank_tiles_cap * 4;
-    ra.tile_splits = h->tile_tables + (u64)h->rank_tiles_cap * 8;
-    ra.slab_total = h->tile_tables + (u64)h->rank_tiles_cap * 9;
-    ra.slab = (tiles + RERANK_SLABS - 1) / RERANK_SLABS;
-    ra.err = h->counts + 2;
-    ra.rank_vals = nullptr;
-    const u32 slabs = (tiles + ra.slab - 1) / ra.slab;
-    hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS, false>), dim3(tiles), dim3(RANK_BLOCK), 0, s, ra);
-    hipLaunchKernelGGL(rerank_scan_kernel, dim3(slabs), dim3(1024), 0, s, ra.tile_agg, ra.tile_prefix, tiles, ra.slab,
-                       ra.slab_total, ra.tile_splits);
+    hipLaunchKernelGGL(rerank_scan_kernel, dim3(r.slabs), dim3(1024), 0, s, r.tile_agg, r.tile_prefix, r.tiles, r.slab,
+                       r.slab_total, r.tile_splits);
     HIP_TRY(hipGetLastError());
     u32* h_slabs = h->h_pinned + 16;
-    HIP_TRY(hipMemcpyAsync(h_slabs, ra.slab_total, slabs * 5 * sizeof(u32), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipMemcpyAsync(h_slabs, r.slab_total, r.slabs * 5 * sizeof(u32), hipMemcpyDeviceToHost, s));
     u32 big_seen = 0;
     int rc = read_counts(L, &big_seen);
     if (rc)
@@ -525,7 +535,7 @@ int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivo
     if (expect_no_big && big_seen != 0) // groups only split; a large group after an all-small generation is a corrupt list
         return fail(CSA_ERR_INTERNAL, "%u members of large groups appeared after a generation without any", big_seen);
     u64 surv = 0, heads = 0, changed = 0;
-    for (u32 sl = 0; sl < slabs; ++sl) {
+    for (u32 sl = 0; sl < r.slabs; ++sl) {
         surv += h_slabs[sl * 5 + 2];
         heads += h_slabs[sl * 5 + 3];
         changed += h_slabs[sl * 5 + 4];
@@ -535,17 +545,38 @@ int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivo
     // Generation 0 ranks every suffix of the partition: on large partitions the n scattered writes go through the
     // two-pass bucketed update. Later generations write only the ranks that changed; when those are many and the
     // partition is larger than one window, they go through the one-pass bucketed update.
-    const bool defer0 = ra.gen0 && ra.m >= h->defer_min;
-    const bool windowed = !ra.gen0 && bit_length(ra.n - 1) > WINDOW_LOG2 && changed >= h->window_min_changed &&
-                          changed >= ra.m / 2;
-    if (defer0 || windowed)
-        ra.rank_vals = buf.vals;
+    const bool defer0 = gen0 && m >= h->defer_min;
+    const bool windowed = !gen0 && bit_length(n - 1) > WINDOW_LOG2 && changed >= h->window_min_changed && changed >= m / 2;
     *rank_update = defer0 ? 1 : windowed ? 2 : 0;
-    hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS, true>), dim3(tiles), dim3(RANK_BLOCK), 0, s, ra);
+    return CSA_OK;
+}
+
+// Ranks the sorted list described by `ra`: counts per tile, scans the counts, reads the totals back, then applies them
+// and brings rank[] up to date, directly from the kernel or through one of the bucketed updates.
+int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivors, u32* groups, int* rank_update,
+                bool expect_no_big)
+{
+    csa_handle* h = L.h;
+    hipStream_t s = L.stream;
+    const RankTables r = rank_tables(h, ra.m, RANK_TILE);
+    ra.tile_agg = r.tile_agg;
+    ra.tile_prefix = r.tile_prefix;
+    ra.tile_splits = r.tile_splits;
+    ra.slab_total = r.slab_total;
+    ra.slab = r.slab;
+    ra.err = h->counts + 2;
+    ra.rank_vals = nullptr;
+    hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS, false>), dim3(r.tiles), dim3(RANK_BLOCK), 0, s, ra);
+    int rc = rank_totals(L, r, ra.gen0 != 0, ra.m, ra.n, expect_no_big, survivors, groups, rank_update);
+    if (rc)
+        return rc;
+    if (*rank_update != 0)
+        ra.rank_vals = buf.vals;
+    hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS, true>), dim3(r.tiles), dim3(RANK_BLOCK), 0, s, ra);
     HIP_TRY(hipGetLastError());
-    if (defer0)
+    if (*rank_update == 1)
         return deferred_rank_update(L, ra.sufs, buf, ra.n);
-    if (windowed)
+    if (*rank_update == 2)
         return windowed_rank_update(L, ra.sufs, buf, ra.m, ra.n);
     return CSA_OK;
 }
@@ -639,84 +670,144 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
             return fail(CSA_ERR_INTERNAL, "generation cap reached with %u suffixes still active", m);
         st->active[gen] = m;
         st->groups[gen] = groups;
-        // small groups are sorted in place by one kernel; the members of large groups are set aside
-        HIP_TRY(hipMemsetAsync(h->counts + 4, 0, sizeof(u32), s));
-        SmallSortArgs sa;
-        sa.sufs = ax;
-        sa.gids = agid;
-        sa.gstart = h->gstart[gp];
-        sa.rank = h->rank;
-        sa.m = m;
-        sa.n = n;
-        sa.h = (u32)h_ctx;
-        sa.sec_bits = sec_bits;
-        sa.groups = groups;
-        sa.err = h->counts + 2;
-        sa.keys_out = key_out;
-        sa.sufs_out = x_out;
-        sa.big_keys = bkey[0];
-        sa.big_sufs = bx[0];
-        sa.big_count = h->counts + 4;
-        hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG>),
-                           dim3((m + SMALL_TILE - 1) / SMALL_TILE), dim3(SMALL_BLOCK), 0, s, sa);
-        HIP_TRY(hipGetLastError());
-        // Groups only ever split: once a generation had no large group, none can appear again, and the host need
-        // not wait for the count (the error word is still read at the rank step's round trip).
-        if (!all_small) {
-            rc = read_counts(L, &big);
+        if (all_small) {
+            // Every group fits the in-tile sort: one kernel gathers, ranks and counts; one applies. Nothing is radix
+            // sorted, no key is written, and the separate counting pass of the general rank step is not needed.
+            const RankTables r = rank_tables(h, m, SMALL_TILE);
+            HIP_TRY(hipMemsetAsync(r.tile_agg, 0, (u64)r.tiles * 4 * sizeof(u32), s));
+            HIP_TRY(hipMemsetAsync(r.tile_splits, 0, (u64)r.tiles * sizeof(u32), s));
+            u32* nr_list = reinterpret_cast<u32*>(key_out); // free: this path writes no keys
+            SmallSortArgs sa;
+            memset(&sa, 0, sizeof(sa));
+            sa.sufs = ax;
+            sa.gids = agid;
+            sa.gstart = h->gstart[gp];
+            sa.rank = h->rank;
+            sa.m = m;
+            sa.n = n;
+            sa.h = (u32)h_ctx;
+            sa.sec_bits = sec_bits;
+            sa.groups = groups;
+            sa.err = h->counts + 2;
+            sa.sufs_out = x_out;
+            sa.big_count = h->counts + 4;
+            sa.gprim = h->gprim[gp];
+            sa.nr_out = nr_list;
+            sa.sa32 = sa32;
+            sa.tile_agg = r.tile_agg;
+            sa.tile_splits = r.tile_splits;
+            hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG, true>), dim3(r.tiles), dim3(SMALL_BLOCK), 0, s,
+                               sa);
+            const u32 m_in = m;
+            rc = rank_totals(L, r, false, m_in, n, false, &m, &groups, &st->rank_update[gen]);
             if (rc)
                 return rc;
-            all_small = big == 0;
-        }
-        st->big[gen] = big;
-        passes = 0;
-        if (big > 0) {
-            const int gid_bits = bit_length(groups > 1 ? groups - 1 : 0);
-            const PassPlan plan = make_plan(0, sec_bits + gid_bits);
-            rc = radix_sort(L, SRC_PAIRS, nullptr, n, 0, 0, bkey[0], bx[0], bkey[1], bx[1], big, plan, &in_out, &passes);
-            if (rc)
-                return rc;
-            PlaceArgs pa;
-            pa.big_keys = bkey[in_out];
-            pa.big_sufs = bx[in_out];
-            pa.mb = big;
-            pa.m = m;
-            pa.groups = groups;
-            pa.sec_bits = sec_bits;
-            pa.gstart = h->gstart[gp];
-            pa.keys_out = key_out;
-            pa.sufs_out = x_out;
-            pa.lookback = h->lookback;
-            pa.epoch = next_epoch(h);
-            pa.err = h->counts + 2;
-            rc = next_ticket(L, &pa.ticket);
-            if (rc)
-                return rc;
-            hipLaunchKernelGGL((place_big_kernel<RANK_BLOCK, RANK_ITEMS>), dim3((big + RANK_TILE - 1) / RANK_TILE),
-                               dim3(RANK_BLOCK), 0, s, pa);
+            ApplySmallArgs aa;
+            aa.sufs = x_out;
+            aa.nr = nr_list;
+            aa.m = m_in;
+            aa.n = n;
+            aa.rank = h->rank;
+            aa.rank_vals = st->rank_update[gen] == 2 ? defer_buf.vals : nullptr;
+            aa.sufs_out = ax;
+            aa.gids_out = agid;
+            aa.gprim_out = h->gprim[gp ^ 1];
+            aa.gstart_out = h->gstart[gp ^ 1];
+            aa.tile_prefix = r.tile_prefix;
+            aa.slab_total = r.slab_total;
+            aa.slab = r.slab;
+            aa.err = h->counts + 2;
+            hipLaunchKernelGGL((apply_small_kernel<SMALL_BLOCK, SMALL_ITEMS>), dim3(r.tiles), dim3(SMALL_BLOCK), 0, s, aa);
             HIP_TRY(hipGetLastError());
+            if (st->rank_update[gen] == 2) {
+                rc = windowed_rank_update(L, x_out, defer_buf, m_in, n);
+                if (rc)
+                    return rc;
+            }
+            st->big[gen] = 0;
+            st->small_only[gen] = 1;
+            passes = 0;
+        } else {
+            // small groups are sorted in place by one kernel; the members of large groups are set aside
+            HIP_TRY(hipMemsetAsync(h->counts + 4, 0, sizeof(u32), s));
+            SmallSortArgs sa;
+            memset(&sa, 0, sizeof(sa));
+            sa.sufs = ax;
+            sa.gids = agid;
+            sa.gstart = h->gstart[gp];
+            sa.rank = h->rank;
+            sa.m = m;
+            sa.n = n;
+            sa.h = (u32)h_ctx;
+            sa.sec_bits = sec_bits;
+            sa.groups = groups;
+            sa.err = h->counts + 2;
+            sa.keys_out = key_out;
+            sa.sufs_out = x_out;
+            sa.big_keys = bkey[0];
+            sa.big_sufs = bx[0];
+            sa.big_count = h->counts + 4;
+            hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG>),
+                               dim3((m + SMALL_TILE - 1) / SMALL_TILE), dim3(SMALL_BLOCK), 0, s, sa);
+            HIP_TRY(hipGetLastError());
+            // Groups only ever split: once a generation had no large group, none can appear again, and the host need
+            // not wait for the count (the error word is still read at the rank step's round trip).
+            if (!all_small) {
+                rc = read_counts(L, &big);
+                if (rc)
+                    return rc;
+                all_small = big == 0;
+            }
+            st->big[gen] = big;
+            passes = 0;
+            if (big > 0) {
+                const int gid_bits = bit_length(groups > 1 ? groups - 1 : 0);
+                const PassPlan plan = make_plan(0, sec_bits + gid_bits);
+                rc = radix_sort(L, SRC_PAIRS, nullptr, n, 0, 0, bkey[0], bx[0], bkey[1], bx[1], big, plan, &in_out, &passes);
+                if (rc)
+                    return rc;
+                PlaceArgs pa;
+                pa.big_keys = bkey[in_out];
+                pa.big_sufs = bx[in_out];
+                pa.mb = big;
+                pa.m = m;
+                pa.groups = groups;
+                pa.sec_bits = sec_bits;
+                pa.gstart = h->gstart[gp];
+                pa.keys_out = key_out;
+                pa.sufs_out = x_out;
+                pa.lookback = h->lookback;
+                pa.epoch = next_epoch(h);
+                pa.err = h->counts + 2;
+                rc = next_ticket(L, &pa.ticket);
+                if (rc)
+                    return rc;
+                hipLaunchKernelGGL((place_big_kernel<RANK_BLOCK, RANK_ITEMS>), dim3((big + RANK_TILE - 1) / RANK_TILE),
+                                   dim3(RANK_BLOCK), 0, s, pa);
+                HIP_TRY(hipGetLastError());
+            }
+            memset(&ra, 0, sizeof(ra));
+            ra.keys = key_out;
+            ra.sufs = x_out;
+            ra.m = m;
+            ra.gen0 = 0;
+            ra.key_words = h->key_words;
+            ra.sec_bits = sec_bits;
+            ra.n = n;
+            ra.ell = ell;
+            ra.text = d_text;
+            ra.gprim_in = h->gprim[gp];
+            ra.groups_in = groups;
+            ra.rank = h->rank;
+            ra.sa32 = sa32;
+            ra.sufs_out = ax;
+            ra.gids_out = agid;
+            ra.gprim_out = h->gprim[gp ^ 1];
+            ra.gstart_out = h->gstart[gp ^ 1];
+            rc = rerank_step(L, ra, defer_buf, &m, &groups, &st->rank_update[gen], all_small && big == 0);
+            if (rc)
+                return rc;
         }
-        memset(&ra, 0, sizeof(ra));
-        ra.keys = key_out;
-        ra.sufs = x_out;
-        ra.m = m;
-        ra.gen0 = 0;
-        ra.key_words = h->key_words;
-        ra.sec_bits = sec_bits;
-        ra.n = n;
-        ra.ell = ell;
-        ra.text = d_text;
-        ra.gprim_in = h->gprim[gp];
-        ra.groups_in = groups;
-        ra.rank = h->rank;
-        ra.sa32 = sa32;
-        ra.sufs_out = ax;
-        ra.gids_out = agid;
-        ra.gprim_out = h->gprim[gp ^ 1];
-        ra.gstart_out = h->gstart[gp ^ 1];
-        rc = rerank_step(L, ra, defer_buf, &m, &groups, &st->rank_update[gen], all_small && big == 0);
-        if (rc)
-            return rc;
         gp ^= 1;
         st->passes[gen] = passes;
         HIP_TRY(hipEventRecord(h->ev_gen[gen + 1], s));

@@ -474,9 +474,17 @@ struct SmallSortArgs {
     u64* big_keys; // elements of groups larger than MAXG
     u32* big_sufs;
     u32* big_count; // zero before the launch
+    // FUSED instantiation (lists known to hold small groups only): no keys are written; every member leaves its
+    // refined rank next to its suffix, singletons go to the suffix array at once, and the tiles of the sorted list
+    // receive their survivor / new-group / changed-rank counts, so that no separate counting pass is needed
+    const u32* gprim; // first rank of each group
+    u32* nr_out;      // refined rank of the member at each sorted place, bit 31 set if it differs from the old rank
+    u32* sa32;
+    u32* tile_agg;    // [tiles][4], zero before the launch: [2] survivors, [3] new groups of each tile of the sorted list
+    u32* tile_splits; // [tiles], zero before the launch: changed ranks
 };
 
-template <int BLOCK, int ITEMS, int MAXG>
+template <int BLOCK, int ITEMS, int MAXG, bool FUSED = false>
 __global__ __launch_bounds__(BLOCK) void smallsort_kernel(SmallSortArgs a)
 {
     constexpr int TILE = BLOCK * ITEMS;
@@ -562,6 +570,83 @@ __global__ __launch_bounds__(BLOCK) void smallsort_kernel(SmallSortArgs a)
     __syncthreads();
     slot += s_bigbase;
 
+    if constexpr (FUSED) {
+        // Rank of a member inside its group = members with a smaller rank[x + h]; members with the same one stay in
+        // list order. That fixes its sorted place, its refined rank (ranks of different groups cannot meet: a group
+        // owns the rank range [gprim, gprim + size)), whether it is alone with its key (it retires) and whether it
+        // heads a new group. Counts go to the tile of the sorted list that the member lands in: its own or, for a
+        // group that straddles a tile border, a neighbour.
+        __shared__ u32 s_nb[2][3]; // survivors, new groups, changed ranks bound for the tile before / after
+        __shared__ u32 s_own[3];
+        if (t < 6)
+            (&s_nb[0][0])[t] = 0;
+        if (t < 3)
+            s_own[t] = 0;
+        __syncthreads();
+        u32 c_surv = 0, c_head = 0, c_chg = 0;
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            const long long e = t0 + k * BLOCK + t;
+            const u32 what = (kind >> (2 * k)) & 3u;
+            if (what == 2u)
+                atomicExch(a.err, DEV_ERR_UNEXPECTED_LARGE_GROUP); // groups only split: cannot happen after an all-small list
+            if (what != 1u)
+                continue;
+            u32 less = 0, eq_before = 0, eq_after = 0;
+            for (u32 j = gs[k]; j < ge[k]; ++j) {
+                const u32 v = s_sec[(long long)j - lo];
+                less += v < sec[k] ? 1u : 0u;
+                if (v == sec[k]) {
+                    eq_before += (long long)j < e ? 1u : 0u;
+                    eq_after += (long long)j > e ? 1u : 0u;
+                }
+            }
+            const u32 pos = gs[k] + less + eq_before;
+            const u32 nr = a.gprim[g[k]] + less;
+            const bool single = eq_before + eq_after == 0;
+            if (nr >= a.n || x[k] >= a.n) {
+                atomicExch(a.err, DEV_ERR_RERANK_RANGE);
+                continue;
+            }
+            a.sufs_out[pos] = x[k];
+            a.nr_out[pos] = nr | (less ? 0x80000000u : 0u);
+            if (single)
+                a.sa32[nr] = x[k];
+            const u32 surv = single ? 0u : 1u, head = (!single && eq_before == 0) ? 1u : 0u, chg = less ? 1u : 0u;
+            const long long dest_tile = (long long)pos / TILE;
+            if (dest_tile == (long long)blockIdx.x) {
+                c_surv += surv;
+                c_head += head;
+                c_chg += chg;
+            } else {
+                const int side = dest_tile < (long long)blockIdx.x ? 0 : 1;
+                if (surv)
+                    atomicAdd(&s_nb[side][0], 1u);
+                if (head)
+                    atomicAdd(&s_nb[side][1], 1u);
+                if (chg)
+                    atomicAdd(&s_nb[side][2], 1u);
+            }
+        }
+        // per wave at most 64 * ITEMS of each: three 10-bit fields travel in one reduction
+        static_assert(64 * ITEMS < 1024, "three counts are packed into one 32-bit word");
+        const u32 packed = wave_reduce_sum(c_surv | (c_head << 10) | (c_chg << 20));
+        if ((t & 63u) == 0) {
+            atomicAdd(&s_own[0], packed & 1023u);
+            atomicAdd(&s_own[1], (packed >> 10) & 1023u);
+            atomicAdd(&s_own[2], packed >> 20);
+        }
+        __syncthreads();
+        if (t < 9) {
+            const u32 which = t / 3, field = t % 3; // 0: own tile, 1: the tile before, 2: the tile after
+            const u32 v = which == 0 ? s_own[field] : s_nb[which - 1][field];
+            const long long tile = (long long)blockIdx.x + (which == 0 ? 0 : (which == 1 ? -1 : 1));
+            if (v && tile >= 0 && tile < (long long)gridDim.x)
+                atomicAdd(field < 2 ? &a.tile_agg[tile * 4 + 2 + field] : &a.tile_splits[tile], v);
+        }
+        return;
+    }
+
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         const long long e = t0 + k * BLOCK + t;
@@ -579,6 +664,123 @@ __global__ __launch_bounds__(BLOCK) void smallsort_kernel(SmallSortArgs a)
             a.big_keys[slot] = key;
             a.big_sufs[slot] = x[k];
             slot++;
+        }
+    }
+}
+
+// Second half of a generation whose groups are all small: the sorted list carries, at every place, the suffix and
+// its refined rank (the FUSED small-group kernel wrote them and counted per tile). Equal ranks are equal keys, so
+// run heads, singletons (already in the suffix array) and new groups follow from neighbour comparison of the
+// ranks; survivors are compacted with the tile prefixes of rerank_scan_kernel. Tiles must be those the counts were
+// attributed to (TILE = the small-group kernel's).
+struct ApplySmallArgs {
+    const u32* sufs;
+    const u32* nr; // bit 31: the rank changed
+    u32 m, n;
+    u32* rank;
+    u32* rank_vals; // null: write rank[x] directly (see RerankArgs::rank_vals)
+    u32* sufs_out;
+    u32* gids_out;
+    u32* gprim_out;
+    u32* gstart_out;
+    const u32* tile_prefix; // [tiles][4]
+    const u32* slab_total;  // [RERANK_SLABS][5]
+    u32 slab;
+    u32* err;
+};
+
+template <int BLOCK, int ITEMS>
+__global__ __launch_bounds__(BLOCK) void apply_small_kernel(ApplySmallArgs a)
+{
+    constexpr int TILE = BLOCK * ITEMS;
+    constexpr int WAVES = BLOCK / WAVE;
+    __shared__ u32 s_nr[TILE + 2];
+    __shared__ u32 s_x[TILE];
+    __shared__ u32 s_w[WAVES][2];
+    const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
+    const u32 tile = blockIdx.x;
+    const u64 tile_base = (u64)tile * TILE;
+    const u32 m = a.m;
+    // striped loads; s_nr[q] holds place tile_base + q - 1
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        const u32 q = j * BLOCK + t;
+        const u64 c = tile_base + q;
+        s_nr[q + 1] = c < m ? a.nr[c] : 0u;
+        s_x[q] = c < m ? a.sufs[c] : 0u;
+    }
+    if (t == 0)
+        s_nr[0] = tile_base >= 1 ? a.nr[tile_base - 1] : 0u;
+    if (t == 1)
+        s_nr[TILE + 1] = tile_base + TILE < m ? a.nr[tile_base + TILE] : 0u;
+    __syncthreads();
+    // blocked: thread t owns places tile_base + t * ITEMS + k
+    const u64 base = tile_base + (u64)t * ITEMS;
+    u32 flags = 0; // 2 bits per item: bit 0 survivor, bit 1 head of a new group
+    u32 lsurv = 0, lhead = 0;
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const u64 c = base + k;
+        if (c < m) {
+            const u32 q = t * ITEMS + k + 1;
+            const u32 me = s_nr[q] & 0x7FFFFFFFu;
+            const bool head = c == 0 || (s_nr[q - 1] & 0x7FFFFFFFu) != me;
+            const bool last = c + 1 == m || (s_nr[q + 1] & 0x7FFFFFFFu) != me;
+            const bool surv = !(head && last);
+            flags |= (surv ? 1u : 0u) << (2 * k);
+            flags |= ((head && surv) ? 2u : 0u) << (2 * k);
+            lsurv += surv ? 1u : 0u;
+            lhead += (head && surv) ? 1u : 0u;
+        }
+    }
+    const u32 is = wave_incl_sum(lsurv), ih = wave_incl_sum(lhead);
+    if (lane == 63u) {
+        s_w[w][0] = is;
+        s_w[w][1] = ih;
+    }
+    __syncthreads();
+    u32 rc = is - lsurv, rh = ih - lhead; // exclusive inside the tile
+    u32 tot_s = 0, tot_h = 0;
+    for (u32 ww = 0; ww < WAVES; ++ww) {
+        if (ww < w) {
+            rc += s_w[ww][0];
+            rh += s_w[ww][1];
+        }
+        tot_s += s_w[ww][0];
+        tot_h += s_w[ww][1];
+    }
+    u32 tile_rc = a.tile_prefix[(u64)tile * 4 + 2], tile_rh = a.tile_prefix[(u64)tile * 4 + 3];
+    for (u32 sl = 0; sl < tile / a.slab; ++sl) {
+        tile_rc += a.slab_total[sl * 5 + 2];
+        tile_rh += a.slab_total[sl * 5 + 3];
+    }
+    if (t == 0 && tile_base + TILE >= m)
+        a.gstart_out[tile_rh + tot_h] = tile_rc + tot_s; // gstart[groups] = survivors
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const u64 c = base + k;
+        if (c >= m)
+            continue;
+        const u32 q = t * ITEMS + k;
+        const u32 word = s_nr[q + 1], nr = word & 0x7FFFFFFFu, x = s_x[q];
+        const u32 f = (flags >> (2 * k)) & 3u;
+        if (nr >= a.n || x >= a.n) {
+            atomicExch(a.err, DEV_ERR_RERANK_RANGE);
+            continue;
+        }
+        if (a.rank_vals)
+            a.rank_vals[c] = (word >> 31) ? nr : NO_RANK;
+        else if (word >> 31)
+            a.rank[x] = nr;
+        if (f & 2u) {
+            a.gprim_out[tile_rh + rh] = nr;
+            a.gstart_out[tile_rh + rh] = tile_rc + rc;
+            rh++;
+        }
+        if (f & 1u) {
+            a.sufs_out[tile_rc + rc] = x;
+            a.gids_out[tile_rc + rc] = tile_rh + rh - 1;
+            rc++;
         }
     }
 }

@@ -49,6 +49,8 @@ typedef struct csa_stats {
     int32_t rank_update[CSA_MAX_GENERATIONS]; /* how generation g wrote its ranks: 0 scattered from the rank pass,
                                                  1 bucketed by two passes into LDS-sized windows (generation 0),
                                                  2 bucketed by one pass into cache-sized windows */
+    int32_t small_only[CSA_MAX_GENERATIONS];  /* 1: generation g held small groups only and ran as two fused kernels
+                                                 (in-tile sort + ranking + counting, then apply) without a radix sort */
     float ms[CSA_MAX_GENERATIONS];        /* device time of generation g */
     float ms_output;                      /* sa40 emission */
     float ms_total;                       /* first kernel to last kernel, on the stream */

@@ -48,6 +48,7 @@ def emu_sort(lib, T, key_words):
     lib.csa_destroy(h)
     assert rc == 0, lib.csa_last_error()
     emu_sort.rank_update = [int(st.rank_update[i]) for i in range(st.generations)]
+    emu_sort.small_only = [int(st.small_only[i]) for i in range(st.generations)]
     return out[:5 * n], [int(st.active[i]) for i in range(st.generations)], [int(st.big[i]) for i in range(st.generations)]
 
 
@@ -91,6 +92,9 @@ def test_small_and_large_groups_take_both_paths(emu):
     # generation 0 takes the two-pass bucketed rank update here and later ones the one-pass kind (the emulation
     # library is built with tiny thresholds for both); the short fixtures above write their ranks directly
     assert emu_sort.rank_update[0] == 1 and 2 in emu_sort.rank_update[1:]
+    # once a generation had no large group, the following ones run as the fused small-group generation
+    first_small = big.index(0, 1)
+    assert emu_sort.small_only == [0] * (first_small + 1) + [1] * (len(big) - first_small - 1) and 1 in emu_sort.small_only
 
 
 def test_emulated_radix_sort_matches_stable_sort(emu):

@@ -245,8 +245,12 @@ def test_sixteen_million_symbols_pass_the_oracle_verifier(torch_mod, config):
         assert s.verify(d, out)
         got = out.cpu().numpy()
         how = s.last_stats["rank_update"]
+        fused = s.last_stats["small_only"]
     assert oracle_lib.is_correct_sa40(got, T)
     assert how[0] == 1  # generation 0 went through the two-pass bucketed rank update
+    assert fused[0] == 0
+    if config in (3, 4):  # their late generations hold small groups only (the long runs of config 5 never do)
+        assert fused[-1] == 1
     if config == 4:     # four letters: nearly every rank changes in generation 1, which takes the one-pass kind
         assert 2 in how[1:] and 0 in how[1:]
 
