@@ -694,8 +694,11 @@ __global__ __launch_bounds__(BLOCK) void apply_small_kernel(ApplySmallArgs a)
 {
     constexpr int TILE = BLOCK * ITEMS;
     constexpr int WAVES = BLOCK / WAVE;
-    __shared__ u32 s_nr[TILE + 2];
-    __shared__ u32 s_x[TILE];
+    // one pad word per ITEMS elements keeps the blocked accesses (stride ITEMS) off a single LDS bank
+    constexpr int PADDED = TILE + 2 + (TILE + 2) / ITEMS + 1;
+    __shared__ u32 s_nr[PADDED];
+    __shared__ u32 s_x[PADDED];
+#define CSA_PADI(q) ((q) + (q) / ITEMS)
     __shared__ u32 s_w[WAVES][2];
     const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
     const u32 tile = blockIdx.x;
@@ -706,13 +709,13 @@ __global__ __launch_bounds__(BLOCK) void apply_small_kernel(ApplySmallArgs a)
     for (int j = 0; j < ITEMS; ++j) {
         const u32 q = j * BLOCK + t;
         const u64 c = tile_base + q;
-        s_nr[q + 1] = c < m ? a.nr[c] : 0u;
-        s_x[q] = c < m ? a.sufs[c] : 0u;
+        s_nr[CSA_PADI(q + 1)] = c < m ? a.nr[c] : 0u;
+        s_x[CSA_PADI(q)] = c < m ? a.sufs[c] : 0u;
     }
     if (t == 0)
-        s_nr[0] = tile_base >= 1 ? a.nr[tile_base - 1] : 0u;
+        s_nr[CSA_PADI(0)] = tile_base >= 1 ? a.nr[tile_base - 1] : 0u;
     if (t == 1)
-        s_nr[TILE + 1] = tile_base + TILE < m ? a.nr[tile_base + TILE] : 0u;
+        s_nr[CSA_PADI(TILE + 1)] = tile_base + TILE < m ? a.nr[tile_base + TILE] : 0u;
     __syncthreads();
     // blocked: thread t owns places tile_base + t * ITEMS + k
     const u64 base = tile_base + (u64)t * ITEMS;
@@ -723,9 +726,9 @@ __global__ __launch_bounds__(BLOCK) void apply_small_kernel(ApplySmallArgs a)
         const u64 c = base + k;
         if (c < m) {
             const u32 q = t * ITEMS + k + 1;
-            const u32 me = s_nr[q] & 0x7FFFFFFFu;
-            const bool head = c == 0 || (s_nr[q - 1] & 0x7FFFFFFFu) != me;
-            const bool last = c + 1 == m || (s_nr[q + 1] & 0x7FFFFFFFu) != me;
+            const u32 me = s_nr[CSA_PADI(q)] & 0x7FFFFFFFu;
+            const bool head = c == 0 || (s_nr[CSA_PADI(q - 1)] & 0x7FFFFFFFu) != me;
+            const bool last = c + 1 == m || (s_nr[CSA_PADI(q + 1)] & 0x7FFFFFFFu) != me;
             const bool surv = !(head && last);
             flags |= (surv ? 1u : 0u) << (2 * k);
             flags |= ((head && surv) ? 2u : 0u) << (2 * k);
@@ -762,7 +765,7 @@ __global__ __launch_bounds__(BLOCK) void apply_small_kernel(ApplySmallArgs a)
         if (c >= m)
             continue;
         const u32 q = t * ITEMS + k;
-        const u32 word = s_nr[q + 1], nr = word & 0x7FFFFFFFu, x = s_x[q];
+        const u32 word = s_nr[CSA_PADI(q + 1)], nr = word & 0x7FFFFFFFu, x = s_x[CSA_PADI(q)];
         const u32 f = (flags >> (2 * k)) & 3u;
         if (nr >= a.n || x >= a.n) {
             atomicExch(a.err, DEV_ERR_RERANK_RANGE);
@@ -784,6 +787,7 @@ __global__ __launch_bounds__(BLOCK) void apply_small_kernel(ApplySmallArgs a)
         }
     }
 }
+#undef CSA_PADI
 
 // Brings the radix-sorted elements of the large groups back into the sorted active list: the k-th sorted
 // element of group g goes to gstart[g] + (k - index of g's first element). One max look-back chain finds
