@@ -218,8 +218,16 @@ def bench_next_rows(args):
                                                                                primary.data_ptr(), keys.data_ptr(), n, st)), args.steps, args.warmup)
         want = (primary[pick].to(torch.int64) << 31) | rank.to(torch.int64)
         ok = bool(torch.equal(keys[pick], want))
-        res = _row_result("messages joined/sec at 1 GPU", "messages for half of a suffix-ordered cohort", msg_c, ms, "join_messages_kernel",
-                          msg_c * (9 + 8 + 4 + 8), {"cohort": n}, args.steps, args.warmup, ok)
+        # the variant that sorts the inbox by target first (5 radix passes in a handle's scratch, then the same search)
+        sorter = PartitionSorter(msg_c)
+        keys.fill_(-1)
+        ms_sorted, _ = _timed(torch, lambda: _native.check(lib.csa_join_messages_sorted_dev(
+            sorter._h, lanes.data_ptr(), rank.data_ptr(), msg_c, suf.data_ptr(), primary.data_ptr(), keys.data_ptr(), n, st)), args.steps, args.warmup)
+        ok = ok and bool(torch.equal(keys[pick], want))
+        sorter.close()
+        res = _row_result("messages joined/sec at 1 GPU", "messages for half of a suffix-ordered cohort", msg_c, ms_sorted,
+                          "unpack + 5 radix passes + join_messages_kernel", msg_c * (9 + 8 + 4 + 8),
+                          {"cohort": n, "ms_unsorted_inbox": round(ms, 3)}, args.steps, args.warmup, ok)
     else:  # scatter
         rank = torch.randperm(n, device=dev).to(torch.int32)
         lanes = torch.randint(0, 256, (5 * n,), dtype=torch.uint8, device=dev)

@@ -979,9 +979,44 @@ int csa_join_messages_dev(const uint8_t* d_msg_target, const uint32_t* d_msg_ran
     if (n > CSA_MAX_PART_SZ)
         return fail(CSA_ERR_TOO_LARGE, "csa_join_messages_dev: %llu suffixes exceed a partition", (unsigned long long)n);
     hipLaunchKernelGGL(join_messages_kernel, dim3((msg_c + 255u) / 256u), dim3(256), 0, (hipStream_t)stream, d_msg_target,
-                       d_msg_rank, msg_c, d_sa, d_primary, d_keys, n);
+                       (const u64*)nullptr, d_msg_rank, msg_c, d_sa, d_primary, d_keys, n);
     HIP_TRY(hipGetLastError());
     return CSA_OK;
+}
+
+int csa_join_messages_sorted_dev(csa_handle* h, const uint8_t* d_msg_target, const uint32_t* d_msg_rank, uint32_t msg_c,
+                                 const uint64_t* d_sa, const uint32_t* d_primary, uint64_t* d_keys, uint64_t n, void* stream)
+{
+    if (!h)
+        return fail(CSA_ERR_ARG, "csa_join_messages_sorted_dev: null handle");
+    if (msg_c == 0)
+        return CSA_OK;
+    if (!d_msg_target || !d_msg_rank || (n && (!d_sa || !d_primary || !d_keys)))
+        return fail(CSA_ERR_ARG, "csa_join_messages_sorted_dev: null buffer");
+    if (n > CSA_MAX_PART_SZ)
+        return fail(CSA_ERR_TOO_LARGE, "csa_join_messages_sorted_dev: %llu suffixes exceed a partition", (unsigned long long)n);
+    if (msg_c > h->cap)
+        return fail(CSA_ERR_ARG, "csa_join_messages_sorted_dev: %u messages exceed the handle's capacity %llu", msg_c,
+                    (unsigned long long)h->cap);
+    Launch L;
+    L.h = h;
+    L.stream = (hipStream_t)stream;
+    L.flags = 0;
+    L.stats = nullptr;
+    hipStream_t s = L.stream;
+    HIP_TRY(hipMemsetAsync(h->counts, 0, 4 * sizeof(u32), s));
+    // (target word, rank) pairs in the handle's arrays, sorted on the 40 target bits
+    hipLaunchKernelGGL(unpack_lanes_kernel, dim3((msg_c + 255u) / 256u), dim3(256), 0, s, d_msg_target, (u64)msg_c, h->key[0]);
+    HIP_TRY(hipMemcpyAsync(h->idx[0], d_msg_rank, (u64)msg_c * sizeof(u32), hipMemcpyDeviceToDevice, s));
+    int in_out = 0, passes = 0;
+    const PassPlan plan = make_plan(0, 40);
+    int rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, h->key[0], h->idx[0], h->key[1], h->idx[1], msg_c, plan, &in_out, &passes);
+    if (rc)
+        return rc;
+    hipLaunchKernelGGL(join_messages_kernel, dim3((msg_c + 255u) / 256u), dim3(256), 0, s, (const u8*)nullptr,
+                       (const u64*)h->key[in_out], (const u32*)h->idx[in_out], msg_c, d_sa, d_primary, d_keys, n);
+    HIP_TRY(hipGetLastError());
+    return read_counts(L, nullptr);
 }
 
 int csa_stage_slab_u16_dev(const uint16_t* d_text, uint64_t n, const uint8_t* d_suf40, uint64_t count, int key_words,

@@ -180,17 +180,26 @@ __global__ __launch_bounds__(1024) void message_offsets_kernel(u32* v, u32 count
 // Delivers every message to its recipient in the suffix-ordered cohort SA[0, n): K[pos] = primary[pos] << 31 |
 // received rank, marked if the message is a pill; a recipient that is not in the cohort has retired and the
 // message is dropped (include/GPU_SACA.cuh:362-389).
-__global__ __launch_bounds__(256) void join_messages_kernel(const u8* __restrict__ msg_target, const u32* __restrict__ msg_rank,
-                                                            u32 msg_c, const u64* __restrict__ sa,
-                                                            const u32* __restrict__ primary, u64* keys, u64 n)
+// The targets come as 5-byte lanes (msg_target) or, when the inbox was sorted by target first, as 64-bit words
+// (target_words): sorted targets probe neighbouring places of the cohort, so that the probes of a wave share
+// cache lines instead of each costing a line from HBM.
+__global__ __launch_bounds__(256) void join_messages_kernel(const u8* __restrict__ msg_target,
+                                                            const u64* __restrict__ target_words,
+                                                            const u32* __restrict__ msg_rank, u32 msg_c,
+                                                            const u64* __restrict__ sa, const u32* __restrict__ primary,
+                                                            u64* keys, u64 n)
 {
     const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
     if (i >= msg_c)
         return;
     u64 tgt = 0;
+    if (target_words) {
+        tgt = target_words[i] & MSG_VAL_MASK;
+    } else {
 #pragma unroll
-    for (int b = 0; b < 5; ++b)
-        tgt |= (u64)msg_target[5 * i + b] << (8 * b);
+        for (int b = 0; b < 5; ++b)
+            tgt |= (u64)msg_target[5 * i + b] << (8 * b);
+    }
     u64 low = 0, high = n;
     while (low < high) {
         const u64 mid = low + (high - low) / 2;
@@ -206,6 +215,19 @@ __global__ __launch_bounds__(256) void join_messages_kernel(const u8* __restrict
     if (r & MSG_PILL_BIT)
         key |= MSG_PILL_RECEIPT;
     keys[low] = key;
+}
+
+// 5-byte lanes -> 64-bit words (the keys of the inbox sort)
+__global__ __launch_bounds__(256) void unpack_lanes_kernel(const u8* __restrict__ lanes, u64 count, u64* __restrict__ words)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= count)
+        return;
+    u64 v = 0;
+#pragma unroll
+    for (int b = 0; b < 5; ++b)
+        v |= (u64)lanes[5 * i + b] << (8 * b);
+    words[i] = v;
 }
 
 } // namespace csa

@@ -177,6 +177,13 @@ int csa_emit_messages_dev(const uint64_t* d_sa, const uint64_t* d_keys, const ui
 int csa_join_messages_dev(const uint8_t* d_msg_target, const uint32_t* d_msg_rank, uint32_t msg_c, const uint64_t* d_sa,
                           const uint32_t* d_primary, uint64_t* d_keys, uint64_t n, void* stream);
 
+/* The same delivery with the handle's scratch: the inbox is first sorted by target (40-bit LSD radix sort inside the
+ * handle, msg_c <= its capacity), so that the searches of neighbouring messages walk neighbouring places of the cohort.
+ * Same result as csa_join_messages_dev; the inbox itself is left as it was. The call returns after the stream has
+ * finished. No counterpart in the reference (it probes in arrival order). */
+int csa_join_messages_sorted_dev(csa_handle* h, const uint8_t* d_msg_target, const uint32_t* d_msg_rank, uint32_t msg_c,
+                                 const uint64_t* d_sa, const uint32_t* d_primary, uint64_t* d_keys, uint64_t n, void* stream);
+
 /* ---- the step after the partition sort, for partitions that come back as (suffix, local rank) pairs ---- */
 
 /* d_sa40 entry rank[i] = d_suf entry i for i in [0, part_sz): 5-byte little-endian lanes in, lanes in rank order out.

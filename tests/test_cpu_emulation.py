@@ -34,6 +34,7 @@ def emu():
     lib.csa_message_offsets_dev.argtypes = [vp, u32, vp]
     lib.csa_emit_messages_dev.argtypes = [vp, vp, vp, u64, u64, i32, vp, u32, vp, vp, vp, vp]
     lib.csa_join_messages_dev.argtypes = [vp, vp, u32, vp, vp, vp, u64, vp]
+    lib.csa_join_messages_sorted_dev.argtypes = [vp, vp, vp, u32, vp, vp, vp, u64, vp]
     return lib
 
 
@@ -190,3 +191,10 @@ def test_emulated_join_matches_the_oracle(emu):
     assert emu.csa_join_messages_dev(lanes.ctypes.data, rank.ctypes.data, tgt.size, sa.ctypes.data, primary.ctypes.data,
                                      keys.ctypes.data, n, None) == 0
     assert np.array_equal(keys, oracle_lib.join_messages(tgt, rank, sa, primary, seed_keys))
+    keys2 = seed_keys.copy()
+    h = C.c_void_p()
+    assert emu.csa_create(tgt.size, 1, C.byref(h)) == 0
+    rc = emu.csa_join_messages_sorted_dev(h, lanes.ctypes.data, rank.ctypes.data, tgt.size, sa.ctypes.data, primary.ctypes.data,
+                                          keys2.ctypes.data, n, None)
+    emu.csa_destroy(h)
+    assert rc == 0 and np.array_equal(keys2, keys)

@@ -89,4 +89,14 @@ def test_join_matches_the_oracle(gpu):
         print(f"  join n={n} messages={tgt.size}", flush=True)
         assert lib.csa_join_messages_dev(to_dev(oracle_lib.u64_to_sa40(tgt)).ptr, to_dev(rank).ptr, tgt.size, to_dev(sa).ptr,
                                          to_dev(primary).ptr, d_keys.ptr, n, None) == 0
-        assert np.array_equal(to_host(d_keys), oracle_lib.join_messages(tgt, rank, sa, primary, seed_keys))
+        want = oracle_lib.join_messages(tgt, rank, sa, primary, seed_keys)
+        assert np.array_equal(to_host(d_keys), want)
+        # the same through the variant that sorts the inbox by target first (scratch of a handle)
+        from cascade_amd import PartitionSorter
+        with PartitionSorter(max(tgt.size, 16)) as s:
+            d_keys2 = to_dev(seed_keys)
+            d_lanes = to_dev(oracle_lib.u64_to_sa40(tgt))
+            assert lib.csa_join_messages_sorted_dev(s._h, d_lanes.ptr, to_dev(rank).ptr, tgt.size, to_dev(sa).ptr,
+                                                    to_dev(primary).ptr, d_keys2.ptr, n, None) == 0
+            assert np.array_equal(to_host(d_keys2), want)
+            assert np.array_equal(to_host(d_lanes), oracle_lib.u64_to_sa40(tgt))  # the inbox is left alone
