@@ -670,96 +670,50 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
             return fail(CSA_ERR_INTERNAL, "generation cap reached with %u suffixes still active", m);
         st->active[gen] = m;
         st->groups[gen] = groups;
+        const u32 m_in = m;
+        const RankTables r = rank_tables(h, m_in, SMALL_TILE);
+        u32* nr_list = reinterpret_cast<u32*>(key_out); // refined rank at every place of the sorted list
+        // 1. gather rank[x + h]; small groups are sorted and ranked inside their tile, members of large groups set aside
+        SmallSortArgs sa;
+        memset(&sa, 0, sizeof(sa));
+        sa.sufs = ax;
+        sa.gids = agid;
+        sa.gstart = h->gstart[gp];
+        sa.gprim = h->gprim[gp];
+        sa.rank = h->rank;
+        sa.m = m_in;
+        sa.n = n;
+        sa.h = (u32)h_ctx;
+        sa.sec_bits = sec_bits;
+        sa.groups = groups;
+        sa.err = h->counts + 2;
+        sa.sufs_out = x_out;
+        sa.nr_out = nr_list;
+        sa.big_keys = bkey[0];
+        sa.big_sufs = bx[0];
+        sa.big_count = h->counts + 4;
+        sa.tile_agg = r.tile_agg;
+        sa.tile_splits = r.tile_splits;
+        passes = 0;
         if (all_small) {
-            // Every group fits the in-tile sort: one kernel gathers, ranks and counts; one applies. Nothing is radix
-            // sorted, no key is written, and the separate counting pass of the general rank step is not needed.
-            const RankTables r = rank_tables(h, m, SMALL_TILE);
+            // Groups only ever split: once a generation had no large group, none can appear again. The small-group
+            // kernel then also counts for the apply step, and nothing else runs before it.
             HIP_TRY(hipMemsetAsync(r.tile_agg, 0, (u64)r.tiles * 4 * sizeof(u32), s));
             HIP_TRY(hipMemsetAsync(r.tile_splits, 0, (u64)r.tiles * sizeof(u32), s));
-            u32* nr_list = reinterpret_cast<u32*>(key_out); // free: this path writes no keys
-            SmallSortArgs sa;
-            memset(&sa, 0, sizeof(sa));
-            sa.sufs = ax;
-            sa.gids = agid;
-            sa.gstart = h->gstart[gp];
-            sa.rank = h->rank;
-            sa.m = m;
-            sa.n = n;
-            sa.h = (u32)h_ctx;
-            sa.sec_bits = sec_bits;
-            sa.groups = groups;
-            sa.err = h->counts + 2;
-            sa.sufs_out = x_out;
-            sa.big_count = h->counts + 4;
-            sa.gprim = h->gprim[gp];
-            sa.nr_out = nr_list;
-            sa.sa32 = sa32;
-            sa.tile_agg = r.tile_agg;
-            sa.tile_splits = r.tile_splits;
             hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG, true>), dim3(r.tiles), dim3(SMALL_BLOCK), 0, s,
                                sa);
-            const u32 m_in = m;
-            rc = rank_totals(L, r, false, m_in, n, false, &m, &groups, &st->rank_update[gen]);
+            HIP_TRY(hipGetLastError());
+            st->small_only[gen] = 1;
+        } else {
+            HIP_TRY(hipMemsetAsync(h->counts + 4, 0, sizeof(u32), s));
+            hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG, false>), dim3(r.tiles), dim3(SMALL_BLOCK), 0, s,
+                               sa);
+            HIP_TRY(hipGetLastError());
+            rc = read_counts(L, &big);
             if (rc)
                 return rc;
-            ApplySmallArgs aa;
-            aa.sufs = x_out;
-            aa.nr = nr_list;
-            aa.m = m_in;
-            aa.n = n;
-            aa.rank = h->rank;
-            aa.rank_vals = st->rank_update[gen] == 2 ? defer_buf.vals : nullptr;
-            aa.sufs_out = ax;
-            aa.gids_out = agid;
-            aa.gprim_out = h->gprim[gp ^ 1];
-            aa.gstart_out = h->gstart[gp ^ 1];
-            aa.tile_prefix = r.tile_prefix;
-            aa.slab_total = r.slab_total;
-            aa.slab = r.slab;
-            aa.err = h->counts + 2;
-            hipLaunchKernelGGL((apply_small_kernel<SMALL_BLOCK, SMALL_ITEMS>), dim3(r.tiles), dim3(SMALL_BLOCK), 0, s, aa);
-            HIP_TRY(hipGetLastError());
-            if (st->rank_update[gen] == 2) {
-                rc = windowed_rank_update(L, x_out, defer_buf, m_in, n);
-                if (rc)
-                    return rc;
-            }
-            st->big[gen] = 0;
-            st->small_only[gen] = 1;
-            passes = 0;
-        } else {
-            // small groups are sorted in place by one kernel; the members of large groups are set aside
-            HIP_TRY(hipMemsetAsync(h->counts + 4, 0, sizeof(u32), s));
-            SmallSortArgs sa;
-            memset(&sa, 0, sizeof(sa));
-            sa.sufs = ax;
-            sa.gids = agid;
-            sa.gstart = h->gstart[gp];
-            sa.rank = h->rank;
-            sa.m = m;
-            sa.n = n;
-            sa.h = (u32)h_ctx;
-            sa.sec_bits = sec_bits;
-            sa.groups = groups;
-            sa.err = h->counts + 2;
-            sa.keys_out = key_out;
-            sa.sufs_out = x_out;
-            sa.big_keys = bkey[0];
-            sa.big_sufs = bx[0];
-            sa.big_count = h->counts + 4;
-            hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG>),
-                               dim3((m + SMALL_TILE - 1) / SMALL_TILE), dim3(SMALL_BLOCK), 0, s, sa);
-            HIP_TRY(hipGetLastError());
-            // Groups only ever split: once a generation had no large group, none can appear again, and the host need
-            // not wait for the count (the error word is still read at the rank step's round trip).
-            if (!all_small) {
-                rc = read_counts(L, &big);
-                if (rc)
-                    return rc;
-                all_small = big == 0;
-            }
-            st->big[gen] = big;
-            passes = 0;
+            all_small = big == 0;
+            // 2. the large groups: radix sort on (group id, rank[x + h]), then back into the list as (suffix, refined rank)
             if (big > 0) {
                 const int gid_bits = bit_length(groups > 1 ? groups - 1 : 0);
                 const PassPlan plan = make_plan(0, sec_bits + gid_bits);
@@ -770,12 +724,14 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
                 pa.big_keys = bkey[in_out];
                 pa.big_sufs = bx[in_out];
                 pa.mb = big;
-                pa.m = m;
+                pa.m = m_in;
+                pa.n = n;
                 pa.groups = groups;
                 pa.sec_bits = sec_bits;
                 pa.gstart = h->gstart[gp];
-                pa.keys_out = key_out;
+                pa.gprim = h->gprim[gp];
                 pa.sufs_out = x_out;
+                pa.nr_out = nr_list;
                 pa.lookback = h->lookback;
                 pa.epoch = next_epoch(h);
                 pa.err = h->counts + 2;
@@ -786,25 +742,36 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
                                    dim3(RANK_BLOCK), 0, s, pa);
                 HIP_TRY(hipGetLastError());
             }
-            memset(&ra, 0, sizeof(ra));
-            ra.keys = key_out;
-            ra.sufs = x_out;
-            ra.m = m;
-            ra.gen0 = 0;
-            ra.key_words = h->key_words;
-            ra.sec_bits = sec_bits;
-            ra.n = n;
-            ra.ell = ell;
-            ra.text = d_text;
-            ra.gprim_in = h->gprim[gp];
-            ra.groups_in = groups;
-            ra.rank = h->rank;
-            ra.sa32 = sa32;
-            ra.sufs_out = ax;
-            ra.gids_out = agid;
-            ra.gprim_out = h->gprim[gp ^ 1];
-            ra.gstart_out = h->gstart[gp ^ 1];
-            rc = rerank_step(L, ra, defer_buf, &m, &groups, &st->rank_update[gen], all_small && big == 0);
+            // 3. per-tile counts of the sorted list (4 bytes read per member)
+            hipLaunchKernelGGL((count_ranks_kernel<SMALL_BLOCK, SMALL_ITEMS>), dim3(r.tiles), dim3(SMALL_BLOCK), 0, s, nr_list, m_in,
+                               r.tile_agg, r.tile_splits);
+            HIP_TRY(hipGetLastError());
+        }
+        st->big[gen] = big;
+        // 4. scan, totals to the host, apply: retire singletons, compact survivors, write the changed ranks
+        rc = rank_totals(L, r, false, m_in, n, all_small && big == 0, &m, &groups, &st->rank_update[gen]);
+        if (rc)
+            return rc;
+        ApplySmallArgs aa;
+        aa.sufs = x_out;
+        aa.nr = nr_list;
+        aa.m = m_in;
+        aa.n = n;
+        aa.rank = h->rank;
+        aa.rank_vals = st->rank_update[gen] == 2 ? defer_buf.vals : nullptr;
+        aa.sa32 = sa32;
+        aa.sufs_out = ax;
+        aa.gids_out = agid;
+        aa.gprim_out = h->gprim[gp ^ 1];
+        aa.gstart_out = h->gstart[gp ^ 1];
+        aa.tile_prefix = r.tile_prefix;
+        aa.slab_total = r.slab_total;
+        aa.slab = r.slab;
+        aa.err = h->counts + 2;
+        hipLaunchKernelGGL((apply_small_kernel<SMALL_BLOCK, SMALL_ITEMS>), dim3(r.tiles), dim3(SMALL_BLOCK), 0, s, aa);
+        HIP_TRY(hipGetLastError());
+        if (st->rank_update[gen] == 2) {
+            rc = windowed_rank_update(L, x_out, defer_buf, m_in, n);
             if (rc)
                 return rc;
         }

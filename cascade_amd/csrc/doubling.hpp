@@ -449,42 +449,45 @@ __global__ __launch_bounds__(256) void scatter_ranks_kernel(const u32* __restric
 }
 
 // ---------------------------------------------------------------------------------------------
-// Generation t >= 1, small groups: gather rank[x + h] and sort inside each group in one pass.
+// Generation t >= 1: gather rank[x + h], and sort inside every small group in the same pass.
 //
 // The active list is grouped (members of a group are contiguous, group g = [gstart[g], gstart[g + 1])).
-// A tile stages the gathered ranks of its elements plus a halo of MAXG elements on either side in LDS;
-// each element of a group of at most MAXG members then counts the members that sort before it
-// (smaller rank[x + h], ties by position) and writes its (key, suffix) pair straight to its sorted
-// place. Elements of larger groups are appended, in no particular order, to a list that goes through
-// the radix sort instead (place_big_kernel brings them back).
-// Replaces, for such groups, the 62-bit key sort of the reference (src/GPU_SACA.cu:1841-1871).
+// A tile stages the gathered ranks of its elements plus a halo of MAXG elements on either side in LDS. For a group
+// of at most MAXG members, each member then derives from its group, all by itself:
+//   its place in the sorted group   = members with a smaller rank[x + h], ties kept in list order;
+//   its refined rank                = gprim[g] + members with a smaller rank[x + h]
+//                                     (reference: include/GPU_SACA.cuh:277, new = old + key-run head - group head);
+// and writes (suffix, refined rank) to its place of the sorted list. Equal refined ranks are equal keys: a group owns
+// the rank range [gprim, gprim + size), so ranks of different groups cannot meet. No key is written at all.
+// Members of larger groups are appended, in no particular order, to a list of (key, suffix) pairs that goes through
+// the radix sort instead (place_big_kernel brings them back in the same (suffix, refined rank) form).
+// Replaces, for small groups, the 62-bit key sort of the reference (src/GPU_SACA.cu:1841-1871).
+//
+// COUNT instantiation (lists known to hold small groups only): the kernel also adds, to the tile of the sorted list
+// that each member lands in, the survivor / new-group / changed-rank counts the apply step needs, so that no
+// counting pass over the sorted list runs at all.
 // ---------------------------------------------------------------------------------------------
 
 struct SmallSortArgs {
     const u32* sufs;   // active list
     const u32* gids;
     const u32* gstart; // [groups + 1]
+    const u32* gprim;  // [groups] first rank of each group
     const u32* rank;
     u32 m, n, h;
     u32 groups;
     int sec_bits;
     u32* err; // set to a DEV_ERR_* code if an invariant of the group tables is violated
-    u64* keys_out; // sorted active list (small groups written here directly)
-    u32* sufs_out;
-    u64* big_keys; // elements of groups larger than MAXG
+    u32* sufs_out; // sorted active list: suffix ...
+    u32* nr_out;   // ... and its refined rank, bit 31 set if it differs from the old rank
+    u64* big_keys; // elements of groups larger than MAXG: (group id << sec_bits) | rank[x + h]
     u32* big_sufs;
     u32* big_count; // zero before the launch
-    // FUSED instantiation (lists known to hold small groups only): no keys are written; every member leaves its
-    // refined rank next to its suffix, singletons go to the suffix array at once, and the tiles of the sorted list
-    // receive their survivor / new-group / changed-rank counts, so that no separate counting pass is needed
-    const u32* gprim; // first rank of each group
-    u32* nr_out;      // refined rank of the member at each sorted place, bit 31 set if it differs from the old rank
-    u32* sa32;
-    u32* tile_agg;    // [tiles][4], zero before the launch: [2] survivors, [3] new groups of each tile of the sorted list
-    u32* tile_splits; // [tiles], zero before the launch: changed ranks
+    u32* tile_agg;    // COUNT: [tiles][4], zero before the launch: [2] survivors, [3] new groups per tile of the sorted list
+    u32* tile_splits; // COUNT: [tiles], zero before the launch: changed ranks
 };
 
-template <int BLOCK, int ITEMS, int MAXG, bool FUSED = false>
+template <int BLOCK, int ITEMS, int MAXG, bool COUNT>
 __global__ __launch_bounds__(BLOCK) void smallsort_kernel(SmallSortArgs a)
 {
     constexpr int TILE = BLOCK * ITEMS;
@@ -551,67 +554,75 @@ __global__ __launch_bounds__(BLOCK) void smallsort_kernel(SmallSortArgs a)
             }
         }
     }
-    __shared__ u32 s_wbig[BLOCK / WAVE];
-    __shared__ u32 s_bigbase;
     const u32 lane = t & 63u, w = t >> 6;
-    const u32 incl = wave_incl_sum(n_big);
-    if (lane == 63u)
-        s_wbig[w] = incl;
-    __syncthreads();
-    u32 slot = incl - n_big; // exclusive prefix inside the block
-    u32 block_big = 0;
-    for (u32 ww = 0; ww < BLOCK / WAVE; ++ww) {
-        if (ww < w)
-            slot += s_wbig[ww];
-        block_big += s_wbig[ww];
+    u32 slot = 0;
+    if constexpr (!COUNT) {
+        __shared__ u32 s_wbig[BLOCK / WAVE];
+        __shared__ u32 s_bigbase;
+        const u32 incl = wave_incl_sum(n_big);
+        if (lane == 63u)
+            s_wbig[w] = incl;
+        __syncthreads();
+        slot = incl - n_big; // exclusive prefix inside the block
+        u32 block_big = 0;
+        for (u32 ww = 0; ww < BLOCK / WAVE; ++ww) {
+            if (ww < w)
+                slot += s_wbig[ww];
+            block_big += s_wbig[ww];
+        }
+        if (t == 0)
+            s_bigbase = block_big ? atomicAdd(a.big_count, block_big) : 0u;
+        __syncthreads();
+        slot += s_bigbase;
     }
-    if (t == 0)
-        s_bigbase = block_big ? atomicAdd(a.big_count, block_big) : 0u;
-    __syncthreads();
-    slot += s_bigbase;
 
-    if constexpr (FUSED) {
-        // Rank of a member inside its group = members with a smaller rank[x + h]; members with the same one stay in
-        // list order. That fixes its sorted place, its refined rank (ranks of different groups cannot meet: a group
-        // owns the rank range [gprim, gprim + size)), whether it is alone with its key (it retires) and whether it
-        // heads a new group. Counts go to the tile of the sorted list that the member lands in: its own or, for a
-        // group that straddles a tile border, a neighbour.
-        __shared__ u32 s_nb[2][3]; // survivors, new groups, changed ranks bound for the tile before / after
-        __shared__ u32 s_own[3];
+    // COUNT: survivors, new groups, changed ranks bound for the own tile (registers) or, for a group that straddles
+    // a tile border, for the tile before / after (LDS)
+    __shared__ u32 s_nb[2][3];
+    __shared__ u32 s_own[3];
+    if constexpr (COUNT) {
         if (t < 6)
             (&s_nb[0][0])[t] = 0;
         if (t < 3)
             s_own[t] = 0;
         __syncthreads();
-        u32 c_surv = 0, c_head = 0, c_chg = 0;
+    }
+    u32 c_surv = 0, c_head = 0, c_chg = 0;
 #pragma unroll
-        for (int k = 0; k < ITEMS; ++k) {
-            const long long e = t0 + k * BLOCK + t;
-            const u32 what = (kind >> (2 * k)) & 3u;
-            if (what == 2u)
+    for (int k = 0; k < ITEMS; ++k) {
+        const long long e = t0 + k * BLOCK + t;
+        const u32 what = (kind >> (2 * k)) & 3u;
+        if (what == 2u) {
+            if constexpr (COUNT) {
                 atomicExch(a.err, DEV_ERR_UNEXPECTED_LARGE_GROUP); // groups only split: cannot happen after an all-small list
-            if (what != 1u)
-                continue;
-            u32 less = 0, eq_before = 0, eq_after = 0;
-            for (u32 j = gs[k]; j < ge[k]; ++j) {
-                const u32 v = s_sec[(long long)j - lo];
-                less += v < sec[k] ? 1u : 0u;
-                if (v == sec[k]) {
-                    eq_before += (long long)j < e ? 1u : 0u;
-                    eq_after += (long long)j > e ? 1u : 0u;
-                }
+            } else {
+                a.big_keys[slot] = ((u64)g[k] << a.sec_bits) | (u64)sec[k];
+                a.big_sufs[slot] = x[k];
+                slot++;
             }
-            const u32 pos = gs[k] + less + eq_before;
-            const u32 nr = a.gprim[g[k]] + less;
+            continue;
+        }
+        if (what != 1u)
+            continue;
+        u32 less = 0, eq_before = 0, eq_after = 0;
+        for (u32 j = gs[k]; j < ge[k]; ++j) {
+            const u32 v = s_sec[(long long)j - lo];
+            less += v < sec[k] ? 1u : 0u;
+            if (v == sec[k]) {
+                eq_before += (long long)j < e ? 1u : 0u;
+                eq_after += (long long)j > e ? 1u : 0u;
+            }
+        }
+        const u32 pos = gs[k] + less + eq_before;
+        const u32 nr = a.gprim[g[k]] + less;
+        if (nr >= a.n || x[k] >= a.n) {
+            atomicExch(a.err, DEV_ERR_RERANK_RANGE);
+            continue;
+        }
+        a.sufs_out[pos] = x[k];
+        a.nr_out[pos] = nr | (less ? 0x80000000u : 0u);
+        if constexpr (COUNT) {
             const bool single = eq_before + eq_after == 0;
-            if (nr >= a.n || x[k] >= a.n) {
-                atomicExch(a.err, DEV_ERR_RERANK_RANGE);
-                continue;
-            }
-            a.sufs_out[pos] = x[k];
-            a.nr_out[pos] = nr | (less ? 0x80000000u : 0u);
-            if (single)
-                a.sa32[nr] = x[k];
             const u32 surv = single ? 0u : 1u, head = (!single && eq_before == 0) ? 1u : 0u, chg = less ? 1u : 0u;
             const long long dest_tile = (long long)pos / TILE;
             if (dest_tile == (long long)blockIdx.x) {
@@ -628,10 +639,12 @@ __global__ __launch_bounds__(BLOCK) void smallsort_kernel(SmallSortArgs a)
                     atomicAdd(&s_nb[side][2], 1u);
             }
         }
+    }
+    if constexpr (COUNT) {
         // per wave at most 64 * ITEMS of each: three 10-bit fields travel in one reduction
         static_assert(64 * ITEMS < 1024, "three counts are packed into one 32-bit word");
         const u32 packed = wave_reduce_sum(c_surv | (c_head << 10) | (c_chg << 20));
-        if ((t & 63u) == 0) {
+        if (lane == 0) {
             atomicAdd(&s_own[0], packed & 1023u);
             atomicAdd(&s_own[1], (packed >> 10) & 1023u);
             atomicAdd(&s_own[2], packed >> 20);
@@ -644,41 +657,80 @@ __global__ __launch_bounds__(BLOCK) void smallsort_kernel(SmallSortArgs a)
             if (v && tile >= 0 && tile < (long long)gridDim.x)
                 atomicAdd(field < 2 ? &a.tile_agg[tile * 4 + 2 + field] : &a.tile_splits[tile], v);
         }
-        return;
-    }
-
-#pragma unroll
-    for (int k = 0; k < ITEMS; ++k) {
-        const long long e = t0 + k * BLOCK + t;
-        const u32 what = (kind >> (2 * k)) & 3u;
-        const u64 key = ((u64)g[k] << a.sec_bits) | (u64)sec[k];
-        if (what == 1u) {
-            u32 cnt = 0;
-            for (u32 j = gs[k]; j < ge[k]; ++j) {
-                const u32 v = s_sec[(long long)j - lo];
-                cnt += (v < sec[k] || (v == sec[k] && (long long)j < e)) ? 1u : 0u;
-            }
-            a.keys_out[gs[k] + cnt] = key;
-            a.sufs_out[gs[k] + cnt] = x[k];
-        } else if (what == 2u) {
-            a.big_keys[slot] = key;
-            a.big_sufs[slot] = x[k];
-            slot++;
-        }
     }
 }
 
-// Second half of a generation whose groups are all small: the sorted list carries, at every place, the suffix and
-// its refined rank (the FUSED small-group kernel wrote them and counted per tile). Equal ranks are equal keys, so
-// run heads, singletons (already in the suffix array) and new groups follow from neighbour comparison of the
-// ranks; survivors are compacted with the tile prefixes of rerank_scan_kernel. Tiles must be those the counts were
-// attributed to (TILE = the small-group kernel's).
+// Counts of the sorted list (suffix, refined rank) per tile, for generations in which large groups came back through
+// the radix sort: survivors (members whose rank is shared), new groups, changed ranks. Reads 4 bytes per member.
+template <int BLOCK, int ITEMS>
+__global__ __launch_bounds__(BLOCK) void count_ranks_kernel(const u32* __restrict__ nr, u32 m, u32* __restrict__ tile_agg,
+                                                            u32* __restrict__ tile_splits)
+{
+    constexpr int TILE = BLOCK * ITEMS;
+    constexpr int WAVES = BLOCK / WAVE;
+    __shared__ u32 s_nr[TILE + 2];
+    __shared__ u32 s_w[WAVES];
+    const u32 t = threadIdx.x;
+    const u64 tile_base = (u64)blockIdx.x * TILE;
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        const u32 q = j * BLOCK + t;
+        const u64 c = tile_base + q;
+        s_nr[q + 1] = c < m ? nr[c] : 0u;
+    }
+    if (t == 0)
+        s_nr[0] = tile_base >= 1 ? nr[tile_base - 1] : 0u;
+    if (t == 1)
+        s_nr[TILE + 1] = tile_base + TILE < m ? nr[tile_base + TILE] : 0u;
+    __syncthreads();
+    u32 c_surv = 0, c_head = 0, c_chg = 0;
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        const u32 q = j * BLOCK + t + 1; // striped: neighbouring lanes, neighbouring LDS words
+        const u64 c = tile_base + q - 1;
+        if (c < m) {
+            const u32 word = s_nr[q], me = word & 0x7FFFFFFFu;
+            const bool head = c == 0 || (s_nr[q - 1] & 0x7FFFFFFFu) != me;
+            const bool last = c + 1 == m || (s_nr[q + 1] & 0x7FFFFFFFu) != me;
+            const bool surv = !(head && last);
+            c_surv += surv ? 1u : 0u;
+            c_head += (head && surv) ? 1u : 0u;
+            c_chg += word >> 31;
+        }
+    }
+    static_assert(64 * ITEMS < 1024, "three counts are packed into one 32-bit word");
+    const u32 packed = wave_reduce_sum(c_surv | (c_head << 10) | (c_chg << 20));
+    if ((t & 63u) == 0)
+        s_w[t >> 6] = packed;
+    __syncthreads();
+    if (t == 0) {
+        u32 sv = 0, hd = 0, ch = 0;
+        for (int ww = 0; ww < WAVES; ++ww) {
+            sv += s_w[ww] & 1023u;
+            hd += (s_w[ww] >> 10) & 1023u;
+            ch += s_w[ww] >> 20;
+        }
+        tile_agg[(u64)blockIdx.x * 4 + 0] = 0;
+        tile_agg[(u64)blockIdx.x * 4 + 1] = 0;
+        tile_agg[(u64)blockIdx.x * 4 + 2] = sv;
+        tile_agg[(u64)blockIdx.x * 4 + 3] = hd;
+        tile_splits[blockIdx.x] = ch;
+    }
+}
+
+// Second half of a generation t >= 1: the sorted list carries, at every place, the suffix and its refined rank.
+// Equal ranks are equal keys, so run heads, singletons and new groups follow from neighbour comparison of the
+// ranks: a singleton retires to its final place in the suffix array, the others are compacted, in order, into the
+// next active list (reference: cub::DevicePartition::Flagged, src/GPU_SACA.cu:1917-1925) with the tile prefixes of
+// rerank_scan_kernel, each with the dense id of its new group; changed ranks are written to rank[] (or handed to
+// the bucketed update). Tiles must be those the counts were attributed to (TILE = the small-group kernel's).
 struct ApplySmallArgs {
     const u32* sufs;
     const u32* nr; // bit 31: the rank changed
     u32 m, n;
     u32* rank;
     u32* rank_vals; // null: write rank[x] directly (see RerankArgs::rank_vals)
+    u32* sa32;      // suffix array under construction
     u32* sufs_out;
     u32* gids_out;
     u32* gprim_out;
@@ -775,6 +827,8 @@ __global__ __launch_bounds__(BLOCK) void apply_small_kernel(ApplySmallArgs a)
             a.rank_vals[c] = (word >> 31) ? nr : NO_RANK;
         else if (word >> 31)
             a.rank[x] = nr;
+        if (!(f & 1u))
+            a.sa32[nr] = x; // alone with its key: the rank is final
         if (f & 2u) {
             a.gprim_out[tile_rh + rh] = nr;
             a.gstart_out[tile_rh + rh] = tile_rc + rc;
@@ -789,20 +843,23 @@ __global__ __launch_bounds__(BLOCK) void apply_small_kernel(ApplySmallArgs a)
 }
 #undef CSA_PADI
 
-// Brings the radix-sorted elements of the large groups back into the sorted active list: the k-th sorted
-// element of group g goes to gstart[g] + (k - index of g's first element). One max look-back chain finds
-// that first element.
+// Brings the radix-sorted members of the large groups back into the sorted active list, in the (suffix, refined
+// rank) form of the small groups: the k-th sorted member of group g goes to place gstart[g] + (k - index of g's first
+// member in the sorted large-group list), and its refined rank is gprim[g] + (index of the head of its key run -
+// index of g's first member). Two max look-back chains find the two heads; wave 0 walks one, wave 1 the other.
 struct PlaceArgs {
     const u64* big_keys; // sorted by (group id, rank[x + h])
     const u32* big_sufs;
     u32 mb;
     u32 m;      // size of the active list
+    u32 n;
     u32 groups; // its groups
     int sec_bits;
     const u32* gstart;
-    u64* keys_out;
+    const u32* gprim;
     u32* sufs_out;
-    u64* lookback; // [tiles]
+    u32* nr_out;
+    u64* lookback; // [tiles][2]
     u32* ticket;
     u32 epoch;
     u32* err;
@@ -813,8 +870,9 @@ __global__ __launch_bounds__(BLOCK) void place_big_kernel(PlaceArgs a)
 {
     constexpr int TILE = BLOCK * ITEMS;
     constexpr int WAVES = BLOCK / WAVE;
-    __shared__ u32 s_wagg[WAVES];
-    __shared__ u32 s_prefix;
+    static_assert(WAVES >= 2, "one wave per look-back chain");
+    __shared__ u32 s_wagg[WAVES][2];
+    __shared__ u32 s_prefix[2];
     __shared__ u32 s_tile;
     const u32 t = threadIdx.x;
     const u32 lane = t & 63u;
@@ -831,46 +889,59 @@ __global__ __launch_bounds__(BLOCK) void place_big_kernel(PlaceArgs a)
         const u64 c = base + k;
         key[k] = (c >= 1 && c - 1 < a.mb) ? a.big_keys[c - 1] : 0;
     }
-    u32 lhead = 0;
+    u32 lg = 0, lk = 0; // last group head / key-run head among this thread's elements (0: none, or element 0)
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         const u64 c = base + k;
-        if (c < a.mb && (c == 0 || (key[k] >> a.sec_bits) != (key[k + 1] >> a.sec_bits)))
-            lhead = (u32)c;
+        if (c < a.mb) {
+            if (c == 0 || (key[k] >> a.sec_bits) != (key[k + 1] >> a.sec_bits))
+                lg = (u32)c;
+            if (c == 0 || key[k] != key[k + 1])
+                lk = (u32)c;
+        }
     }
-    const u32 incl = wave_incl_max(lhead);
-    if (lane == 63u)
-        s_wagg[w] = incl;
+    const u32 ig = wave_incl_max(lg), ik = wave_incl_max(lk);
+    if (lane == 63u) {
+        s_wagg[w][0] = ig;
+        s_wagg[w][1] = ik;
+    }
     __syncthreads();
-    u32 excl = __shfl_up(incl, 1);
+    u32 xg = __shfl_up(ig, 1), xk = __shfl_up(ik, 1);
     if (lane == 0)
-        excl = 0;
-    for (u32 ww = 0; ww < w; ++ww)
-        excl = excl > s_wagg[ww] ? excl : s_wagg[ww];
-    if (w == 0) {
+        xg = xk = 0;
+    for (u32 ww = 0; ww < w; ++ww) {
+        xg = xg > s_wagg[ww][0] ? xg : s_wagg[ww][0];
+        xk = xk > s_wagg[ww][1] ? xk : s_wagg[ww][1];
+    }
+    if (w < 2) {
         u32 agg = 0;
         for (int ww = 0; ww < WAVES; ++ww)
-            agg = agg > s_wagg[ww] ? agg : s_wagg[ww];
-        const u32 prefix = lb_wave_exclusive<true>(a.lookback, 1, tile, a.epoch, agg, a.err);
+            agg = agg > s_wagg[ww][w] ? agg : s_wagg[ww][w];
+        const u32 prefix = lb_wave_exclusive<true>(a.lookback + w, 2, tile, a.epoch, agg, a.err);
         if (lane == 0)
-            s_prefix = prefix;
+            s_prefix[w] = prefix;
     }
     __syncthreads();
-    u32 head = excl > s_prefix ? excl : s_prefix;
+    u32 ghead = xg > s_prefix[0] ? xg : s_prefix[0];
+    u32 khead = xk > s_prefix[1] ? xk : s_prefix[1];
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         const u64 c = base + k;
         if (c < a.mb) {
             const u32 g = (u32)(key[k + 1] >> a.sec_bits);
             if (c == 0 || (key[k] >> a.sec_bits) != g)
-                head = (u32)c;
-            const u32 dest = g < a.groups ? a.gstart[g] + ((u32)c - head) : a.m;
-            if (dest >= a.m || head > (u32)c) {
+                ghead = (u32)c;
+            if (c == 0 || key[k] != key[k + 1])
+                khead = (u32)c;
+            const bool ok = g < a.groups && ghead <= khead && khead <= (u32)c;
+            const u32 dest = ok ? a.gstart[g] + ((u32)c - ghead) : a.m;
+            const u32 nr = ok ? a.gprim[g] + (khead - ghead) : a.n;
+            if (dest >= a.m || nr >= a.n) {
                 atomicExch(a.err, DEV_ERR_PLACE_RANGE);
                 continue;
             }
-            a.keys_out[dest] = key[k + 1];
             a.sufs_out[dest] = a.big_sufs[c];
+            a.nr_out[dest] = nr | (khead != ghead ? 0x80000000u : 0u);
         }
     }
 }
