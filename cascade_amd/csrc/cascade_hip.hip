@@ -551,10 +551,9 @@ int rank_totals(Launch& L, const RankTables& r, bool gen0, u32 m, u32 n, bool ex
     return CSA_OK;
 }
 
-// Ranks the sorted list described by `ra`: counts per tile, scans the counts, reads the totals back, then applies them
-// and brings rank[] up to date, directly from the kernel or through one of the bucketed updates.
-int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivors, u32* groups, int* rank_update,
-                bool expect_no_big)
+// Generation 0: ranks the sorted list described by `ra`: counts per tile, scans the counts, reads the totals back, then
+// applies them and brings rank[] up to date, directly from the kernel or through the two-pass bucketed update.
+int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivors, u32* groups, int* rank_update)
 {
     csa_handle* h = L.h;
     hipStream_t s = L.stream;
@@ -567,7 +566,7 @@ int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivo
     ra.err = h->counts + 2;
     ra.rank_vals = nullptr;
     hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS, false>), dim3(r.tiles), dim3(RANK_BLOCK), 0, s, ra);
-    int rc = rank_totals(L, r, ra.gen0 != 0, ra.m, ra.n, expect_no_big, survivors, groups, rank_update);
+    int rc = rank_totals(L, r, true, ra.m, ra.n, false, survivors, groups, rank_update);
     if (rc)
         return rc;
     if (*rank_update != 0)
@@ -576,8 +575,6 @@ int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivo
     HIP_TRY(hipGetLastError());
     if (*rank_update == 1)
         return deferred_rank_update(L, ra.sufs, buf, ra.n);
-    if (*rank_update == 2)
-        return windowed_rank_update(L, ra.sufs, buf, ra.m, ra.n);
     return CSA_OK;
 }
 
@@ -634,15 +631,11 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     ra.keys = k_sorted;
     ra.sufs = sa32;
     ra.m = n;
-    ra.gen0 = 1;
     ra.key_words = h->key_words;
-    ra.sec_bits = 0;
     ra.n = n;
     ra.ell = ell;
     ra.text = d_text;
-    ra.gprim_in = nullptr;
     ra.rank = h->rank;
-    ra.sa32 = sa32;
     ra.sufs_out = ax;
     ra.gids_out = agid;
     ra.gprim_out = h->gprim[0];
@@ -651,7 +644,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     const DeferBuffers defer_buf = {bx[0], bx[1], reinterpret_cast<u32*>(bkey[0]), reinterpret_cast<u32*>(bkey[1]),
                                     reinterpret_cast<u32*>(bkey[1]) + h->cap};
     u32 m = 0, groups = 0, big = 0;
-    rc = rerank_step(L, ra, defer_buf, &m, &groups, &st->rank_update[0], false);
+    rc = rerank_step(L, ra, defer_buf, &m, &groups, &st->rank_update[0]);
     if (rc)
         return rc;
     st->passes[0] = passes;

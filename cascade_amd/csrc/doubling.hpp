@@ -8,21 +8,16 @@
 namespace csa {
 
 // ---------------------------------------------------------------------------------------------
-// Rank assignment + compaction in three launches: per-tile aggregates, a scan of the aggregates over the tiles,
-// and the pass that applies them. (A single launch with a decoupled look-back over four chains was measured at
-// 2.5 to 4 times the duration of these three on this part: with 8 XCDs the look-back words travel over the
-// fabric, and the few resident workgroups per CU spent most of their life waiting for their predecessors.)
+// Generation 0: rank assignment + compaction of the sorted K-gram keys in three launches: per-tile aggregates, a scan
+// of the aggregates over the tiles, and the pass that applies them. (A single launch with a decoupled look-back
+// was measured at 2.5 to 4 times the duration of these three on this part: with 8 XCDs the look-back words travel
+// over the fabric, and the few resident workgroups per CU spent most of their life waiting for their predecessors.)
 //
-// Input: the active suffixes sorted by key, keys[c] / sufs[c] for c in [0, m).
-//   generation 0 : key = packed K-gram(s); one primary group (the whole partition, rank 0)
-//   generation t : key = (group id << sec_bits) | rank[x + h]; group g starts at rank gprim_in[g]
-// With a(c) = index of the head of c's run of equal keys and b(c) = index of the head of c's run of
-// equal group ids, the refined rank is  prim + a(c) - b(c)  (reference: include/GPU_SACA.cuh:191-208
-// for generation 0, :218-280 for the later ones; the two max-scans of src/GPU_SACA.cu:1241-1247,
-// 1888-1902 are the look-back chains "a" and "b" here). A suffix whose run has length 1 retires:
-// its rank is final and it is written to its place in the suffix array. The others are compacted,
-// in order, into the next active list (reference: cub::DevicePartition::Flagged,
-// src/GPU_SACA.cu:1253-1261,1917-1925), each with the dense id of its new group.
+// Input: all suffixes sorted by key, keys[c] / sufs[c] for c in [0, n). The rank of a suffix is the index of the
+// head of its run of equal keys (reference: include/GPU_SACA.cuh:191-208; the max-scan of src/GPU_SACA.cu:1241-1247
+// is the max chain here). A suffix whose run has length 1 retires: its rank is final, and the sorted index array
+// already holds it at its place of the suffix array. The others are compacted, in order, into the first active list
+// (reference: cub::DevicePartition::Flagged, src/GPU_SACA.cu:1253-1261), each with the dense id of its group.
 // ---------------------------------------------------------------------------------------------
 
 constexpr u32 NO_RANK = 0xFFFFFFFFu; // ranks are below 2^31
@@ -30,30 +25,25 @@ constexpr u32 NO_RANK = 0xFFFFFFFFu; // ranks are below 2^31
 struct RerankArgs {
     const u64* keys;
     const u32* sufs;
-    u32 m;
-    int gen0;      // 1: generation 0 rules
-    int key_words; // generation 0: 1 or 2 (the low word is re-read from the text when 2)
-    int sec_bits;  // generation t: low bits of the key that hold rank[x + h]
+    u32 m;         // = n: generation 0 ranks every suffix
+    int key_words; // 1 or 2 (the low word is re-read from the text when 2)
     u32 n;         // partition size
     u32 ell;       // symbols in the generation-0 key
     const u16* text;
-    const u32* gprim_in; // generation t: first rank of each incoming group
-    u32 groups_in;       // generation t: number of incoming groups
-    u32* rank;           // [n] by text position
+    u32* rank;     // [n] by text position
     // Deferred rank update: instead of the scattered write rank[x] = r, the new rank of the suffix at sorted
-    // index c is stored at rank_vals[c] (a coalesced stream; the suffix itself is sufs[c]; NO_RANK where the rank
-    // did not change). The (x, r) pairs then go through one or two radix passes on the high bits of x before
-    // they are written to rank[], so that those writes fall into one window of rank[] at a time.
+    // index c is stored at rank_vals[c] (a coalesced stream; the suffix itself is sufs[c]). The (x, r) pairs then go
+    // through radix passes on the high bits of x before they are written to rank[], so that those writes fall into
+    // one window of rank[] at a time. (Later generations mark unchanged ranks with NO_RANK in such a stream.)
     u32* rank_vals; // null: write rank[x] directly
-    u32* sa32;           // [n] suffix array under construction
-    u32* sufs_out;       // next active list
+    u32* sufs_out;  // first active list
     u32* gids_out;
     u32* gprim_out;
-    u32* gstart_out; // index in the next active list where each new group starts; [groups] = survivors
-    u32* tile_agg;    // [tiles][4]: last key-run head, last group head, survivors, new groups of each tile
-    u32* tile_splits; // [tiles]: elements whose rank changes | elements that change if the tile starts inside a split group << 16
-    u32* tile_prefix; // [tiles][4]: the same, combined over the earlier tiles of the tile's slab (max, max, sum, sum)
-    u32* slab_total;  // [RERANK_SLABS][5]: combination over each slab of tiles (max, max, sum, sum; changed ranks)
+    u32* gstart_out; // index in the active list where each group starts; [groups] = survivors
+    u32* tile_agg;    // [tiles][4]: last key-run head (1-based, 0 = none), unused, survivors, groups of each tile
+    u32* tile_splits; // [tiles]: changed-rank counts for the scan (zero here: generation 0 writes every rank)
+    u32* tile_prefix; // [tiles][4]: the aggregates combined over the earlier tiles of the tile's slab (max, -, sum, sum)
+    u32* slab_total;  // [RERANK_SLABS][5]: combination over each slab of tiles
     u32 slab;         // tiles per slab
     u32* err;
 };
@@ -65,16 +55,15 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
 {
     constexpr int TILE = BLOCK * ITEMS;
     constexpr int WAVES = BLOCK / WAVE;
-    static_assert(TILE < 65536, "two per-tile counts are packed into one 32-bit word");
     // The tile is read from and written to HBM in striped order (consecutive lanes, consecutive elements) and
     // exchanged through LDS with the blocked order (each thread, ITEMS consecutive elements) the scans want.
     // One pad slot per ITEMS elements keeps the blocked LDS accesses off a single bank.
     constexpr int SLOTS = TILE + 2;               // element tile_base - 1, the tile, element tile_base + TILE
     constexpr int PADDED = SLOTS + SLOTS / ITEMS + 1;
     __shared__ u64 s_key[PADDED]; // later: compacted survivors (suffixes, group ids)
-    __shared__ u32 s_suf[PADDED]; // later: tables of the new groups (first rank, start)
-    __shared__ u32 s_rv[TILE];    // new ranks in list order (deferred rank update only)
-    __shared__ u32 s_wagg[WAVES][4];
+    __shared__ u32 s_suf[PADDED]; // later: tables of the groups (first rank, start)
+    __shared__ u32 s_rv[TILE];    // ranks in list order (deferred rank update only)
+    __shared__ u32 s_wagg[WAVES][3];
 #define CSA_PAD(q) ((q) + (q) / ITEMS)
 
     const u32 t = threadIdx.x;
@@ -113,161 +102,105 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
         suf[k] = s_suf[CSA_PAD(q)];
     }
     // eq[k]: elements (base+k-1) and (base+k) exist and belong to one run of equal keys
-    // pq[k]: ... and to one primary group
-    bool eq[ITEMS + 1], pq[ITEMS + 1];
+    bool eq[ITEMS + 1];
 #pragma unroll
     for (int k = 0; k < ITEMS + 1; ++k) {
         const u64 c = base + k; // right element of the pair
-        const bool both = c >= 1 && c < m;
-        bool e = both && key[k] == key[k + 1];
-        bool p = both;
-        if (a.gen0) {
-            if (e && a.key_words == 2)
-                e = load_kgram(a.text, a.n, suf[k], 1) == load_kgram(a.text, a.n, suf[k + 1], 1);
-            // a suffix that runs off the text inside its key ties with nobody (include/bit-layout.hpp:99-100)
-            if (e && ((u64)suf[k] + a.ell >= a.n || (u64)suf[k + 1] + a.ell >= a.n))
-                e = false;
-        } else {
-            p = both && (key[k] >> a.sec_bits) == (key[k + 1] >> a.sec_bits);
-        }
+        bool e = c >= 1 && c < m && key[k] == key[k + 1];
+        if (e && a.key_words == 2)
+            e = load_kgram(a.text, a.n, suf[k], 1) == load_kgram(a.text, a.n, suf[k + 1], 1);
+        // a suffix that runs off the text inside its key ties with nobody (include/bit-layout.hpp:99-100)
+        if (e && ((u64)suf[k] + a.ell >= a.n || (u64)suf[k + 1] + a.ell >= a.n))
+            e = false;
         eq[k] = e;
-        pq[k] = p;
     }
 
-    // thread-local aggregates
-    // head positions are kept 1-based (c + 1), so that 0 means "no head so far"
-    u32 la = 0, lb = 0, lcnt = 0, lheads = 0;
+    // thread-local aggregates; head positions are kept 1-based (c + 1), so that 0 means "no head so far"
+    u32 la = 0, lcnt = 0, lheads = 0;
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         const u64 c = base + k;
         if (c < m) {
             const bool ka = !eq[k];
-            const bool pb = !pq[k];
             const bool single = ka && !eq[k + 1];
             if (ka)
                 la = (u32)c + 1u;
-            if (pb)
-                lb = (u32)c + 1u;
             lcnt += single ? 0u : 1u;
             lheads += (ka && !single) ? 1u : 0u;
         }
     }
 
-    // block-wide exclusive prefix of (max a, max b, sum cnt, sum heads)
-    const u32 ia = wave_incl_max(la), ib = wave_incl_max(lb), ic = wave_incl_sum(lcnt), ih = wave_incl_sum(lheads);
+    // block-wide exclusive prefix of (max a, sum cnt, sum heads)
+    const u32 ia = wave_incl_max(la), ic = wave_incl_sum(lcnt), ih = wave_incl_sum(lheads);
     if (lane == 63u) {
         s_wagg[w][0] = ia;
-        s_wagg[w][1] = ib;
-        s_wagg[w][2] = ic;
-        s_wagg[w][3] = ih;
+        s_wagg[w][1] = ic;
+        s_wagg[w][2] = ih;
     }
     __syncthreads(); // also: every thread holds its elements in registers, the staging arrays may be reused
-    u32 xa = __shfl_up(ia, 1), xb = __shfl_up(ib, 1), xc = __shfl_up(ic, 1), xh = __shfl_up(ih, 1);
+    u32 xa = __shfl_up(ia, 1), xc = __shfl_up(ic, 1), xh = __shfl_up(ih, 1);
     if (lane == 0)
-        xa = xb = xc = xh = 0;
-    for (u32 ww = 0; ww < w; ++ww) {
-        xa = xa > s_wagg[ww][0] ? xa : s_wagg[ww][0];
-        xb = xb > s_wagg[ww][1] ? xb : s_wagg[ww][1];
-        xc += s_wagg[ww][2];
-        xh += s_wagg[ww][3];
+        xa = xc = xh = 0;
+    u32 tile_a = 0, tile_total_surv = 0, tile_total_heads = 0;
+    for (u32 ww = 0; ww < WAVES; ++ww) {
+        if (ww < w) {
+            xa = xa > s_wagg[ww][0] ? xa : s_wagg[ww][0];
+            xc += s_wagg[ww][1];
+            xh += s_wagg[ww][2];
+        }
+        tile_a = tile_a > s_wagg[ww][0] ? tile_a : s_wagg[ww][0];
+        tile_total_surv += s_wagg[ww][1];
+        tile_total_heads += s_wagg[ww][2];
     }
     if (!APPLY) {
-        if (t < 4) {
-            u32 agg = 0;
-            for (int ww = 0; ww < WAVES; ++ww)
-                agg = t < 2 ? (agg > s_wagg[ww][t] ? agg : s_wagg[ww][t]) : agg + s_wagg[ww][t];
-            a.tile_agg[(u64)tile * 4 + t] = agg;
-        }
-        // Elements whose rank will change (key-run head behind the group head), for the host's choice of how to
-        // write the ranks: those the tile can tell by itself, and those before its first head, which change if
-        // the tiles before end inside a split group. Packed as changed | undecided << 16.
-        u32 ra = xa, rb = xb, lchg = 0, lund = 0;
-#pragma unroll
-        for (int k = 0; k < ITEMS; ++k) {
-            const u64 c = base + k;
-            if (c < m) {
-                if (!eq[k])
-                    ra = (u32)c + 1u;
-                if (!pq[k])
-                    rb = (u32)c + 1u;
-                if (ra == 0)
-                    lund++;
-                else if (ra != rb)
-                    lchg++;
-            }
-        }
-        const u32 wpacked = wave_reduce_sum(lchg | (lund << 16)); // at most TILE <= 65535 each: no carry between the halves
-        __syncthreads(); // s_wagg has been read: reuse its first column
-        if (lane == 0)
-            s_wagg[w][0] = wpacked;
-        __syncthreads();
         if (t == 0) {
-            u32 sp = 0;
-            for (int ww = 0; ww < WAVES; ++ww)
-                sp += s_wagg[ww][0];
-            a.tile_splits[tile] = sp;
+            a.tile_agg[(u64)tile * 4 + 0] = tile_a;
+            a.tile_agg[(u64)tile * 4 + 1] = 0;
+            a.tile_agg[(u64)tile * 4 + 2] = tile_total_surv;
+            a.tile_agg[(u64)tile * 4 + 3] = tile_total_heads;
+            a.tile_splits[tile] = 0;
         }
         return;
     }
-    u32 tile_total_surv = 0, tile_total_heads = 0;
-    for (int ww = 0; ww < WAVES; ++ww) {
-        tile_total_surv += s_wagg[ww][2];
-        tile_total_heads += s_wagg[ww][3];
-    }
     // prefix of the tile = totals of the slabs before its slab, combined with its prefix inside the slab
-    u32 pre_a = a.tile_prefix[(u64)tile * 4 + 0], pre_b = a.tile_prefix[(u64)tile * 4 + 1];
+    u32 pre_a = a.tile_prefix[(u64)tile * 4 + 0];
     u32 tile_rc = a.tile_prefix[(u64)tile * 4 + 2], tile_rh = a.tile_prefix[(u64)tile * 4 + 3];
     for (u32 sl = 0; sl < tile / a.slab; ++sl) {
-        const u32 sa_ = a.slab_total[sl * 5 + 0], sb_ = a.slab_total[sl * 5 + 1];
+        const u32 sa_ = a.slab_total[sl * 5 + 0];
         pre_a = pre_a > sa_ ? pre_a : sa_;
-        pre_b = pre_b > sb_ ? pre_b : sb_;
         tile_rc += a.slab_total[sl * 5 + 2];
         tile_rh += a.slab_total[sl * 5 + 3];
     }
     if (t == 0 && tile_base + TILE >= m) // the last tile knows the totals
         a.gstart_out[tile_rh + tile_total_heads] = tile_rc + tile_total_surv; // gstart[groups] = survivors
     u32 ra = xa > pre_a ? xa : pre_a;
-    u32 rb = xb > pre_b ? xb : pre_b;
     u32 rc = xc; // tile-local from here on
     u32 rh = xh;
     __syncthreads(); // every thread has read s_wagg and holds its elements in registers: the staging arrays are free
     u32* s_osuf = reinterpret_cast<u32*>(s_key); // [TILE] survivors of the tile, compacted
-    u32* s_ogid = s_osuf + TILE;                 // [TILE] their new group ids
-    u32* s_oprim = s_suf;                        // [TILE / 2] first rank of each new group of the tile
-    u32* s_ostart = s_suf + TILE / 2;            // [TILE / 2] and its start in the next active list
+    u32* s_ogid = s_osuf + TILE;                 // [TILE] their group ids
+    u32* s_oprim = s_suf;                        // [TILE / 2] first rank of each group of the tile
+    u32* s_ostart = s_suf + TILE / 2;            // [TILE / 2] and its start in the active list
 
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         const u64 c = base + k;
         if (c < m) {
             const bool ka = !eq[k];
-            const bool pb = !pq[k];
             const bool single = ka && !eq[k + 1];
             if (ka)
                 ra = (u32)c + 1u;
-            if (pb)
-                rb = (u32)c + 1u;
             const u32 x = suf[k + 1];
-            u32 prim = 0;
-            if (!a.gen0) {
-                const u32 g = (u32)(key[k + 1] >> a.sec_bits);
-                prim = g < a.groups_in ? a.gprim_in[g] : a.n;
-            }
-            const u32 nr = prim + (ra - rb);
-            if (nr >= a.n || x >= a.n) { // a corrupt sorted list: report it instead of writing out of bounds
+            const u32 nr = ra - 1u; // element 0 is always a head, so ra >= 1 here
+            if (ra == 0 || nr >= a.n || x >= a.n) { // a corrupt sorted list: report it instead of writing out of bounds
                 atomicExch(a.err, DEV_ERR_RERANK_RANGE);
                 continue;
             }
-            const bool changed = a.gen0 || ra != rb;
-            if (a.rank_vals) {
-                s_rv[t * ITEMS + k] = changed ? nr : NO_RANK;
-            } else if (changed) {
+            if (a.rank_vals)
+                s_rv[t * ITEMS + k] = nr;
+            else
                 a.rank[x] = nr;
-            }
-            if (single) {
-                if (!a.gen0)
-                    a.sa32[nr] = x;
-            } else {
+            if (!single) {
                 if (ka) {
                     s_oprim[rh] = nr;
                     s_ostart[rh] = tile_rc + rc;
