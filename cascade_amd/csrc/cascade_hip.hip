@@ -837,15 +837,16 @@ int csa_partition_ids_u16_dev(const uint16_t* d_text, uint64_t n, uint64_t text_
     a.packed = d_packed;
     a.psz = reinterpret_cast<unsigned long long*>(d_psz);
     a.tiles = (u32)tiles64;
-    const u32 grid = a.tiles < 2048u ? a.tiles : 2048u;
+    const u32 grid = a.tiles < 8192u ? a.tiles : 8192u;
     hipStream_t s = (hipStream_t)stream;
     const bool piv_lds = (u64)(p - 1) * (u64)pivot_words <= PID_LDS_PIVOT_WORDS;
+    const u32 lds = partition_ids_lds_bytes(pivot_words, p, piv_lds, d_psz != nullptr, &a.hist_copies_log2);
 #define CSA_LAUNCH_PID(W)                                                                                  \
     do {                                                                                                   \
         if (piv_lds)                                                                                       \
-            hipLaunchKernelGGL((partition_ids_kernel<W, true>), dim3(grid), dim3(PID_BLOCK), 0, s, a);    \
+            hipLaunchKernelGGL((partition_ids_kernel<W, true>), dim3(grid), dim3(PID_BLOCK), lds, s, a);  \
         else                                                                                               \
-            hipLaunchKernelGGL((partition_ids_kernel<W, false>), dim3(grid), dim3(PID_BLOCK), 0, s, a);   \
+            hipLaunchKernelGGL((partition_ids_kernel<W, false>), dim3(grid), dim3(PID_BLOCK), lds, s, a); \
     } while (0)
     switch (pivot_words) {
     case 1: CSA_LAUNCH_PID(1); break;

@@ -336,6 +336,14 @@ __device__ __forceinline__ u64 load_kgram(const u16* __restrict__ T, u32 n, u32 
     return k;
 }
 
+// LDS whose size is given at launch: `extern __shared__` on the device; the CPU emulation of the kernels hands out
+// one buffer per launch instead.
+#ifdef HIPEMU
+#define CSA_DYNAMIC_LDS(T, name) T* name = reinterpret_cast<T*>(hipemu::dynamic_lds())
+#else
+#define CSA_DYNAMIC_LDS(T, name) extern __shared__ T name[]
+#endif
+
 // ---- a stretch of the text in LDS ----
 //
 // Consecutive suffixes share all but one symbol of their K-grams, and the text is only 2-byte aligned, so kernels

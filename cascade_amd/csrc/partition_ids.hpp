@@ -19,6 +19,7 @@ struct PartitionIdArgs {
     u64* packed;  // the packed map (`bits` words per 64 suffixes), or null
     unsigned long long* psz; // [p] partition sizes, added to; or null
     u32 tiles;
+    u32 hist_copies_log2; // LDS histogram: counters per partition (hot partitions spread over them)
 };
 
 constexpr int PID_BLOCK = 256;
@@ -26,6 +27,19 @@ constexpr int PID_ITEMS = 8; // groups of 64 suffixes per wave and tile
 constexpr int PID_TILE = PID_BLOCK * PID_ITEMS;
 constexpr u32 PID_LDS_PIVOT_WORDS = 4096; // pivots are searched in LDS when they fit
 constexpr u32 PID_LDS_BINS = 4096;        // partition sizes are counted in LDS when they fit
+
+// LDS bytes of a workgroup, and the histogram replication that goes with them: at most 16 counters per partition and
+// at most 16 KB of histogram.
+inline u32 partition_ids_lds_bytes(int W, u32 p, bool piv_lds, bool want_sizes, u32* copies_log2)
+{
+    u32 c = 0;
+    const bool hist_lds = want_sizes && p <= PID_LDS_BINS;
+    while (hist_lds && c < 4 && (p << (c + 1)) <= PID_LDS_BINS)
+        ++c;
+    *copies_log2 = c;
+    const u32 text_words = (PID_TILE + 4 * W + 6) / 4 + 2;
+    return text_words * 8u + (piv_lds ? (p - 1u) * (u32)W * 8u : 0u) + (hist_lds ? (p << c) * 4u : 0u);
+}
 
 // W: 64-bit words per pivot (the reference's K_WORDS, include/Packed_Prefix.hpp:26-34). PIV_LDS: the pivots fit in LDS.
 // A wave handles 64 consecutive suffixes at a time: exactly one group of the packed map, whose `bits` words the
@@ -36,15 +50,18 @@ constexpr u32 PID_LDS_BINS = 4096;        // partition sizes are counted in LDS 
 template <int W, bool PIV_LDS>
 __global__ __launch_bounds__(PID_BLOCK) void partition_ids_kernel(PartitionIdArgs a)
 {
-    __shared__ u64 s_text[(PID_TILE + 4 * W + 6) / 4 + 2];
-    __shared__ u64 s_piv[PIV_LDS ? PID_LDS_PIVOT_WORDS : 1];
-    __shared__ u32 s_hist[PID_LDS_BINS];
-    const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
+    // LDS is sized at launch (partition_ids_lds_bytes): the staged text, then the pivots (PIV_LDS), then the
+    // histogram copies. A workgroup that needs little of it leaves room for more workgroups per CU, which is what
+    // hides the latency of the stage -> search -> write chain of a tile.
+    CSA_DYNAMIC_LDS(u64, s_dyn);
+    constexpr u32 TEXT_WORDS = (PID_TILE + 4 * W + 6) / 4 + 2;
+    u64* s_text = s_dyn;
     const u32 np = a.p - 1u; // pivots
+    u64* s_piv = s_dyn + TEXT_WORDS;
+    u32* s_hist = reinterpret_cast<u32*>(s_piv + (PIV_LDS ? np * (u32)W : 0u));
+    const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
     const bool hist_lds = a.psz != nullptr && a.p <= PID_LDS_BINS;
-    u32 copies_log2 = 0; // counters per partition in the LDS histogram
-    while (copies_log2 < 4 && (a.p << (copies_log2 + 1)) <= PID_LDS_BINS)
-        ++copies_log2;
+    const u32 copies_log2 = a.hist_copies_log2; // counters per partition in the LDS histogram
     if (PIV_LDS)
         for (u32 i = t; i < np * (u32)W; i += PID_BLOCK)
             s_piv[i] = a.pivots[i];

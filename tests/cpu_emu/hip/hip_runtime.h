@@ -52,14 +52,23 @@ inline thread_local Wave* wave = nullptr;
 inline thread_local Block* block = nullptr;
 inline thread_local unsigned lane = 0;
 
-inline void launch(dim3 grid, dim3 blk, const std::function<void()>& body);
+inline void launch(dim3 grid, dim3 blk, size_t shmem, const std::function<void()>& body);
+// dynamic LDS of the running launch (workgroups run one after the other, so one buffer serves them all)
+inline std::vector<unsigned long long>& dynamic_lds_storage()
+{
+    static std::vector<unsigned long long> v;
+    return v;
+}
+inline void* dynamic_lds() { return dynamic_lds_storage().data(); }
 } // namespace hipemu
+#define HIPEMU 1
 
 inline thread_local dim3 threadIdx, blockIdx, blockDim, gridDim;
 
-inline void hipemu::launch(dim3 grid, dim3 blk, const std::function<void()>& body)
+inline void hipemu::launch(dim3 grid, dim3 blk, size_t shmem, const std::function<void()>& body)
 {
     const unsigned B = blk.x;
+    dynamic_lds_storage().assign(shmem / 8 + 2, 0ull);
     if (B % 64 != 0)
         std::abort();
     // HIPEMU_REVERSE=1 runs the workgroups from the last blockIdx to the first: results must not depend on it
@@ -90,7 +99,7 @@ inline void hipemu::launch(dim3 grid, dim3 blk, const std::function<void()>& bod
 }
 
 #define hipLaunchKernelGGL(kernel, grid, blk, shmem, stream, ...) \
-    hipemu::launch((grid), (blk), [&] { kernel(__VA_ARGS__); })
+    hipemu::launch((grid), (blk), (shmem), [&] { kernel(__VA_ARGS__); })
 
 // ---- synchronisation and wave operations ----
 inline void __syncthreads() { hipemu::block->bar->arrive_and_wait(); }
