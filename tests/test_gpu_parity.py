@@ -273,3 +273,40 @@ def test_random_small_texts_against_the_oracle(torch_mod):
             print(f"  random case={case} n={n} sigma={sigma} key_words={kw}", flush=True)
             got = s.sort(to_dev(torch_mod, T)).cpu().numpy()
         assert np.array_equal(got, oracle_lib.build_sa40(T)), (case, n, sigma, kw)
+
+
+def test_three_dispatcher_threads_with_their_own_handles_and_streams(torch_mod):
+    """The reference drives three buffer sets from three threads, one stream each (include/GPU_SACA.hpp:90-91,
+    src/GPU_SACA.cu:1539-1589): handles must not share state. Three threads sort different partitions at once,
+    several times over, each on its own stream and handle; every result is byte-equal to the oracle's."""
+    import threading
+    from cascade_amd import PartitionSorter
+    torch = torch_mod
+    rng = np.random.default_rng(33)
+    jobs = []
+    for k in range(3):
+        texts_k = [texts.random_text(int(rng.integers(20000, 90000)), 2 + k, 100 * k + r, sep_every=0) for r in range(4)]
+        jobs.append([(T, oracle_lib.build_sa40(T)) for T in texts_k])
+    errors = []
+
+    def worker(k):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream), PartitionSorter(100000, key_words=1 + k % 2) as s:
+                for rep in range(3):
+                    for T, want in jobs[k]:
+                        d = torch.from_numpy(np.ascontiguousarray(T).view(np.int16)).cuda(non_blocking=False)
+                        got = s.sort(d)
+                        stream.synchronize()
+                        if not np.array_equal(got.cpu().numpy(), want):
+                            errors.append((k, rep, T.size))
+        except Exception as e:  # noqa: BLE001 - reported below, in the main thread
+            errors.append((k, repr(e)))
+
+    print("  three threads, three handles, three streams", flush=True)
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(3)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
