@@ -80,78 +80,12 @@ __device__ __forceinline__ u64 lb_load(const u64* p)
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// The protocol in two steps, so that a kernel can publish its aggregate as soon as it is known and wait
-// for its predecessors as late as possible.
-// Step 1: publish `aggregate` of `tile` on the chain whose word for tile t lives at chain[t * stride].
+// Publishes `aggregate` of `tile` on the chain whose word for tile t lives at chain[t * stride] (tile 0's aggregate is
+// its inclusive prefix). A kernel publishes as soon as the aggregate is known and waits for its predecessors as late
+// as possible; the two walks below do the waiting.
 __device__ __forceinline__ void lb_publish(u64* chain, u32 stride, u32 tile, u32 epoch, u32 aggregate)
 {
     lb_store(chain + (u64)tile * stride, lb_pack(epoch, tile == 0 ? LB_INCL : LB_AGG, aggregate));
-}
-
-// Step 2: returns the combination of the aggregates of tiles [0, tile) and upgrades the tile's own word
-// to "inclusive". Combination is max if IS_MAX, else a 32-bit sum.
-// The walk towards tile 0 reads W predecessor words per round, all loads in flight together, and then consumes
-// them in order up to the first inclusive one. A serial walk (one dependent load per predecessor) would cap
-// the whole launch at one tile per memory round trip, because the nearest inclusive word is about as far back
-// as there are unresolved tiles in flight.
-// On a timeout (a predecessor never published) sets *err and returns what it has, so that every wave still
-// leaves the kernel.
-template <bool IS_MAX, int W = 8>
-__device__ __forceinline__ u32 lb_wait_exclusive(u64* chain, u32 stride, u32 tile, u32 epoch, u32 aggregate, u32* err)
-{
-    if (tile == 0)
-        return 0;
-    u32 excl = 0;
-    long long next = (long long)tile - 1; // nearest predecessor not yet consumed
-    u32 idle = 0;
-    bool done = false;
-    while (!done) {
-        u64 word[W];
-#pragma unroll
-        for (int j = 0; j < W; ++j) {
-            const long long idx = next - j;
-            word[j] = idx >= 0 ? lb_load(chain + (u64)idx * stride) : 0ull;
-        }
-        u32 consumed = 0;
-#pragma unroll
-        for (int j = 0; j < W; ++j) {
-            if (done || consumed != (u32)j)
-                continue; // stopped at an earlier word of this round
-            if (next - j < 0) { // cannot happen: tile 0 publishes an inclusive word
-                done = true;
-                continue;
-            }
-            const u64 wd = word[j];
-            const u32 status = (u32)(wd >> 32) & 3u;
-            if ((u32)(wd >> 34) != epoch || status == 0)
-                continue; // not published yet: poll again from here
-            const u32 v = (u32)wd;
-            excl = IS_MAX ? (excl > v ? excl : v) : excl + v;
-            consumed++;
-            if (status == LB_INCL)
-                done = true;
-        }
-        next -= consumed;
-        if (!done && consumed == 0) {
-            if (++idle >= LB_SPIN_LIMIT) {
-                atomicExch(err, DEV_ERR_LOOKBACK_TIMEOUT);
-                return excl;
-            }
-            __builtin_amdgcn_s_sleep(1);
-        } else {
-            idle = 0;
-        }
-    }
-    const u32 incl = IS_MAX ? (excl > aggregate ? excl : aggregate) : excl + aggregate;
-    lb_store(chain + (u64)tile * stride, lb_pack(epoch, LB_INCL, incl));
-    return excl;
-}
-
-template <bool IS_MAX, int W = 16>
-__device__ __forceinline__ u32 lb_exclusive_prefix(u64* chain, u32 stride, u32 tile, u32 epoch, u32 aggregate, u32* err)
-{
-    lb_publish(chain, stride, tile, epoch, aggregate);
-    return lb_wait_exclusive<IS_MAX, W>(chain, stride, tile, epoch, aggregate, err);
 }
 
 // ---- two-level look-back (one chain per thread, many chains per tile: the radix pass) ----
@@ -182,8 +116,9 @@ __device__ __forceinline__ u64 lb_wait_word(const u64* p, u32 epoch, u32* err)
     }
 }
 
-// tile_chain: word of tile t at tile_chain[t * stride], published with lb_publish_aggregate_only beforehand.
-// group_chain: word of group g at group_chain[g * stride]. Returns the sum of the aggregates of tiles [0, tile).
+// tile_chain: word of tile t at tile_chain[t * stride]; it only ever holds the tile's own aggregate (lb2_publish).
+// group_chain: word of group g at group_chain[g * stride]. lb2_wait_exclusive returns the sum of the aggregates of
+// tiles [0, tile).
 __device__ __forceinline__ void lb2_publish(u64* tile_chain, u32 stride, u32 tile, u32 epoch, u32 aggregate)
 {
     lb_store(tile_chain + (u64)tile * stride, lb_pack(epoch, LB_AGG, aggregate));
