@@ -1,0 +1,177 @@
+"""A miniature of the reference's multi-partition pipeline (src/GPU_SACA.cu:1999-2103 and the steps it drives), used to
+prove that the library's stage kernels compose into a correct suffix array when partitions only exchange ranks
+through messages: partition ids -> per generation and partition [slab staging -> sort -> rank -> active/retired
+split -> message count / offsets / emission] -> inbox routing -> join -> ... -> rank-order scatter.
+
+Every stage that the library exports runs through the C ABI of `lib` (the GPU library or the CPU emulation of the same
+kernel sources); the glue between them (the per-partition sorts, run ranking and the split, which the library
+does differently for partitions resident in HBM) is plain numpy. Test infrastructure only."""
+import numpy as np
+
+import oracle_lib
+
+PILL_RECEIPT = np.uint64(1 << 62)
+KEY62 = np.uint64((1 << 62) - 1)
+SEC_MASK = np.uint64((1 << 31) - 1)
+VAL48 = np.uint64((1 << 48) - 1)
+ABSENT = np.uint64(0xFFFFFFFFFFFFFFFF)
+
+
+def _run_heads(*cols):
+    """index of the head of every run of equal rows (rows are sorted)"""
+    n = cols[0].size
+    head = np.zeros(n, dtype=bool)
+    head[0] = True
+    for c in cols:
+        head[1:] |= c[1:] != c[:-1]
+    idx = np.where(head, np.arange(n), 0)
+    return np.maximum.accumulate(idx), head
+
+
+def build_sa(lib, to_dev, to_host, T, p, key_words=1, pivot_words=2, seed=0, max_generations=64, log=None, join_handle=None):
+    """Returns (sa uint64[n], generations run). `to_dev(np array)` gives an object with .ptr; `to_host(obj)` the array back.
+    log (a list) receives (generation, partition, cohort, survivors, messages, pills) per step. join_handle: a handle
+    whose scratch the join may use to sort the inbox first (csa_join_messages_sorted_dev)."""
+    T = np.ascontiguousarray(T, dtype=np.uint16)
+    n, ell = T.size, 4 * key_words
+    rng = np.random.default_rng(seed)
+    d_T = to_dev(T)
+
+    # ---- partition ids, packed map, partition sizes (src/GPU_SACA.cu:854-1000) ----
+    pivots = oracle_lib.sample_pivots(T, p, pivot_words, rng)
+    bits = oracle_lib.partition_id_bits(p)
+    d_pid = to_dev(np.zeros(n, dtype=np.uint16))
+    d_map = to_dev(np.zeros(((n + 63) // 64) * bits + 1, dtype=np.uint64))
+    d_psz = to_dev(np.zeros(p, dtype=np.uint64))
+    d_piv = to_dev(pivots.reshape(-1) if pivots.size else np.zeros(1, dtype=np.uint64))
+    assert lib.csa_partition_ids_u16_dev(d_T.ptr, n, n, d_piv.ptr if p > 1 else None, pivot_words, p, d_pid.ptr, d_map.ptr,
+                                         d_psz.ptr, None) == 0
+    pid, words, psz = to_host(d_pid), to_host(d_map).copy(), to_host(d_psz)
+    assert int(psz.sum()) == n
+    P_off = np.concatenate([[0], np.cumsum(psz)]).astype(np.int64)
+
+    part = []
+    for q in range(p):
+        suf = np.flatnonzero(pid == q).astype(np.uint64)
+        rng.shuffle(suf)  # a partition's suffixes arrive in no particular order
+        part.append({"suf": suf, "rank": np.zeros(suf.size, dtype=np.uint32), "active": suf.size})
+    inbox = [(np.zeros(0, dtype=np.uint64), np.zeros(0, dtype=np.uint32)) for _ in range(p)]
+
+    gen, ctx = 0, ell
+    while any(pt["active"] > 0 for pt in part):
+        assert gen < max_generations
+        d_map = to_dev(words)
+        outboxes = [([], []) for _ in range(p)]
+        retired_now = []
+        for q in range(p):
+            pt = part[q]
+            a = pt["active"]
+            if a == 0:
+                continue
+            suf, prim = pt["suf"][:a].copy(), pt["rank"][:a].copy()
+            # ---- staging (src/GPU_SACA.cu:1611-1692): keys at generation 0, routing tags always ----
+            d_keys = to_dev(np.zeros(a * key_words, dtype=np.uint64))
+            d_beta = to_dev(np.zeros(a, dtype=np.uint32))
+            d_lanes = to_dev(oracle_lib.u64_to_sa40(suf))
+            assert lib.csa_stage_slab_u16_dev(d_T.ptr, n, d_lanes.ptr, a, key_words, d_map.ptr, p, ctx,
+                                              1 if gen == 0 else 0, d_keys.ptr if gen == 0 else None, d_beta.ptr, None) == 0
+            beta = to_host(d_beta)
+            if gen == 0:
+                keys = to_host(d_keys).reshape(a, key_words)
+                tag = (beta >> np.uint32(16)).astype(np.uint64)
+                # sort by (key, forward tag) (src/GPU_SACA.cu:1165-1227)
+                order = np.lexsort((tag,) + tuple(keys[:, w] for w in reversed(range(key_words))))
+                keys, tag, suf, beta = keys[order], tag[order], suf[order], beta[order]
+                heads, is_head = _run_heads(tag, *[keys[:, w] for w in range(key_words)])
+                rank = heads.astype(np.uint64)  # partition-local: offset of the run's head (include/GPU_SACA.cuh:191-208)
+                K = rank.copy()
+                sa_words = suf | (tag << np.uint64(48))  # the tag rides in the word's top bits (include/GPU_SACA.cuh:116)
+            else:
+                # suffix order, join the inbox (src/GPU_SACA.cu:1769-1835)
+                o = np.argsort(suf, kind="stable")
+                suf, prim, beta = suf[o], prim[o], beta[o]
+                d_K = to_dev(np.full(a, ABSENT))
+                tgt, rk = inbox[q]
+                if tgt.size:
+                    d_tgt, d_rk, d_suf, d_prim = to_dev(oracle_lib.u64_to_sa40(tgt)), to_dev(rk), to_dev(suf), to_dev(prim)
+                    if join_handle is not None:
+                        assert lib.csa_join_messages_sorted_dev(join_handle, d_tgt.ptr, d_rk.ptr, tgt.size, d_suf.ptr, d_prim.ptr,
+                                                                d_K.ptr, a, None) == 0
+                    else:
+                        assert lib.csa_join_messages_dev(d_tgt.ptr, d_rk.ptr, tgt.size, d_suf.ptr, d_prim.ptr, d_K.ptr, a, None) == 0
+                K = to_host(d_K).copy()
+                assert not (K == ABSENT).any(), f"generation {gen}, partition {q}: a cohort member received no message"
+                # sort by (primary, secondary) = key bits [0, 62) (src/GPU_SACA.cu:1841-1871)
+                o = np.argsort(K & KEY62, kind="stable")
+                K, suf, beta = K[o], suf[o], beta[o]
+                key62 = K & KEY62
+                old_prim = key62 >> np.uint64(31)
+                kg, is_head = _run_heads(K)  # full words: tied entries agree on the pill receipt (coherence invariant)
+                pg, _ = _run_heads(old_prim)
+                new_prim = old_prim + (kg - pg).astype(np.uint64)  # include/GPU_SACA.cuh:268-280
+                K = (new_prim << np.uint64(31)) | (K & SEC_MASK) | (K & PILL_RECEIPT)
+                rank = new_prim
+                sa_words = suf
+            nxt_head = np.concatenate([is_head[1:], [True]])
+            active = ~(is_head & nxt_head)  # tied with a neighbour (include/GPU_SACA.cuh:201-207,256-258)
+            # active first, retirees after, in reverse (cub::DevicePartition::Flagged, src/GPU_SACA.cu:1253-1261)
+            perm = np.concatenate([np.flatnonzero(active), np.flatnonzero(~active)[::-1]])
+            sa_words, K, beta, rank, suf = sa_words[perm], K[perm], beta[perm], rank[perm], suf[perm]
+            a_new = int(active.sum())
+            # ---- messages (src/GPU_SACA.cu:1266-1287,1930-1951) ----
+            d_sa, d_Kr, d_b = to_dev(sa_words), to_dev(K), to_dev(beta)
+            d_off = to_dev(np.zeros(p + 1, dtype=np.uint32))
+            packed = 0 if gen == 0 else 1
+            assert lib.csa_count_messages_dev(d_sa.ptr, d_Kr.ptr, d_b.ptr, a, ctx, packed, p, d_off.ptr, None) == 0
+            cnt = to_host(d_off).copy()
+            assert lib.csa_message_offsets_dev(d_off.ptr, p + 1, None) == 0
+            total = int(cnt.sum())
+            d_mt, d_mr = to_dev(np.zeros(5 * max(total, 1), dtype=np.uint8)), to_dev(np.zeros(max(total, 1), dtype=np.uint32))
+            d_act = to_dev(np.array([a_new], dtype=np.uint64))
+            assert lib.csa_emit_messages_dev(d_sa.ptr, d_Kr.ptr, d_b.ptr, a, ctx, packed, d_act.ptr, p, d_mt.ptr, d_mr.ptr, d_off.ptr,
+                                             None) == 0
+            end = to_host(d_off)
+            m_tgt, m_rank = oracle_lib.sa40_to_u64(to_host(d_mt))[:total], to_host(d_mr)[:total]
+            start = 0
+            for dest in range(p):  # the host splits the outbox by the end offsets (src/Partition_Backend.cpp:516-554)
+                e = int(end[dest])
+                outboxes[dest][0].append(m_tgt[start:e])
+                outboxes[dest][1].append(m_rank[start:e])
+                start = e
+            # ---- persist: ranks and suffixes, active first (src/GPU_SACA.cu:1289-1327) ----
+            pt["suf"][:a], pt["rank"][:a] = suf, rank.astype(np.uint32)
+            pt["active"] = a_new
+            retired_now.append(suf[a_new:])
+            if log is not None:
+                log.append((gen, q, a, a_new, total, int((m_rank >> np.uint32(31)).sum())))
+        # retirement flags of this generation's retirees (GPU_SACA::destage_slab, src/GPU_SACA.cu:1695-1711)
+        if retired_now:
+            oracle_lib.set_retired(words, bits, np.concatenate(retired_now))
+        inbox = [(np.concatenate(t) if t else np.zeros(0, dtype=np.uint64), np.concatenate(r) if r else np.zeros(0, dtype=np.uint32))
+                 for t, r in outboxes]
+        gen += 1
+        ctx *= 2
+
+    # ---- every partition to rank order, partitions concatenated (src/GPU_SACA.cu:2107-2164) ----
+    sa = np.zeros(n, dtype=np.uint64)
+    h = lib_handle(lib)
+    try:
+        for q in range(p):
+            m = part[q]["suf"].size
+            if m == 0:
+                continue
+            d_out = to_dev(np.zeros(5 * m, dtype=np.uint8))
+            d_suf, d_rank = to_dev(oracle_lib.u64_to_sa40(part[q]["suf"])), to_dev(part[q]["rank"])
+            rc = lib.csa_scatter_to_rank_order_dev(h, d_suf.ptr, d_rank.ptr, m, d_out.ptr, None)
+            assert rc == 0, f"partition {q}: the ranks are not a permutation"
+            sa[P_off[q]:P_off[q] + m] = oracle_lib.sa40_to_u64(to_host(d_out))
+    finally:
+        lib.csa_destroy(h)
+    return sa, gen
+
+
+def lib_handle(lib):
+    import ctypes as C
+    h = C.c_void_p()
+    assert lib.csa_create(16, 1, C.byref(h)) == 0
+    return h

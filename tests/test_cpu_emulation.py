@@ -198,3 +198,23 @@ def test_emulated_join_matches_the_oracle(emu):
                                           keys2.ctypes.data, n, None)
     emu.csa_destroy(h)
     assert rc == 0 and np.array_equal(keys2, keys)
+
+
+@pytest.mark.parametrize("p,key_words,sigma,n", [(3, 1, 3, 3000), (7, 2, 2, 2500), (5, 1, 1, 400), (4, 1, 2, 2000)])
+def test_multi_partition_pipeline_through_the_emulated_stage_kernels(emu, p, key_words, sigma, n):
+    """Partitions that exchange ranks only through messages: every exported stage kernel (partition ids, slab staging,
+    message count / offsets / emission, join, rank-order scatter) in the reference's order of use; the suffix array that
+    comes out must be the oracle's."""
+    import multi_partition
+    T = texts.random_text(n, sigma, 11 * p + n, sep_every=0)
+    T[-7:] = 0
+    if n == 2000:  # long repeats: many generations, pills forwarded over several of them
+        T[700:1300] = T[:600]
+        T[1500:1900] = T[100:500]
+    log = []
+    sa, gens = multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, p, key_words=key_words,
+                                        log=log)
+    assert np.array_equal(sa, oracle_lib.sa40_to_u64(oracle_lib.build_sa40(T))), (p, key_words, gens)
+    assert gens >= 2
+    if n == 2000:
+        assert gens >= 6 and sum(step[5] for step in log if step[0] >= 1) > 0  # pills travelled in later generations

@@ -87,8 +87,8 @@ def test_join_matches_the_oracle(gpu):
         seed_keys = np.full(n, np.uint64(0xFFFFFFFFFFFFFFFF))
         d_keys = to_dev(seed_keys)
         print(f"  join n={n} messages={tgt.size}", flush=True)
-        assert lib.csa_join_messages_dev(to_dev(oracle_lib.u64_to_sa40(tgt)).ptr, to_dev(rank).ptr, tgt.size, to_dev(sa).ptr,
-                                         to_dev(primary).ptr, d_keys.ptr, n, None) == 0
+        d_tgt, d_rank, d_sa, d_primary = to_dev(oracle_lib.u64_to_sa40(tgt)), to_dev(rank), to_dev(sa), to_dev(primary)  # kept alive
+        assert lib.csa_join_messages_dev(d_tgt.ptr, d_rank.ptr, tgt.size, d_sa.ptr, d_primary.ptr, d_keys.ptr, n, None) == 0
         want = oracle_lib.join_messages(tgt, rank, sa, primary, seed_keys)
         assert np.array_equal(to_host(d_keys), want)
         # the same through the variant that sorts the inbox by target first (scratch of a handle)
@@ -96,7 +96,7 @@ def test_join_matches_the_oracle(gpu):
         with PartitionSorter(max(tgt.size, 16)) as s:
             d_keys2 = to_dev(seed_keys)
             d_lanes = to_dev(oracle_lib.u64_to_sa40(tgt))
-            assert lib.csa_join_messages_sorted_dev(s._h, d_lanes.ptr, to_dev(rank).ptr, tgt.size, to_dev(sa).ptr,
-                                                    to_dev(primary).ptr, d_keys2.ptr, n, None) == 0
+            assert lib.csa_join_messages_sorted_dev(s._h, d_lanes.ptr, d_rank.ptr, tgt.size, d_sa.ptr, d_primary.ptr, d_keys2.ptr, n,
+                                                    None) == 0
             assert np.array_equal(to_host(d_keys2), want)
             assert np.array_equal(to_host(d_lanes), oracle_lib.u64_to_sa40(tgt))  # the inbox is left alone
