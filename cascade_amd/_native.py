@@ -20,7 +20,7 @@ EXPORTS = (
     "csa_pack_keys_u16_dev", "csa_radix_sort_pairs_dev", "csa_verify_sa40_dev", "csa_last_error",
     "csa_partition_id_bits", "csa_partition_ids_u16_dev", "csa_scatter_to_rank_order_dev", "csa_output_cut",
     "csa_stage_slab_u16_dev", "csa_count_messages_dev", "csa_message_offsets_dev", "csa_emit_messages_dev",
-    "csa_join_messages_dev", "csa_join_messages_sorted_dev",
+    "csa_join_messages_dev", "csa_join_messages_sorted_dev", "csa_sort_init_dev", "csa_sort_rerank_dev",
 )
 
 
@@ -101,6 +101,10 @@ def load():
     lib.csa_join_messages_dev.argtypes = [vp, vp, u32, vp, vp, vp, u64, vp]
     lib.csa_join_messages_sorted_dev.restype = i32
     lib.csa_join_messages_sorted_dev.argtypes = [vp, vp, vp, u32, vp, vp, vp, u64, vp]
+    lib.csa_sort_init_dev.restype = i32
+    lib.csa_sort_init_dev.argtypes = [vp, vp, i32, vp, vp, u64, u32, vp, vp, vp, vp, vp, vp, vp]
+    lib.csa_sort_rerank_dev.restype = i32
+    lib.csa_sort_rerank_dev.argtypes = [vp, vp, vp, vp, u64, vp, vp, u32, u64, u32, vp, vp, vp, vp, vp, vp, vp]
     lib.csa_output_cut.restype = None
     lib.csa_output_cut.argtypes = [u64, u64, u64, u64, u64, C.POINTER(u64 * 6)]
     _lib = lib

@@ -6,6 +6,7 @@
 #include "doubling.hpp"
 #include "messages.hpp"
 #include "partition_ids.hpp"
+#include "pipeline_steps.hpp"
 #include "radix_sort.hpp"
 
 #include <cstdarg>
@@ -134,6 +135,7 @@ struct csa_handle {
     u32 epoch = 0;
     u32 xcd_chunk = 0;         // tiles of a radix pass that one XCD takes in a row (0: numbered by arrival)
     u32 defer_min = DEFER_MIN; // lists at least this long use the bucketed rank update (env CASCADE_DEFER_MIN overrides)
+    u64* step64[2] = {nullptr, nullptr}; // two more 8-byte arrays of the capacity, for the per-generation partition steps
     u32 window_min_changed = WINDOW_MIN_CHANGED; // env CASCADE_WINDOW_MIN_CHANGED overrides (0xFFFFFFFF: never)
     std::vector<hipEvent_t> events;
     hipEvent_t ev_gen[CSA_MAX_GENERATIONS + 2] = {};
@@ -1022,6 +1024,223 @@ int csa_stage_slab_u16_dev(const uint16_t* d_text, uint64_t n, const uint8_t* d_
     return CSA_OK;
 }
 
+extern "C++" {
+namespace {
+
+// Shared tail of the two partition steps: the list (keys, suffix words, routing tags) sorted by key is ranked and split
+// into active / retired, the cohort's messages are emitted, ranks and lanes are narrowed for the caller.
+template <bool GEN0>
+int finish_partition_step(Launch& L, const u64* sorted_key0, const u64* sorted_key1, const u64* sorted_words, const u32* sorted_beta,
+                          u64 m, u64 ctx, u32 p, u64* key_r, u64* words_r, u32* beta_r, u32* d_rank_out, u8* d_suf40_out,
+                          u8* d_msg_target, u32* d_msg_rank, u32* d_msg_off, csa_step_result* res)
+{
+    csa_handle* h = L.h;
+    hipStream_t s = L.stream;
+    const RankTables r = rank_tables(h, (u32)m, STEP_TILE);
+    unsigned long long* d_active = reinterpret_cast<unsigned long long*>(h->counts + 8);
+    StepRankArgs ra;
+    ra.key0 = sorted_key0;
+    ra.key1 = sorted_key1;
+    ra.words = sorted_words;
+    ra.beta = sorted_beta;
+    ra.m = m;
+    ra.key_out = key_r;
+    ra.words_out = words_r;
+    ra.beta_out = beta_r;
+    ra.tile_agg = r.tile_agg;
+    ra.tile_splits = r.tile_splits;
+    ra.tile_prefix = r.tile_prefix;
+    ra.slab_total = r.slab_total;
+    ra.slab = r.slab;
+    ra.slabs = r.slabs;
+    ra.active_out = d_active;
+    hipLaunchKernelGGL((step_rank_kernel<GEN0, false>), dim3(r.tiles), dim3(STEP_BLOCK), 0, s, ra);
+    hipLaunchKernelGGL(rerank_scan_kernel, dim3(r.slabs), dim3(1024), 0, s, r.tile_agg, r.tile_prefix, r.tiles, r.slab, r.slab_total,
+                       r.tile_splits);
+    hipLaunchKernelGGL((step_rank_kernel<GEN0, true>), dim3(r.tiles), dim3(STEP_BLOCK), 0, s, ra);
+    HIP_TRY(hipGetLastError());
+    // the cohort's messages, collated by destination (src/GPU_SACA.cu:1266-1287,1930-1951)
+    MessageArgs ma;
+    int rc = fill_message_args(ma, "partition step", key_r ? words_r : nullptr, key_r, beta_r, m, ctx, GEN0 ? 0 : 1, p);
+    if (rc)
+        return rc;
+    HIP_TRY(hipMemsetAsync(d_msg_off, 0, ((u64)p + 1) * sizeof(u32), s));
+    ma.msg_off = d_msg_off;
+    const u32 grid = ma.tiles < 4096u ? ma.tiles : 4096u;
+    hipLaunchKernelGGL(count_messages_kernel, dim3(grid), dim3(MSG_BLOCK), 0, s, ma);
+    hipLaunchKernelGGL(message_offsets_kernel, dim3(1), dim3(1024), 0, s, d_msg_off, p + 1);
+    ma.active_sz = d_active;
+    ma.msg_target = d_msg_target;
+    ma.msg_rank = d_msg_rank;
+    hipLaunchKernelGGL(emit_messages_kernel, dim3(grid), dim3(MSG_BLOCK), 0, s, ma);
+    // what the caller persists: narrowed ranks and lanes (src/GPU_SACA.cu:1289-1305)
+    hipLaunchKernelGGL(narrow_and_pack_kernel, dim3((u32)((m + 255) / 256)), dim3(256), 0, s, (const u64*)key_r, (const u64*)words_r, m,
+                       GEN0 ? 0 : 1, d_rank_out, d_suf40_out);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpyAsync(h->h_pinned + 8, h->counts + 8, 2 * sizeof(u32), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipMemcpyAsync(h->h_pinned + 10, d_msg_off + (p - 1), sizeof(u32), hipMemcpyDeviceToHost, s));
+    rc = read_counts(L, nullptr);
+    if (rc)
+        return rc;
+    if (res) {
+        res->active = (u64)h->h_pinned[8] | ((u64)h->h_pinned[9] << 32);
+        res->messages = h->h_pinned[10];
+    }
+    return CSA_OK;
+}
+
+int check_step_args(csa_handle* h, const char* who, u64 m, u32 p, const void* a, const void* b, const void* c, const void* d)
+{
+    if (!h)
+        return fail(CSA_ERR_ARG, "%s: null handle", who);
+    if (p < 1 || p > 32768u)
+        return fail(CSA_ERR_ARG, "%s: p = %u is outside [1, 32768]", who, p);
+    if (m > h->cap)
+        return fail(CSA_ERR_ARG, "%s: %llu suffixes exceed the handle's capacity %llu", who, (unsigned long long)m,
+                    (unsigned long long)h->cap);
+    if (m && (!a || !b || !c || !d))
+        return fail(CSA_ERR_ARG, "%s: null buffer", who);
+    for (int i = 0; i < 2; ++i)
+        if (!h->step64[i]) {
+            const hipError_t e = hipMalloc((void**)&h->step64[i], (h->cap ? h->cap : 1) * sizeof(u64));
+            if (e != hipSuccess)
+                return fail(CSA_ERR_HIP, "%s: %s while allocating the step scratch", who, hipGetErrorString(e));
+        }
+    return CSA_OK;
+}
+
+} // namespace
+} // extern "C++"
+
+int csa_sort_init_dev(csa_handle* h, const uint64_t* d_keys, int key_words, const uint8_t* d_suf40, const uint32_t* d_beta,
+                      uint64_t m, uint32_t p, uint32_t* d_rank_out, uint8_t* d_suf40_out, uint8_t* d_msg_target,
+                      uint32_t* d_msg_rank, uint32_t* d_msg_off, void* stream, csa_step_result* res)
+{
+    if (key_words != 1 && key_words != 2)
+        return fail(CSA_ERR_ARG, "csa_sort_init_dev: key_words must be 1 or 2");
+    int rc = check_step_args(h, "csa_sort_init_dev", m, p, d_keys, d_suf40, d_beta, d_msg_off);
+    if (rc)
+        return rc;
+    if (res)
+        res->active = res->messages = 0;
+    if (m == 0) {
+        HIP_TRY(hipMemsetAsync(d_msg_off, 0, ((u64)p + 1) * sizeof(u32), (hipStream_t)stream));
+        return CSA_OK;
+    }
+    if (!d_rank_out || !d_suf40_out || !d_msg_target || !d_msg_rank)
+        return fail(CSA_ERR_ARG, "csa_sort_init_dev: null output buffer");
+    Launch L;
+    L.h = h;
+    L.stream = (hipStream_t)stream;
+    L.flags = 0;
+    L.stats = nullptr;
+    hipStream_t s = L.stream;
+    const u32 blocks = (u32)((m + 255) / 256);
+    HIP_TRY(hipMemsetAsync(h->counts, 0, 4 * sizeof(u32), s));
+    // stable LSD sort by (key words, forward tag): the tag first, then the words from the least significant one
+    // (src/GPU_SACA.cu:1165-1227), always on (64-bit key, permutation) pairs
+    u64* K[2] = {h->key[0], h->key[1]};
+    u32* P[2] = {h->idx[0], h->idx[1]};
+    int kc = 0, pc = 0; // the arrays that hold the current keys / permutation
+    hipLaunchKernelGGL(iota_kernel, dim3(blocks), dim3(256), 0, s, P[pc], m);
+    hipLaunchKernelGGL(tag_keys_kernel, dim3(blocks), dim3(256), 0, s, d_beta, m, K[kc]);
+    int in_out = 0, passes = 0;
+    rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, K[kc], P[pc], K[kc ^ 1], P[pc ^ 1], (u32)m, make_plan(0, 16), &in_out, &passes);
+    if (rc)
+        return rc;
+    pc ^= in_out;
+    for (int w = key_words - 1; w >= 0; --w) {
+        hipLaunchKernelGGL(gather_u64_kernel, dim3(blocks), dim3(256), 0, s, (const u64*)d_keys, (const u32*)P[pc], m, (u32)key_words,
+                           (u32)w, K[0]);
+        rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, K[0], P[pc], K[1], P[pc ^ 1], (u32)m, make_plan(0, 64), &in_out, &passes);
+        if (rc)
+            return rc;
+        kc = in_out;
+        pc ^= in_out;
+    }
+    // sorted: key word 0 in K[kc], the permutation in P[pc]
+    u64* sorted_key1 = nullptr;
+    if (key_words == 2) {
+        sorted_key1 = K[kc ^ 1];
+        hipLaunchKernelGGL(gather_u64_kernel, dim3(blocks), dim3(256), 0, s, (const u64*)d_keys, (const u32*)P[pc], m, 2u, 1u, sorted_key1);
+    }
+    u64* sorted_words = h->key[2];
+    u32* sorted_beta = h->idx[2];
+    hipLaunchKernelGGL(unpack_words_kernel, dim3(blocks), dim3(256), 0, s, d_suf40, d_beta, (const u32*)P[pc], m, 1, sorted_words,
+                       sorted_beta);
+    HIP_TRY(hipGetLastError());
+    return finish_partition_step<true>(L, K[kc], sorted_key1, sorted_words, sorted_beta, m, 4ull * (u64)key_words, p, h->step64[0],
+                                       h->step64[1], h->idx[3], d_rank_out, d_suf40_out, d_msg_target, d_msg_rank, d_msg_off, res);
+}
+
+int csa_sort_rerank_dev(csa_handle* h, const uint32_t* d_rank, const uint8_t* d_suf40, const uint32_t* d_beta, uint64_t m,
+                        const uint8_t* d_inbox_target, const uint32_t* d_inbox_rank, uint32_t inbox_sz, uint64_t ctx,
+                        uint32_t p, uint32_t* d_rank_out, uint8_t* d_suf40_out, uint8_t* d_msg_target, uint32_t* d_msg_rank,
+                        uint32_t* d_msg_off, void* stream, csa_step_result* res)
+{
+    int rc = check_step_args(h, "csa_sort_rerank_dev", m, p, d_rank, d_suf40, d_beta, d_msg_off);
+    if (rc)
+        return rc;
+    if (res)
+        res->active = res->messages = 0;
+    if (m == 0) {
+        HIP_TRY(hipMemsetAsync(d_msg_off, 0, ((u64)p + 1) * sizeof(u32), (hipStream_t)stream));
+        return CSA_OK;
+    }
+    if (!d_rank_out || !d_suf40_out || !d_msg_target || !d_msg_rank || (inbox_sz && (!d_inbox_target || !d_inbox_rank)))
+        return fail(CSA_ERR_ARG, "csa_sort_rerank_dev: null buffer");
+    Launch L;
+    L.h = h;
+    L.stream = (hipStream_t)stream;
+    L.flags = 0;
+    L.stats = nullptr;
+    hipStream_t s = L.stream;
+    const u32 blocks = (u32)((m + 255) / 256);
+    HIP_TRY(hipMemsetAsync(h->counts, 0, 4 * sizeof(u32), s));
+    u64* K[2] = {h->key[0], h->key[1]};
+    u32* P[2] = {h->idx[0], h->idx[1]};
+    // 1. the cohort in suffix order, so that messages can be joined by search (src/GPU_SACA.cu:1769-1800)
+    hipLaunchKernelGGL(unpack_words_kernel, dim3(blocks), dim3(256), 0, s, d_suf40, (const u32*)nullptr, (const u32*)nullptr, m, 0, K[0],
+                       (u32*)nullptr);
+    hipLaunchKernelGGL(iota_kernel, dim3(blocks), dim3(256), 0, s, P[0], m);
+    int in_out = 0, passes = 0;
+    rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, K[0], P[0], K[1], P[1], (u32)m, make_plan(0, 40), &in_out, &passes);
+    if (rc)
+        return rc;
+    u64* words_by_suffix = K[in_out];
+    u64* free64 = K[in_out ^ 1];
+    u32* perm = P[in_out];
+    u32* primary_by_suffix = h->idx[2];
+    u32* beta_by_suffix = h->idx[3];
+    hipLaunchKernelGGL(gather_u32_kernel, dim3(blocks), dim3(256), 0, s, d_rank, (const u32*)perm, m, primary_by_suffix);
+    hipLaunchKernelGGL(gather_u32_kernel, dim3(blocks), dim3(256), 0, s, d_beta, (const u32*)perm, m, beta_by_suffix);
+    // 2. composite keys from the inbox: primary << 31 | received rank, all ones where nothing arrives
+    //    (src/GPU_SACA.cu:1803-1835)
+    u64* keys = h->key[2];
+    hipLaunchKernelGGL(fill_u64_kernel, dim3(blocks), dim3(256), 0, s, keys, m, ~0ull);
+    if (inbox_sz)
+        hipLaunchKernelGGL(join_messages_kernel, dim3((inbox_sz + 255u) / 256u), dim3(256), 0, s, d_inbox_target, (const u64*)nullptr,
+                           d_inbox_rank, inbox_sz, (const u64*)words_by_suffix, (const u32*)primary_by_suffix, keys, m);
+    HIP_TRY(hipGetLastError());
+    // 3. sort by (primary, secondary): key bits [0, 62) (src/GPU_SACA.cu:1841-1871)
+    hipLaunchKernelGGL(iota_kernel, dim3(blocks), dim3(256), 0, s, P[0], m);
+    rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, keys, P[0], free64, P[1], (u32)m, make_plan(0, 62), &in_out, &passes);
+    if (rc)
+        return rc;
+    u64* sorted_keys = in_out ? free64 : keys;
+    u64* spare64 = in_out ? keys : free64;
+    perm = P[in_out];
+    u64* sorted_words = h->step64[0];
+    u32* sorted_beta = h->idx[4];
+    hipLaunchKernelGGL(gather_u64_kernel, dim3(blocks), dim3(256), 0, s, (const u64*)words_by_suffix, (const u32*)perm, m, 1u, 0u,
+                       sorted_words);
+    hipLaunchKernelGGL(gather_u32_kernel, dim3(blocks), dim3(256), 0, s, (const u32*)beta_by_suffix, (const u32*)perm, m, sorted_beta);
+    HIP_TRY(hipGetLastError());
+    // 4. refine, split, messages, narrow
+    return finish_partition_step<false>(L, sorted_keys, nullptr, sorted_words, sorted_beta, m, ctx, p, h->step64[1], spare64,
+                                        primary_by_suffix, d_rank_out, d_suf40_out, d_msg_target, d_msg_rank, d_msg_off, res);
+}
+
 int csa_scatter_to_rank_order_dev(csa_handle* h, const uint8_t* d_suf, const uint32_t* d_rank, uint64_t part_sz,
                                   uint8_t* d_sa40, void* stream)
 {
@@ -1171,6 +1390,8 @@ void csa_destroy(csa_handle* h)
     (void)hipFree(h->ghist);
     (void)hipFree(h->digit_base);
     (void)hipFree(h->tickets);
+    (void)hipFree(h->step64[0]);
+    (void)hipFree(h->step64[1]);
     (void)hipFree(h->counts);
     if (h->h_pinned)
         (void)hipHostFree(h->h_pinned);

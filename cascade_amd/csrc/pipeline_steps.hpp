@@ -1,0 +1,237 @@
+// Kernels of the per-generation partition steps that keep the reference's exchange scheme: a partition arrives as
+// (key | rank, suffix lane, routing tags [, inbox]) and leaves as (rank, suffix lane) in "active first, retired after"
+// order plus an outbox of rank messages (reference: GPU_SACA::sort_and_init_rank_and_filter and
+// GPU_SACA::sort_and_re_rank_and_filter, src/GPU_SACA.cu:1112-1331 and 1715-1995). The sorts are the library's radix
+// sort on (64-bit key, 32-bit permutation) pairs, as the reference sorts with cub; the kernels here are the glue:
+// lane unpacking, gathers through the permutation, run ranking with the active/retired split, narrowing.
+#pragma once
+
+#include "device_utils.hpp"
+#include "doubling.hpp"
+#include "messages.hpp"
+
+namespace csa {
+
+constexpr int STEP_BLOCK = 256;
+constexpr int STEP_ITEMS = 4;
+constexpr int STEP_TILE = STEP_BLOCK * STEP_ITEMS;
+constexpr u64 STEP_KEY62 = (1ull << 62) - 1ull;    // (primary, secondary): the sorted bits of a composite key
+constexpr u64 STEP_SECONDARY = (1ull << 31) - 1ull;
+
+__global__ __launch_bounds__(256) void iota_kernel(u32* p, u64 count)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i < count)
+        p[i] = (u32)i;
+}
+
+// keys[i] = forward tag of suffix i: the high half of its routing-tag pair (include/bit-layout.hpp:141-145)
+__global__ __launch_bounds__(256) void tag_keys_kernel(const u32* __restrict__ beta, u64 count, u64* __restrict__ keys)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i < count)
+        keys[i] = beta[i] >> 16;
+}
+
+// dst[i] = src[perm[i] * stride + offset]
+__global__ __launch_bounds__(256) void gather_u64_kernel(const u64* __restrict__ src, const u32* __restrict__ perm, u64 count,
+                                                         u32 stride, u32 offset, u64* __restrict__ dst)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i < count)
+        dst[i] = src[(u64)perm[i] * stride + offset];
+}
+
+__global__ __launch_bounds__(256) void gather_u32_kernel(const u32* __restrict__ src, const u32* __restrict__ perm, u64 count,
+                                                         u32* __restrict__ dst)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i < count)
+        dst[i] = src[perm[i]];
+}
+
+// words[i] = suffix of lane perm[i] (or i), with the forward tag of its routing tags in the top 16 bits when with_tag
+// (reference: unpack_tagged_lanes_kernel / unpack_lanes_kernel, include/GPU_SACA.cuh:94-119); beta_out[i] = beta[perm[i]].
+__global__ __launch_bounds__(256) void unpack_words_kernel(const u8* __restrict__ lanes, const u32* __restrict__ beta,
+                                                           const u32* __restrict__ perm, u64 count, int with_tag,
+                                                           u64* __restrict__ words, u32* __restrict__ beta_out)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= count)
+        return;
+    const u64 j = perm ? perm[i] : i;
+    u64 v = 0;
+#pragma unroll
+    for (int b = 0; b < 5; ++b)
+        v |= (u64)lanes[5 * j + b] << (8 * b);
+    const u32 bt = beta ? beta[j] : 0u;
+    words[i] = with_tag ? (v | ((u64)(bt >> 16) << 48)) : v;
+    if (beta_out)
+        beta_out[i] = bt;
+}
+
+// Run ranking with the active / retired split, in the three launches of the rank step (count, rerank_scan_kernel, apply).
+// Generation 0: the list is sorted by (key words, forward tag); rank = offset of the head of the run of equal
+// (key, tag), stored as a plain rank (include/GPU_SACA.cuh:191-208). Generation t: the list is sorted by the composite
+// key; refined primary = primary + (head of the key run - head of the primary run), secondary and pill receipt kept
+// (include/GPU_SACA.cuh:218-280). An entry is active iff its run is longer than one. Active entries go first, in
+// order; retired ones follow (reference: cub::DevicePartition::Flagged, which reverses them: their order carries nothing).
+struct StepRankArgs {
+    const u64* key0;  // generation 0: sorted key word 0; generation t: sorted composite keys
+    const u64* key1;  // generation 0 with 128-bit keys: sorted key word 1, else null
+    const u64* words; // suffix words in the same order (generation 0: forward tag in the top 16 bits)
+    const u32* beta;
+    u64 m;
+    u64* key_out;
+    u64* words_out;
+    u32* beta_out;
+    u32* tile_agg;    // [tiles][4]
+    u32* tile_splits; // [tiles]
+    u32* tile_prefix; // [tiles][4]
+    u32* slab_total;  // [RERANK_SLABS][5]
+    u32 slab;
+    u32 slabs;
+    unsigned long long* active_out; // size of the active set
+};
+
+template <bool GEN0>
+__device__ __forceinline__ bool step_same_key(const StepRankArgs& a, u64 i, u64 j)
+{
+    if (GEN0)
+        return a.key0[i] == a.key0[j] && (!a.key1 || a.key1[i] == a.key1[j]) && (a.words[i] >> 48) == (a.words[j] >> 48);
+    return a.key0[i] == a.key0[j]; // whole words: tied entries agree on the pill receipt
+}
+
+template <bool GEN0>
+__device__ __forceinline__ bool step_same_primary(const StepRankArgs& a, u64 i, u64 j)
+{
+    if (GEN0)
+        return true; // one primary group: the partition
+    return ((a.key0[i] & STEP_KEY62) >> 31) == ((a.key0[j] & STEP_KEY62) >> 31);
+}
+
+template <bool GEN0, bool APPLY>
+__global__ __launch_bounds__(STEP_BLOCK) void step_rank_kernel(StepRankArgs a)
+{
+    constexpr int WAVES = STEP_BLOCK / WAVE;
+    __shared__ u32 s_w[WAVES][3];
+    const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
+    const u32 tile = blockIdx.x;
+    const u64 base = (u64)tile * STEP_TILE + (u64)t * STEP_ITEMS;
+    // heads are 1-based positions (0 = none so far)
+    bool kh[STEP_ITEMS + 1], ph[STEP_ITEMS];
+    u32 la = 0, lb = 0, lact = 0;
+#pragma unroll
+    for (int k = 0; k < STEP_ITEMS + 1; ++k) {
+        const u64 i = base + k;
+        kh[k] = i < a.m ? (i == 0 || !step_same_key<GEN0>(a, i, i - 1)) : true; // the end of the list closes the last run
+    }
+#pragma unroll
+    for (int k = 0; k < STEP_ITEMS; ++k) {
+        const u64 i = base + k;
+        ph[k] = i < a.m && (i == 0 || !step_same_primary<GEN0>(a, i, i - 1));
+        if (i < a.m) {
+            if (kh[k])
+                la = (u32)i + 1u;
+            if (ph[k])
+                lb = (u32)i + 1u;
+            lact += (kh[k] && kh[k + 1]) ? 0u : 1u;
+        }
+    }
+    const u32 ia = wave_incl_max(la), ib = wave_incl_max(lb), ic = wave_incl_sum(lact);
+    if (lane == 63u) {
+        s_w[w][0] = ia;
+        s_w[w][1] = ib;
+        s_w[w][2] = ic;
+    }
+    __syncthreads();
+    u32 xa = __shfl_up(ia, 1), xb = __shfl_up(ib, 1), xc = __shfl_up(ic, 1);
+    if (lane == 0)
+        xa = xb = xc = 0;
+    u32 ta = 0, tb = 0, tc = 0;
+    for (u32 ww = 0; ww < WAVES; ++ww) {
+        if (ww < w) {
+            xa = xa > s_w[ww][0] ? xa : s_w[ww][0];
+            xb = xb > s_w[ww][1] ? xb : s_w[ww][1];
+            xc += s_w[ww][2];
+        }
+        ta = ta > s_w[ww][0] ? ta : s_w[ww][0];
+        tb = tb > s_w[ww][1] ? tb : s_w[ww][1];
+        tc += s_w[ww][2];
+    }
+    if (!APPLY) {
+        if (t == 0) {
+            a.tile_agg[(u64)tile * 4 + 0] = ta;
+            a.tile_agg[(u64)tile * 4 + 1] = tb;
+            a.tile_agg[(u64)tile * 4 + 2] = tc;
+            a.tile_agg[(u64)tile * 4 + 3] = 0;
+            a.tile_splits[tile] = 0;
+        }
+        return;
+    }
+    u32 pre_a = a.tile_prefix[(u64)tile * 4 + 0], pre_b = a.tile_prefix[(u64)tile * 4 + 1];
+    u32 pre_c = a.tile_prefix[(u64)tile * 4 + 2];
+    u32 total_active = 0;
+    for (u32 sl = 0; sl < a.slabs; ++sl) {
+        if (sl < tile / a.slab) {
+            const u32 sa_ = a.slab_total[sl * 5 + 0], sb_ = a.slab_total[sl * 5 + 1];
+            pre_a = pre_a > sa_ ? pre_a : sa_;
+            pre_b = pre_b > sb_ ? pre_b : sb_;
+            pre_c += a.slab_total[sl * 5 + 2];
+        }
+        total_active += a.slab_total[sl * 5 + 2];
+    }
+    if (tile == 0 && t == 0)
+        *a.active_out = total_active;
+    u32 ra = xa > pre_a ? xa : pre_a, rb = xb > pre_b ? xb : pre_b;
+    u32 act_before = pre_c + xc; // active entries before this thread's first
+#pragma unroll
+    for (int k = 0; k < STEP_ITEMS; ++k) {
+        const u64 i = base + k;
+        if (i >= a.m)
+            continue;
+        if (kh[k])
+            ra = (u32)i + 1u;
+        if (ph[k])
+            rb = (u32)i + 1u;
+        const bool active = !(kh[k] && kh[k + 1]);
+        const u64 old = a.key0[i];
+        u64 key;
+        if (GEN0) {
+            key = (u64)(ra - 1u); // plain rank: offset of the run's head
+        } else {
+            const u64 primary = ((old & STEP_KEY62) >> 31) + (u64)(ra - rb);
+            key = (primary << 31) | (old & STEP_SECONDARY) | (old & MSG_PILL_RECEIPT);
+        }
+        const u64 dest = active ? (u64)act_before : (u64)total_active + (i - act_before);
+        a.key_out[dest] = key;
+        a.words_out[dest] = a.words[i];
+        a.beta_out[dest] = a.beta[i];
+        act_before += active ? 1u : 0u;
+    }
+}
+
+// What a step persists per suffix: its partition-local rank narrowed to 32 bits and its 5-byte lane
+// (reference: extract_primary_keys_kernel, include/GPU_SACA.cuh:397-409; pack_lanes_kernel, :126-133).
+__global__ __launch_bounds__(256) void narrow_and_pack_kernel(const u64* __restrict__ keys, const u64* __restrict__ words, u64 count,
+                                                              int packed, u32* __restrict__ rank_out, u8* __restrict__ lanes_out)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= count)
+        return;
+    const u64 k = keys[i];
+    rank_out[i] = packed ? (u32)((k & STEP_KEY62) >> 31) : (u32)k;
+    const u64 v = words[i];
+#pragma unroll
+    for (int b = 0; b < 5; ++b)
+        lanes_out[5 * i + b] = (u8)(v >> (8 * b));
+}
+
+__global__ __launch_bounds__(256) void fill_u64_kernel(u64* p, u64 count, u64 v)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i < count)
+        p[i] = v;
+}
+
+} // namespace csa

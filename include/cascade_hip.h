@@ -184,6 +184,42 @@ int csa_join_messages_dev(const uint8_t* d_msg_target, const uint32_t* d_msg_ran
 int csa_join_messages_sorted_dev(csa_handle* h, const uint8_t* d_msg_target, const uint32_t* d_msg_rank, uint32_t msg_c,
                                  const uint64_t* d_sa, const uint32_t* d_primary, uint64_t* d_keys, uint64_t n, void* stream);
 
+/* ---- per-generation steps of a partition that exchanges ranks through messages ---- */
+
+typedef struct csa_step_result {
+    uint64_t active;   /* size of the partition's new active set: entries [0, active) of the outputs */
+    uint64_t messages; /* messages in the outbox */
+} csa_step_result;
+
+/* Generation 0 of one partition of m suffixes (m <= the handle's capacity), everything resident in HBM:
+ *   in : d_keys[i * key_words + w] packed K-gram words, d_suf40 5-byte lanes, d_beta routing-tag pairs (forward tag in
+ *        the high half), in any order: what csa_stage_slab_u16_dev (or the reference's stage_slab) produces;
+ *   out: d_rank_out[i] partition-local ranks (offset of the head of the run of equal (key, forward tag)) and
+ *        d_suf40_out lanes, the tied ("active") suffixes first, in sorted order, the retired ones after them;
+ *        the outbox: 5-byte targets, ranks (MSB = the sender retired), d_msg_off[q] = exclusive END of the group bound
+ *        for partition q (p + 1 counters); ctx = 4 * key_words symbols were resolved.
+ * The outbox needs room for m messages. The call returns after the stream has finished; res may be NULL.
+ * The handle lends its sort scratch and, from the first call on, two more 8-byte arrays of its capacity.
+ * Replaces GPU_SACA::sort_and_init_rank_and_filter (include/GPU_SACA.hpp:272, src/GPU_SACA.cu:1112-1331) between the
+ * upload of the slabs and their download. */
+int csa_sort_init_dev(csa_handle* h, const uint64_t* d_keys, int key_words, const uint8_t* d_suf40, const uint32_t* d_beta,
+                      uint64_t m, uint32_t p, uint32_t* d_rank_out, uint8_t* d_suf40_out, uint8_t* d_msg_target,
+                      uint32_t* d_msg_rank, uint32_t* d_msg_off, void* stream, csa_step_result* res);
+
+/* Generation t >= 1 (context ctx = ell * 2^t) of one partition's active set:
+ *   in : d_rank partition-local ranks, d_suf40 lanes, d_beta routing-tag pairs (route of suffix - ctx | route of
+ *        suffix - ctx / 2 << 16), in any order; the inbox (targets, ranks) of the messages sent to this partition at the
+ *        end of the previous generation, in any order;
+ *   out: as csa_sort_init_dev, ranks refined by (primary, received rank); the outbox needs room for 2 * m messages
+ *        (payloads and forwarded pills).
+ * A cohort member that received no message sorts with an all-ones secondary, as in the reference (the exchange
+ * scheme guarantees there is none).
+ * Replaces GPU_SACA::sort_and_re_rank_and_filter (include/GPU_SACA.hpp:279, src/GPU_SACA.cu:1715-1995). */
+int csa_sort_rerank_dev(csa_handle* h, const uint32_t* d_rank, const uint8_t* d_suf40, const uint32_t* d_beta, uint64_t m,
+                        const uint8_t* d_inbox_target, const uint32_t* d_inbox_rank, uint32_t inbox_sz, uint64_t ctx,
+                        uint32_t p, uint32_t* d_rank_out, uint8_t* d_suf40_out, uint8_t* d_msg_target, uint32_t* d_msg_rank,
+                        uint32_t* d_msg_off, void* stream, csa_step_result* res);
+
 /* ---- the step after the partition sort, for partitions that come back as (suffix, local rank) pairs ---- */
 
 /* d_sa40 entry rank[i] = d_suf entry i for i in [0, part_sz): 5-byte little-endian lanes in, lanes in rank order out.

@@ -28,10 +28,13 @@ def _run_heads(*cols):
     return np.maximum.accumulate(idx), head
 
 
-def build_sa(lib, to_dev, to_host, T, p, key_words=1, pivot_words=2, seed=0, max_generations=64, log=None, join_handle=None):
+def build_sa(lib, to_dev, to_host, T, p, key_words=1, pivot_words=2, seed=0, max_generations=64, log=None, join_handle=None,
+             step_handle=None):
     """Returns (sa uint64[n], generations run). `to_dev(np array)` gives an object with .ptr; `to_host(obj)` the array back.
     log (a list) receives (generation, partition, cohort, survivors, messages, pills) per step. join_handle: a handle
-    whose scratch the join may use to sort the inbox first (csa_join_messages_sorted_dev)."""
+    whose scratch the join may use to sort the inbox first (csa_join_messages_sorted_dev). step_handle: a handle of at
+    least the largest partition's capacity; with it, each partition step is ONE call of csa_sort_init_dev /
+    csa_sort_rerank_dev (sorts, ranking, split and messages inside the library) instead of numpy glue between stages."""
     T = np.ascontiguousarray(T, dtype=np.uint16)
     n, ell = T.size, 4 * key_words
     rng = np.random.default_rng(seed)
@@ -76,6 +79,42 @@ def build_sa(lib, to_dev, to_host, T, p, key_words=1, pivot_words=2, seed=0, max
             assert lib.csa_stage_slab_u16_dev(d_T.ptr, n, d_lanes.ptr, a, key_words, d_map.ptr, p, ctx,
                                               1 if gen == 0 else 0, d_keys.ptr if gen == 0 else None, d_beta.ptr, None) == 0
             beta = to_host(d_beta)
+            if step_handle is not None:
+                # ---- the whole step inside the library (src/GPU_SACA.cu:1112-1331 / 1715-1995) ----
+                import ctypes as C
+
+                class StepResult(C.Structure):
+                    _fields_ = [("active", C.c_uint64), ("messages", C.c_uint64)]
+                res = StepResult()
+                d_rank_out, d_suf_out = to_dev(np.zeros(a, dtype=np.uint32)), to_dev(np.zeros(5 * a, dtype=np.uint8))
+                d_mt, d_mr = to_dev(np.zeros(5 * 2 * a, dtype=np.uint8)), to_dev(np.zeros(2 * a, dtype=np.uint32))
+                d_off = to_dev(np.zeros(p + 1, dtype=np.uint32))
+                if gen == 0:
+                    rc = lib.csa_sort_init_dev(step_handle, d_keys.ptr, key_words, d_lanes.ptr, d_beta.ptr, a, p, d_rank_out.ptr,
+                                               d_suf_out.ptr, d_mt.ptr, d_mr.ptr, d_off.ptr, None, C.byref(res))
+                else:
+                    tgt, rk = inbox[q]
+                    d_tgt, d_rk, d_prim = to_dev(oracle_lib.u64_to_sa40(tgt)), to_dev(rk), to_dev(prim)
+                    rc = lib.csa_sort_rerank_dev(step_handle, d_prim.ptr, d_lanes.ptr, d_beta.ptr, a, d_tgt.ptr if tgt.size else None,
+                                                 d_rk.ptr if tgt.size else None, tgt.size, ctx, p, d_rank_out.ptr, d_suf_out.ptr,
+                                                 d_mt.ptr, d_mr.ptr, d_off.ptr, None, C.byref(res))
+                assert rc == 0, lib.csa_last_error()
+                a_new, total = int(res.active), int(res.messages)
+                end = to_host(d_off)
+                assert total == int(end[p - 1])
+                m_tgt, m_rank = oracle_lib.sa40_to_u64(to_host(d_mt))[:total], to_host(d_mr)[:total]
+                start = 0
+                for dest in range(p):
+                    e = int(end[dest])
+                    outboxes[dest][0].append(m_tgt[start:e])
+                    outboxes[dest][1].append(m_rank[start:e])
+                    start = e
+                pt["suf"][:a], pt["rank"][:a] = oracle_lib.sa40_to_u64(to_host(d_suf_out)), to_host(d_rank_out)
+                pt["active"] = a_new
+                retired_now.append(pt["suf"][a_new:a].copy())
+                if log is not None:
+                    log.append((gen, q, a, a_new, total, int((m_rank >> np.uint32(31)).sum())))
+                continue
             if gen == 0:
                 keys = to_host(d_keys).reshape(a, key_words)
                 tag = (beta >> np.uint32(16)).astype(np.uint64)

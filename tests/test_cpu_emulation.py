@@ -35,6 +35,8 @@ def emu():
     lib.csa_emit_messages_dev.argtypes = [vp, vp, vp, u64, u64, i32, vp, u32, vp, vp, vp, vp]
     lib.csa_join_messages_dev.argtypes = [vp, vp, u32, vp, vp, vp, u64, vp]
     lib.csa_join_messages_sorted_dev.argtypes = [vp, vp, vp, u32, vp, vp, vp, u64, vp]
+    lib.csa_sort_init_dev.argtypes = [vp, vp, i32, vp, vp, u64, u32, vp, vp, vp, vp, vp, vp, vp]
+    lib.csa_sort_rerank_dev.argtypes = [vp, vp, vp, vp, u64, vp, vp, u32, u64, u32, vp, vp, vp, vp, vp, vp, vp]
     return lib
 
 
@@ -218,3 +220,26 @@ def test_multi_partition_pipeline_through_the_emulated_stage_kernels(emu, p, key
     assert gens >= 2
     if n == 2000:
         assert gens >= 6 and sum(step[5] for step in log if step[0] >= 1) > 0  # pills travelled in later generations
+
+
+@pytest.mark.parametrize("p,key_words,sigma,n", [(5, 2, 2, 900), (4, 1, 2, 1300)])
+def test_multi_partition_pipeline_with_the_emulated_step_entries(emu, p, key_words, sigma, n):
+    """The same pipeline with each partition step as one call of csa_sort_init_dev / csa_sort_rerank_dev."""
+    import multi_partition
+    T = texts.random_text(n, sigma, 13 * p + n, sep_every=0)
+    T[-7:] = 0
+    if key_words == 1:  # long repeats: many generations, pills forwarded
+        T[500:900] = T[:400]
+        T[1000:1250] = T[100:350]
+    h = C.c_void_p()
+    assert emu.csa_create(n, 1, C.byref(h)) == 0
+    log, glue_log = [], []
+    try:
+        sa, gens = multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, p, key_words=key_words,
+                                            log=log, step_handle=h)
+    finally:
+        emu.csa_destroy(h)
+    assert np.array_equal(sa, oracle_lib.sa40_to_u64(oracle_lib.build_sa40(T))), (p, key_words, gens)
+    # the same run with numpy glue between the stages: the same cohorts, survivors and message counts at every step
+    multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, p, key_words=key_words, log=glue_log)
+    assert log == glue_log

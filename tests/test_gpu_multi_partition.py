@@ -33,8 +33,11 @@ def gpu():
     return _native.load(), to_dev, to_host
 
 
-@pytest.mark.parametrize("p,key_words,sorted_join", [(3, 1, False), (16, 1, True), (33, 2, False)])
-def test_partitions_that_only_exchange_messages_build_the_oracles_suffix_array(gpu, p, key_words, sorted_join):
+@pytest.mark.parametrize("p,key_words,sorted_join,steps", [(3, 1, False, False), (16, 1, True, False), (33, 2, False, False),
+                                                           (3, 1, False, True), (16, 2, False, True), (40, 1, False, True)])
+def test_partitions_that_only_exchange_messages_build_the_oracles_suffix_array(gpu, p, key_words, sorted_join, steps):
+    """steps = False: numpy glue between the exported stage kernels; True: each partition step is one call of
+    csa_sort_init_dev / csa_sort_rerank_dev."""
     lib, to_dev, to_host = gpu
     n = 120000
     T = texts.random_text(n, 4, 7 * p, sep_every=0)
@@ -44,9 +47,9 @@ def test_partitions_that_only_exchange_messages_build_the_oracles_suffix_array(g
     h = C.c_void_p()
     assert lib.csa_create(n, 1, C.byref(h)) == 0
     try:
-        print(f"  multi-partition n={n} p={p} key_words={key_words}", flush=True)
+        print(f"  multi-partition n={n} p={p} key_words={key_words} steps={steps}", flush=True)
         sa, gens = multi_partition.build_sa(lib, to_dev, to_host, T, p, key_words=key_words, log=log,
-                                            join_handle=h if sorted_join else None)
+                                            join_handle=h if sorted_join else None, step_handle=h if steps else None)
     finally:
         lib.csa_destroy(h)
     want, _ = oracle_lib.prefix_doubling(T, key_words)
