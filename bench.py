@@ -228,6 +228,65 @@ def bench_next_rows(args):
         res = _row_result("messages joined/sec at 1 GPU", "messages for half of a suffix-ordered cohort", msg_c, ms_sorted,
                           "unpack + 5 radix passes + join_messages_kernel", msg_c * (9 + 8 + 4 + 8),
                           {"cohort": n, "ms_unsorted_inbox": round(ms, 3)}, args.steps, args.warmup, ok)
+    elif args.row in ("step_init", "step_rerank"):
+        # one partition step under the exchange scheme: everything the reference does between the upload of a partition's
+        # slabs and their download (src/GPU_SACA.cu:1112-1331 / 1715-1995). The synthetic partition: n suffixes of the
+        # workload's text in random order, p partitions by sampled pivots.
+        import ctypes as C
+
+        class StepResult(C.Structure):
+            _fields_ = [("active", C.c_uint64), ("messages", C.c_uint64)]
+        T = workloads.generate(args.config, n)
+        pivots = oracle_lib.sample_pivots(T[:1 << 22], p, 2, rng)
+        d_text = torch.from_numpy(T.view(np.int16)).to(dev)
+        _, packed, _ = partition_ids(d_text, torch.from_numpy(pivots.view(np.int64)).to(dev).reshape(-1, 2), p, want_ids=False)
+        suf = torch.randperm(n, device=dev)
+        lanes = torch.stack([(suf >> (8 * b)) & 0xFF for b in range(5)], dim=1).to(torch.uint8).reshape(-1).contiguous()
+        keys, beta = stage_slab(d_text, lanes, 1, packed, p, 4, True)
+        sorter = PartitionSorter(n)
+        rank_out = torch.empty(n, dtype=torch.int32, device=dev)
+        suf_out = torch.empty(5 * n, dtype=torch.uint8, device=dev)
+        mt, mr = torch.empty(5 * 2 * n, dtype=torch.uint8, device=dev), torch.empty(2 * n, dtype=torch.int32, device=dev)
+        off = torch.zeros(p + 1, dtype=torch.int32, device=dev)
+        res = StepResult()
+        st = torch.cuda.current_stream(dev).cuda_stream
+        init = lambda: _native.check(lib.csa_sort_init_dev(sorter._h, keys.data_ptr(), 1, lanes.data_ptr(), beta.data_ptr(), n, p,
+                                                            rank_out.data_ptr(), suf_out.data_ptr(), mt.data_ptr(), mr.data_ptr(),
+                                                            off.data_ptr(), st, C.byref(res)))
+        if args.row == "step_init":
+            ms, _ = _timed(torch, init, args.steps, args.warmup)
+            # the whole text as one partition: its step-0 ranks are those of the resident sort's generation 0, so as many
+            # suffixes survive as the partition sort reports active after generation 0
+            check = PartitionSorter(n)
+            check.sort(d_text)
+            resident = check.last_stats["active"][1] if check.last_stats["generations"] > 1 else 0
+            # with several partitions the forward tag (the partition of the suffix one context further) refines the order
+            ok = int(res.active) == resident if p == 1 else int(res.active) <= resident
+            check.close()
+            alg = n * (8 + 5 + 4 + 2 * 2 * 24 + 8 * 2 * 24 + 41 + 41 + 9)  # tag sort, key sort, rank, split, narrow
+            res_row = _row_result("suffixes through a generation-0 partition step/sec at 1 GPU", workloads.NAMES[args.config], n, ms,
+                                  "csa_sort_init_dev (10 radix passes + glue)", alg,
+                                  {"partitions": p, "active_after": int(res.active), "messages": int(res.messages)}, args.steps, args.warmup, ok)
+        else:
+            init()
+            a = int(res.active)
+            total = int(res.messages)
+            # the next generation of the survivors, fed with their own outbox as the inbox of a one-partition run would be
+            beta1 = torch.zeros(a, dtype=torch.int32, device=dev)
+            rk_in, sf_in = rank_out[:a].clone(), suf_out[:5 * a].clone()
+            in_t, in_r = mt[:5 * total].clone(), mr[:total].clone()
+            rer = lambda: _native.check(lib.csa_sort_rerank_dev(sorter._h, rk_in.data_ptr(), sf_in.data_ptr(), beta1.data_ptr(), a,
+                                                                 in_t.data_ptr(), in_r.data_ptr(), total, 8, p, rank_out.data_ptr(),
+                                                                 suf_out.data_ptr(), mt.data_ptr(), mr.data_ptr(), off.data_ptr(), st,
+                                                                 C.byref(res)))
+            ms, _ = _timed(torch, rer, args.steps, args.warmup)
+            ok = int(res.active) <= a
+            alg = a * (5 * 2 * 24 + 29 + 8 * 2 * 24 + 90 + 9)  # suffix-order sort, join, key sort, re-rank, narrow (rows a8-a11)
+            res_row = _row_result("active suffixes through a later partition step/sec at 1 GPU", workloads.NAMES[args.config], a, ms,
+                                  "csa_sort_rerank_dev (13 radix passes + join + glue)", alg,
+                                  {"partitions": p, "inbox": total, "active_after": int(res.active)}, args.steps, args.warmup, ok)
+        sorter.close()
+        res = res_row
     else:  # scatter
         rank = torch.randperm(n, device=dev).to(torch.int32)
         lanes = torch.randint(0, 256, (5 * n,), dtype=torch.uint8, device=dev)
@@ -256,7 +315,7 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=1 << 26, help="symbols of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--generations", action="store_true", help="print the per-generation table to stderr")
-    ap.add_argument("--row", default="sort", choices=["sort", "partition_ids", "stage_slab", "messages", "join", "scatter"],
+    ap.add_argument("--row", default="sort", choices=["sort", "partition_ids", "stage_slab", "messages", "join", "scatter", "step_init", "step_rerank"],
                     help="which step to measure: the partition sort (the headline, default) or one of the steps around it")
     ap.add_argument("--partitions", type=int, default=256, help="partitions of --row partition_ids")
     args = ap.parse_args()

@@ -96,6 +96,10 @@ constexpr u32 DEFER_MIN = CSA_DEFER_MIN;
 #endif
 constexpr int WINDOW_LOG2 = CSA_WINDOW_LOG2;
 constexpr u32 WINDOW_MIN_CHANGED = CSA_WINDOW_MIN_CHANGED;
+// smallest cohort for which the message join builds a directory over the suffix-ordered cohort first
+#ifndef CSA_JOIN_DIR_MIN
+#define CSA_JOIN_DIR_MIN 4096u
+#endif
 
 
 int bit_length(u64 v)
@@ -932,6 +936,30 @@ int csa_emit_messages_dev(const uint64_t* d_sa, const uint64_t* d_keys, const ui
     return CSA_OK;
 }
 
+extern "C++" {
+namespace {
+// Builds the join directory of the suffix-ordered cohort d_sa[0, n) in `dir` (room for `room` entries) and returns the
+// log2 of its bucket count through *dir_log2; leaves *dir_log2 = 0 and builds nothing when the cohort is small.
+int build_join_directory(const u64* d_sa, u64 n, u32* dir, u64 room, hipStream_t s, u32* dir_log2)
+{
+    *dir_log2 = 0;
+    if (n < CSA_JOIN_DIR_MIN || room < 3)
+        return CSA_OK;
+    u32 lg = (u32)bit_length(n) - 2u; // two to four cohort entries per bucket
+    if (lg > 22u)
+        lg = 22u;
+    while (lg && (1ull << lg) + 1 > room)
+        --lg;
+    if (lg == 0)
+        return CSA_OK;
+    hipLaunchKernelGGL(join_directory_kernel, dim3((u32)(((1ull << lg) + 256) / 256)), dim3(256), 0, s, d_sa, n, lg, dir);
+    HIP_TRY(hipGetLastError());
+    *dir_log2 = lg;
+    return CSA_OK;
+}
+} // namespace
+} // extern "C++"
+
 int csa_join_messages_dev(const uint8_t* d_msg_target, const uint32_t* d_msg_rank, uint32_t msg_c, const uint64_t* d_sa,
                           const uint32_t* d_primary, uint64_t* d_keys, uint64_t n, void* stream)
 {
@@ -942,7 +970,7 @@ int csa_join_messages_dev(const uint8_t* d_msg_target, const uint32_t* d_msg_ran
     if (n > CSA_MAX_PART_SZ)
         return fail(CSA_ERR_TOO_LARGE, "csa_join_messages_dev: %llu suffixes exceed a partition", (unsigned long long)n);
     hipLaunchKernelGGL(join_messages_kernel, dim3((msg_c + 255u) / 256u), dim3(256), 0, (hipStream_t)stream, d_msg_target,
-                       (const u64*)nullptr, d_msg_rank, msg_c, d_sa, d_primary, d_keys, n);
+                       (const u64*)nullptr, d_msg_rank, msg_c, d_sa, d_primary, d_keys, n, (const u32*)nullptr, 0u);
     HIP_TRY(hipGetLastError());
     return CSA_OK;
 }
@@ -976,8 +1004,13 @@ int csa_join_messages_sorted_dev(csa_handle* h, const uint8_t* d_msg_target, con
     int rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, h->key[0], h->idx[0], h->key[1], h->idx[1], msg_c, plan, &in_out, &passes);
     if (rc)
         return rc;
+    u32 dir_log2 = 0;
+    rc = build_join_directory(d_sa, n, h->idx[2], h->cap, s, &dir_log2);
+    if (rc)
+        return rc;
     hipLaunchKernelGGL(join_messages_kernel, dim3((msg_c + 255u) / 256u), dim3(256), 0, s, (const u8*)nullptr,
-                       (const u64*)h->key[in_out], (const u32*)h->idx[in_out], msg_c, d_sa, d_primary, d_keys, n);
+                       (const u64*)h->key[in_out], (const u32*)h->idx[in_out], msg_c, d_sa, d_primary, d_keys, n,
+                       (const u32*)(dir_log2 ? h->idx[2] : nullptr), dir_log2);
     HIP_TRY(hipGetLastError());
     return read_counts(L, nullptr);
 }
@@ -1218,9 +1251,17 @@ int csa_sort_rerank_dev(csa_handle* h, const uint32_t* d_rank, const uint8_t* d_
     //    (src/GPU_SACA.cu:1803-1835)
     u64* keys = h->key[2];
     hipLaunchKernelGGL(fill_u64_kernel, dim3(blocks), dim3(256), 0, s, keys, m, ~0ull);
-    if (inbox_sz)
+    if (inbox_sz) {
+        // the permutation of the suffix-order sort has been consumed: its other buffer holds the directory
+        u32* dir = P[in_out ^ 1];
+        u32 dir_log2 = 0;
+        rc = build_join_directory(words_by_suffix, m, dir, h->cap, s, &dir_log2);
+        if (rc)
+            return rc;
         hipLaunchKernelGGL(join_messages_kernel, dim3((inbox_sz + 255u) / 256u), dim3(256), 0, s, d_inbox_target, (const u64*)nullptr,
-                           d_inbox_rank, inbox_sz, (const u64*)words_by_suffix, (const u32*)primary_by_suffix, keys, m);
+                           d_inbox_rank, inbox_sz, (const u64*)words_by_suffix, (const u32*)primary_by_suffix, keys, m,
+                           (const u32*)(dir_log2 ? dir : nullptr), dir_log2);
+    }
     HIP_TRY(hipGetLastError());
     // 3. sort by (primary, secondary): key bits [0, 62) (src/GPU_SACA.cu:1841-1871)
     hipLaunchKernelGGL(iota_kernel, dim3(blocks), dim3(256), 0, s, P[0], m);

@@ -177,17 +177,46 @@ __global__ __launch_bounds__(1024) void message_offsets_kernel(u32* v, u32 count
     }
 }
 
+// A directory over the suffix-ordered cohort SA[0, n): dir[b] = first place whose suffix is >= b << shift, for b in
+// [0, 2^dir_log2], where shift spreads the directory over the values up to the cohort's largest suffix. A search for a
+// target then starts inside one bucket (a few neighbouring entries, one or two cache lines) instead of walking the whole
+// array, which would cost a cache line from HBM for every level below the cached top of the search tree.
+__device__ __forceinline__ u32 join_directory_shift(const u64* __restrict__ sa, u64 n, u32 dir_log2)
+{
+    const u64 largest = sa[n - 1] & MSG_VAL_MASK;
+    const u32 span = 64u - (u32)__builtin_clzll(largest | 1ull);
+    return span > dir_log2 ? span - dir_log2 : 0u;
+}
+
+__global__ __launch_bounds__(256) void join_directory_kernel(const u64* __restrict__ sa, u64 n, u32 dir_log2, u32* __restrict__ dir)
+{
+    const u64 b = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (b > (1ull << dir_log2))
+        return;
+    const u64 v = b << join_directory_shift(sa, n, dir_log2);
+    u64 low = 0, high = n;
+    while (low < high) {
+        const u64 mid = low + (high - low) / 2;
+        if ((sa[mid] & MSG_VAL_MASK) < v)
+            low = mid + 1;
+        else
+            high = mid;
+    }
+    dir[b] = (u32)low;
+}
+
 // Delivers every message to its recipient in the suffix-ordered cohort SA[0, n): K[pos] = primary[pos] << 31 |
 // received rank, marked if the message is a pill; a recipient that is not in the cohort has retired and the
 // message is dropped (include/GPU_SACA.cuh:362-389).
 // The targets come as 5-byte lanes (msg_target) or, when the inbox was sorted by target first, as 64-bit words
 // (target_words): sorted targets probe neighbouring places of the cohort, so that the probes of a wave share
-// cache lines instead of each costing a line from HBM.
+// cache lines instead of each costing a line from HBM. With a directory (dir != null, from join_directory_kernel) the
+// search is confined to the target's bucket.
 __global__ __launch_bounds__(256) void join_messages_kernel(const u8* __restrict__ msg_target,
                                                             const u64* __restrict__ target_words,
                                                             const u32* __restrict__ msg_rank, u32 msg_c,
                                                             const u64* __restrict__ sa, const u32* __restrict__ primary,
-                                                            u64* keys, u64 n)
+                                                            u64* keys, u64 n, const u32* __restrict__ dir, u32 dir_log2)
 {
     const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
     if (i >= msg_c)
@@ -201,6 +230,14 @@ __global__ __launch_bounds__(256) void join_messages_kernel(const u8* __restrict
             tgt |= (u64)msg_target[5 * i + b] << (8 * b);
     }
     u64 low = 0, high = n;
+    if (dir) {
+        const u64 b = tgt >> join_directory_shift(sa, n, dir_log2);
+        if (b >= (1ull << dir_log2))
+            return; // beyond the cohort's largest suffix
+        low = dir[b];
+        high = dir[b + 1];
+    }
+    const u64 end = high;
     while (low < high) {
         const u64 mid = low + (high - low) / 2;
         if ((sa[mid] & MSG_VAL_MASK) < tgt)
@@ -208,7 +245,8 @@ __global__ __launch_bounds__(256) void join_messages_kernel(const u8* __restrict
         else
             high = mid;
     }
-    if (low == n || (sa[low] & MSG_VAL_MASK) != tgt)
+    // a target that is absent from its bucket is absent from the cohort: the next bucket starts above it
+    if (low == end || (sa[low] & MSG_VAL_MASK) != tgt)
         return;
     const u32 r = msg_rank[i];
     u64 key = ((u64)primary[low] << 31) | (u64)(r & ~MSG_PILL_BIT);
