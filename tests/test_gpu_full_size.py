@@ -39,3 +39,30 @@ def test_full_size_configuration_sorts_to_a_verified_suffix_array(config):
         assert s.verify(d_text, out2)
     finally:
         s.close()
+
+
+@pytest.mark.timeout(300)
+def test_largest_partition_at_the_largest_index_base():
+    """n = 2^31 - 1 suffixes (MAX_PART_SZ, include/bit-layout.hpp:63-68) ending at suffix index 2^40 - 1, the last
+    one a 5-byte entry can hold (include/sa40.hpp:72-75): uniform random symbols, generated on the device."""
+    import torch
+    from cascade_amd import PartitionSorter
+    n = (1 << 31) - 1
+    base = (1 << 40) - n
+    print(f"  largest partition n={n} index_base={base}", flush=True)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(20240531)
+    d_text = torch.randint(-32768, 32768, (n,), dtype=torch.int16, device="cuda", generator=g)
+    s = PartitionSorter(n, key_words=1)
+    try:
+        out = s.sort(d_text, index_base=base)
+        assert s.last_stats["n"] == n and s.last_stats["generations"] >= 1
+        assert s.verify(d_text, out, index_base=base)
+        assert not s.verify(d_text, out, index_base=base - 1)
+        lanes = out.view(n, 5)
+        total = sum(int(lanes[:, k].sum(dtype=torch.int64)) << (8 * k) for k in range(5))
+        assert total == n * (n - 1) // 2 + n * base
+        # the largest entry is 2^40 - 1: all five bytes 0xFF somewhere in the output
+        assert bool((lanes == 255).all(dim=1).any())
+    finally:
+        s.close()
