@@ -228,6 +228,66 @@ def bench_next_rows(args):
         res = _row_result("messages joined/sec at 1 GPU", "messages for half of a suffix-ordered cohort", msg_c, ms_sorted,
                           "unpack + 5 radix passes + join_messages_kernel", msg_c * (9 + 8 + 4 + 8),
                           {"cohort": n, "ms_unsorted_inbox": round(ms, 3)}, args.steps, args.warmup, ok)
+    elif args.row == "overlap":
+        # Host buffers in and out, as the reference's pipeline hands partitions over: three dispatcher threads, each with its
+        # own handle, stream and device buffers (STREAM_C = 3, include/GPU_SACA.hpp:90-91; the dispatcher loop of
+        # src/GPU_SACA.cu:1539-1589), take independent texts from pinned host memory, sort them and bring the suffix arrays
+        # back into pinned host memory. One thread's upload and download overlap the other threads' sorts.
+        import threading
+        parts = min(p, 12)
+        n = args.n if args.n is not None else 1 << 26
+        T = workloads.generate(args.config, parts * n)
+        h_text = torch.from_numpy(T.view(np.int16)).reshape(parts, n).pin_memory()
+        h_out = torch.empty((parts, 5 * n), dtype=torch.uint8).pin_memory()
+
+        def run(dispatchers):
+            errors, in_hbm_ms = [], [0.0] * dispatchers
+
+            def dispatcher(t):
+                try:
+                    stream = torch.cuda.Stream(device=dev)
+                    sorter = PartitionSorter(n)
+                    d_text = torch.empty(n, dtype=torch.int16, device=dev)
+                    d_out = torch.empty(5 * n + 128, dtype=torch.uint8, device=dev)
+                    with torch.cuda.stream(stream):
+                        for q in range(t, parts, dispatchers):
+                            d_text.copy_(h_text[q], non_blocking=True)
+                            st = sorter.sort_ptr(d_text.data_ptr(), n, d_out.data_ptr(), 0, stream.cuda_stream)
+                            in_hbm_ms[t] += st["ms_total"]
+                            h_out[q].copy_(d_out[:5 * n], non_blocking=True)
+                        stream.synchronize()
+                    sorter.close()
+                except Exception as e:  # reported by the main thread
+                    errors.append(e)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            threads = [threading.Thread(target=dispatcher, args=(t,)) for t in range(dispatchers)]
+            for th in threads:
+                th.start()
+            for th in threads:
+                th.join()
+            torch.cuda.synchronize()
+            if errors:
+                raise errors[0]
+            return (time.perf_counter() - t0) * 1e3, sum(in_hbm_ms)
+        for _ in range(args.warmup):
+            run(3)
+        ms3 = min(run(3)[0] for _ in range(args.steps))
+        ms1, in_hbm = run(1)
+        sorter = PartitionSorter(n)
+        ok = True
+        for q in (0, parts // 2, parts - 1):
+            ok = ok and sorter.verify(h_text[q].to(dev), h_out[q].to(dev))
+        sorter.close()
+        pcie_bytes = parts * n * 7
+        res = _row_result("suffixes sorted/sec at 1 GPU, host buffers in and out", workloads.NAMES[args.config], parts * n, ms3,
+                          "whole job: upload, partition sorts, download on three streams", pcie_bytes,
+                          {"texts": parts, "n_each": n, "dispatchers": 3, "ms_one_dispatcher": round(ms1, 2),
+                           "ms_in_hbm_sorts_only": round(in_hbm, 2), "pcie_GBps_both_ways": round(pcie_bytes / ms3 / 1e6, 1)},
+                          args.steps, args.warmup, ok)
+        res["roofline"]["bound"] = "pcie (not an HBM figure: 2 B up + 5 B down per suffix over the host link)"
+        res["roofline"]["peak"] = None
+        res["roofline"]["frac"] = None
     elif args.row in ("step_init", "step_rerank"):
         # one partition step under the exchange scheme: everything the reference does between the upload of a partition's
         # slabs and their download (src/GPU_SACA.cu:1112-1331 / 1715-1995). The synthetic partition: n suffixes of the
@@ -315,8 +375,10 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=1 << 26, help="symbols of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--generations", action="store_true", help="print the per-generation table to stderr")
-    ap.add_argument("--row", default="sort", choices=["sort", "partition_ids", "stage_slab", "messages", "join", "scatter", "step_init", "step_rerank"],
+    ap.add_argument("--row", default="sort", choices=["sort", "partition_ids", "stage_slab", "messages", "join", "scatter", "step_init", "step_rerank", "overlap"],
                     help="which step to measure: the partition sort (the headline, default) or one of the steps around it")
+    ap.add_argument("--shared-device", action="store_true",
+                    help="measure the headline with the default tile order (safe next to other launches) only")
     ap.add_argument("--partitions", type=int, default=256, help="partitions of --row partition_ids")
     args = ap.parse_args()
 
@@ -343,7 +405,9 @@ def main():
     d_text = torch.from_numpy(T.view(np.int16)).to(dev)
     del T
     out = torch.empty(5 * n + 128, dtype=torch.uint8, device=dev)
-    sorter = PartitionSorter(n, key_words=args.key_words)
+    # bench.py is the only user of the GPU while it runs, which is what csa_set_device_exclusive asks the caller to
+    # declare; the time of the default tile order (safe next to other launches) is measured beside it
+    sorter = PartitionSorter(n, key_words=args.key_words, device_exclusive=not args.shared_device)
     print(f"[bench] C{args.config} n={n} generated in {t_gen:.1f}s; scratch {sorter.bytes_per_suffix() * n / 2**30:.1f} GiB",
           file=sys.stderr, flush=True)
 
@@ -373,12 +437,26 @@ def main():
     elapsed = time.perf_counter() - t0
     ms_per_step = 1e3 * elapsed / args.steps
     st = sorter.last_stats
-
     verified = None
     if not args.no_verify:
         verified = sorter.verify(d_text, out)
         if not verified:
             print("[bench] the device verifier REJECTED the suffix array", file=sys.stderr)
+
+    ms_by_arrival = ms_per_step
+    if not args.shared_device:
+        sorter.set_device_exclusive(False)
+        sorter.sort(d_text, out=out)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            sorter.sort(d_text, out=out)
+        torch.cuda.synchronize()
+        ms_by_arrival = 1e3 * (time.perf_counter() - t0) / args.steps
+        sorter.set_device_exclusive(True)
+        if verified and not sorter.verify(d_text, out):
+            verified = False
+            print("[bench] the device verifier REJECTED the suffix array of the default tile order", file=sys.stderr)
 
     per_gen, a_out = algorithmic_bytes(n, st["active"])
     a_total = sum(per_gen) + a_out
@@ -417,7 +495,9 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u64 keys / u32 ranks", "data": "synthetic",
         "config": {"workload": workloads.NAMES[args.config], "n": n, "key_words": args.key_words,
-                   "generations": st["generations"], "bit_exact_verified": verified},
+                   "generations": st["generations"], "bit_exact_verified": verified,
+                   "tile_order": "by arrival" if args.shared_device else "XCD-chunked (device declared exclusive)",
+                   "ms_per_step_tiles_by_arrival": round(ms_by_arrival, 3)},
         "roofline": roofline,
         "job_hbm_frac": round(a_total / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         "job_algorithmic_bytes_per_suffix": round(a_total / n, 1),

@@ -21,6 +21,7 @@ EXPORTS = (
     "csa_partition_id_bits", "csa_partition_ids_u16_dev", "csa_scatter_to_rank_order_dev", "csa_output_cut",
     "csa_stage_slab_u16_dev", "csa_count_messages_dev", "csa_message_offsets_dev", "csa_emit_messages_dev",
     "csa_join_messages_dev", "csa_join_messages_sorted_dev", "csa_sort_init_dev", "csa_sort_rerank_dev",
+    "csa_set_device_exclusive",
 )
 
 
@@ -71,6 +72,8 @@ def load():
     lib.csa_create.argtypes = [u64, i32, C.POINTER(vp)]
     lib.csa_destroy.restype = None
     lib.csa_destroy.argtypes = [vp]
+    lib.csa_set_device_exclusive.restype = C.c_int
+    lib.csa_set_device_exclusive.argtypes = [vp, C.c_int]
     lib.csa_sort_partition_u16_dev.restype = i32
     lib.csa_sort_partition_u16_dev.argtypes = [vp, vp, u64, u64, vp, vp, u32, C.POINTER(CsaStats)]
     lib.csa_sort_partition_u16.restype = i32

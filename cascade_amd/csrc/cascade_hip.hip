@@ -137,7 +137,8 @@ struct csa_handle {
     u32* counts = nullptr; // [2] error flag; [3] verifier flag; [4] members of large groups
     u32* h_pinned = nullptr; // host mirror: [0..3] counts/err, [16 ..) histogram
     u32 epoch = 0;
-    u32 xcd_chunk = 0;         // tiles of a radix pass that one XCD takes in a row (0: numbered by arrival)
+    u32 xcd_chunk = 0;         // tiles of a radix pass that one XCD takes in a row (0: numbered by arrival); in use
+    u32 xcd_chunk_exclusive = 0; // the value for a caller that has the device to itself (csa_set_device_exclusive)
     u32 defer_min = DEFER_MIN; // lists at least this long use the bucketed rank update (env CASCADE_DEFER_MIN overrides)
     u64* step64[2] = {nullptr, nullptr}; // two more 8-byte arrays of the capacity, for the per-generation partition steps
     u32 window_min_changed = WINDOW_MIN_CHANGED; // env CASCADE_WINDOW_MIN_CHANGED overrides (0xFFFFFFFF: never)
@@ -1368,9 +1369,12 @@ int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
     int cus = 0;
     if (e == hipSuccess)
         e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, h->device);
-    h->xcd_chunk = cus >= 2 * 8 * (int)XCD_CHUNK ? XCD_CHUNK : 0;
+    // XCD-chunked tile order needs 8 * XCD_CHUNK workgroups of a pass resident at once: offered only on a device with room
+    // for twice that many, and used only after csa_set_device_exclusive (the default numbers tiles by arrival)
+    h->xcd_chunk_exclusive = cus >= 2 * 8 * (int)XCD_CHUNK ? XCD_CHUNK : 0;
     if (const char* c = getenv("CASCADE_XCD_CHUNK"))
-        h->xcd_chunk = (u32)strtoul(c, nullptr, 10);
+        h->xcd_chunk_exclusive = (u32)strtoul(c, nullptr, 10);
+    h->xcd_chunk = 0;
     auto alloc = [&](void** p, u64 bytes) {
         if (e == hipSuccess)
             e = hipMalloc(p, bytes ? bytes : 4);
@@ -1409,6 +1413,14 @@ int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
         return rc;
     }
     *out = h;
+    return CSA_OK;
+}
+
+int csa_set_device_exclusive(csa_handle* h, int exclusive)
+{
+    if (!h)
+        return fail(CSA_ERR_ARG, "csa_set_device_exclusive: null handle");
+    h->xcd_chunk = exclusive ? h->xcd_chunk_exclusive : 0u;
     return CSA_OK;
 }
 

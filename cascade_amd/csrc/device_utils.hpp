@@ -57,13 +57,38 @@ __device__ __forceinline__ u32 wave_incl_max(u32 v)
 // between launches. Words are read and written with relaxed agent-scope atomics only: status and
 // value travel in the same word, so no fence is needed and the accesses are coherent across XCDs.
 // Tiles are numbered by an atomic ticket taken when a workgroup starts, hence every predecessor
-// of a waiting tile is already resident or finished. (The radix pass may instead derive the tile from
-// the workgroup index; its predecessors are then at most a bounded number of dispatches behind.)
-// Every wait has a spin limit that turns a predecessor that never shows up into an error word.
+// of a waiting tile is already resident or finished and the waits end whatever else shares the device.
+// (The radix pass may instead derive the tile from the workgroup index, for callers that have the device to
+// themselves: a predecessor may then belong to a workgroup that is dispatched later, which only ends if enough
+// workgroups of the launch are resident together.)
+// Every wait has a spin limit that turns a predecessor that never shows up into an error word, and gives up
+// early once another wait has failed; kernels that take the error word leave at once when it is set.
 
 constexpr u32 LB_AGG = 1;  // value = this tile's aggregate
 constexpr u32 LB_INCL = 2; // value = aggregate of tiles [0, tile]
-constexpr u32 LB_SPIN_LIMIT = 1u << 24;
+#ifndef CSA_LB_SPIN_LIMIT
+#define CSA_LB_SPIN_LIMIT (1u << 21) // polls of one word; a poll takes a microsecond or more
+#endif
+constexpr u32 LB_SPIN_LIMIT = CSA_LB_SPIN_LIMIT;
+
+// After a device invariant has failed, the arrays downstream of the failure hold neither a valid order nor valid
+// indices: every kernel that takes the error word leaves at once, and the host reports the code when it reads the
+// word back at the end of the step.
+__device__ __forceinline__ bool dev_failed(const u32* err)
+{
+    return err != nullptr && __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+}
+
+// The same answer in every thread of the workgroup (one thread reads), so that a workgroup leaves as a whole.
+// Must be called by all threads of the workgroup.
+__device__ __forceinline__ bool block_dev_failed(const u32* err)
+{
+    __shared__ u32 s_failed;
+    if (threadIdx.x == 0)
+        s_failed = dev_failed(err) ? 1u : 0u;
+    __syncthreads();
+    return s_failed != 0u;
+}
 
 __device__ __forceinline__ u64 lb_pack(u32 epoch, u32 status, u32 value)
 {
@@ -112,6 +137,8 @@ __device__ __forceinline__ u64 lb_wait_word(const u64* p, u32 epoch, u32* err)
             atomicExch(err, DEV_ERR_LOOKBACK_TIMEOUT);
             return 0;
         }
+        if ((idle & 1023u) == 0u && dev_failed(err))
+            return 0; // another wait has failed: the launch is lost, leave without waiting out the limit
         __builtin_amdgcn_s_sleep(2);
     }
 }
@@ -240,6 +267,8 @@ __device__ __forceinline__ u32 lb_wave_exclusive(u64* chain, u32 stride, u32 til
                     atomicExch(err, DEV_ERR_LOOKBACK_TIMEOUT);
                 return excl;
             }
+            if ((idle & 1023u) == 0u && __ballot(dev_failed(err)) != 0ull)
+                return excl; // another wait has failed: the launch is lost
             __builtin_amdgcn_s_sleep(1);
         } else {
             idle = 0;

@@ -223,12 +223,16 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
     // each XCD has an L2 of its own. With xcd_chunk = C, every XCD works on chunks of C consecutive tiles, so the
     // runs of one digit written by neighbouring tiles meet in the same L2 and leave it as full lines; measured
     // 15% faster per pass than arrival order at C = 16. The predecessor of a tile may then belong to a workgroup
-    // dispatched up to 8 (C - 1) places later, so C is only used where that many workgroups are resident at
-    // once (the host decides). Tiles past the last whole group of 8 chunks, and every tile when C = 0, are
-    // numbered so that all predecessors have started.
+    // dispatched up to 8 (C - 1) places later: the waits only end if that many workgroups of this launch are
+    // resident at once, which holds on a device that runs nothing else and not, in general, next to other launches
+    // (their waiting workgroups can fill the places this launch needs). The host therefore passes C > 0 only for a
+    // caller that has declared the device its own. Tiles past the last whole group of 8 chunks, and every tile when
+    // C = 0, are numbered by arrival, so that all predecessors have started.
     if (t == 0) {
         u32 tl;
-        if (a.xcd_chunk == 0) {
+        if (dev_failed(a.err)) {
+            tl = 0xFFFFFFFFu; // the step is lost already: leave, and take no ticket
+        } else if (a.xcd_chunk == 0) {
             tl = atomicAdd(a.ticket, 1u);
         } else {
             const u32 b = blockIdx.x;
@@ -246,6 +250,8 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
         s_whist[i] = 0;
     __syncthreads();
     const u32 tile = s_tile;
+    if (tile == 0xFFFFFFFFu)
+        return;
     const u64 base = (u64)tile * TILE;
     const u32 valid = (u32)((u64)a.n - base < (u64)TILE ? (u64)a.n - base : (u64)TILE);
     const u32 sh = (u32)a.shift & 31u;

@@ -38,13 +38,20 @@ def stats_to_dict(st):
 class PartitionSorter:
     """Owns the device scratch for partitions of up to `max_part_sz` suffixes (csa_create / csa_destroy)."""
 
-    def __init__(self, max_part_sz, key_words=1):
+    def __init__(self, max_part_sz, key_words=1, device_exclusive=False):
         self._lib = _native.load()
         self._h = C.c_void_p()
         _native.check(self._lib.csa_create(int(max_part_sz), int(key_words), C.byref(self._h)))
         self.max_part_sz = int(max_part_sz)
         self.key_words = int(key_words)
         self.last_stats = None
+        if device_exclusive:
+            self.set_device_exclusive(True)
+
+    def set_device_exclusive(self, exclusive):
+        """Declares that nothing else runs on the device during this handle's calls (csa_set_device_exclusive): the
+        radix passes may then use the XCD-chunked tile order, which is not safe next to other launches."""
+        _native.check(self._lib.csa_set_device_exclusive(self._h, 1 if exclusive else 0))
 
     def close(self):
         if self._h:

@@ -243,3 +243,29 @@ def test_multi_partition_pipeline_with_the_emulated_step_entries(emu, p, key_wor
     # the same run with numpy glue between the stages: the same cohorts, survivors and message counts at every step
     multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, p, key_words=key_words, log=glue_log)
     assert log == glue_log
+
+
+def test_chunked_tile_order_without_resident_workgroups_ends_in_an_error_not_a_hang(emu, monkeypatch):
+    # The XCD-chunked tile order of the radix pass waits for tiles whose workgroups are dispatched later. The emulator
+    # runs one workgroup at a time, the extreme case of a device shared with other launches: the wait must run into
+    # its spin limit, every later workgroup and kernel of the step must leave at once, and the call must report
+    # CSA_ERR_INTERNAL. By default (no csa_set_device_exclusive) tiles are numbered by arrival and the same text sorts.
+    emu.csa_set_device_exclusive.argtypes = [C.c_void_p, C.c_int]
+    monkeypatch.setenv("CASCADE_XCD_CHUNK", "16")
+    T = texts.random_text(140000, 5, 3, sep_every=0)  # 137 tiles of 1024 keys: one whole group of 8 chunks of 16
+    n = T.size
+    h = C.c_void_p()
+    assert emu.csa_create(n, 1, C.byref(h)) == 0
+    out = np.zeros(5 * n + 8, dtype=np.uint8)
+    st = _native.CsaStats()
+    try:
+        assert emu.csa_set_device_exclusive(h, 1) == 0
+        rc = emu.csa_sort_partition_u16_dev(h, T.ctypes.data, n, 0, out.ctypes.data, None, 0, C.byref(st))
+        assert rc == -4 and b"spin limit" in emu.csa_last_error(), (rc, emu.csa_last_error())
+        assert emu.csa_set_device_exclusive(h, 0) == 0
+        small = T[:6000].copy()
+        rc = emu.csa_sort_partition_u16_dev(h, small.ctypes.data, small.size, 0, out.ctypes.data, None, 0, C.byref(st))
+        assert rc == 0, emu.csa_last_error()
+        assert np.array_equal(out[:5 * small.size], oracle_lib.build_sa40(small))
+    finally:
+        emu.csa_destroy(h)

@@ -9,8 +9,8 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.timeout(300)
-@pytest.mark.parametrize("config", [2, 3, 5, 4])
-def test_full_size_configuration_sorts_to_a_verified_suffix_array(config):
+@pytest.mark.parametrize("config,exclusive", [(2, False), (3, False), (3, True), (5, True), (4, False)])
+def test_full_size_configuration_sorts_to_a_verified_suffix_array(config, exclusive):
     import torch
     from cascade_amd import PartitionSorter, workloads
     n = workloads.default_n(config)
@@ -18,7 +18,8 @@ def test_full_size_configuration_sorts_to_a_verified_suffix_array(config):
     T = workloads.generate(config, n)
     d_text = torch.from_numpy(T.view(np.int16)).cuda()
     del T
-    s = PartitionSorter(n, key_words=1)
+    # exclusive: the XCD-chunked tile order of the radix passes (the test is the only user of the device)
+    s = PartitionSorter(n, key_words=1, device_exclusive=exclusive)
     try:
         out = s.sort(d_text)
         stats = s.last_stats
