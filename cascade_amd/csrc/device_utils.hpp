@@ -62,7 +62,7 @@ __device__ __forceinline__ u32 wave_incl_max(u32 v)
 // themselves: a predecessor may then belong to a workgroup that is dispatched later, which only ends if enough
 // workgroups of the launch are resident together.)
 // Every wait has a spin limit that turns a predecessor that never shows up into an error word, and gives up
-// early once another wait has failed; kernels that take the error word leave at once when it is set.
+// early once another wait has failed; the kernels that wait leave at once when the word is set.
 
 constexpr u32 LB_AGG = 1;  // value = this tile's aggregate
 constexpr u32 LB_INCL = 2; // value = aggregate of tiles [0, tile]
@@ -72,22 +72,12 @@ constexpr u32 LB_INCL = 2; // value = aggregate of tiles [0, tile]
 constexpr u32 LB_SPIN_LIMIT = CSA_LB_SPIN_LIMIT;
 
 // After a device invariant has failed, the arrays downstream of the failure hold neither a valid order nor valid
-// indices: every kernel that takes the error word leaves at once, and the host reports the code when it reads the
-// word back at the end of the step.
+// indices: the kernels that wait for other workgroups leave at once, and the host reports the code when it reads the
+// word back at the end of the step. (Kernels without a wait check the indices they are given instead, and raise the
+// word themselves: reading it first would put a memory round trip in front of every workgroup.)
 __device__ __forceinline__ bool dev_failed(const u32* err)
 {
     return err != nullptr && __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
-}
-
-// The same answer in every thread of the workgroup (one thread reads), so that a workgroup leaves as a whole.
-// Must be called by all threads of the workgroup.
-__device__ __forceinline__ bool block_dev_failed(const u32* err)
-{
-    __shared__ u32 s_failed;
-    if (threadIdx.x == 0)
-        s_failed = dev_failed(err) ? 1u : 0u;
-    __syncthreads();
-    return s_failed != 0u;
 }
 
 __device__ __forceinline__ u64 lb_pack(u32 epoch, u32 status, u32 value)

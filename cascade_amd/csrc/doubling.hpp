@@ -73,8 +73,6 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
     const u64 tile_base = (u64)tile * TILE;
     const u64 base = tile_base + (u64)t * ITEMS;
     const u32 m = a.m;
-    if (block_dev_failed(a.err))
-        return; // the sorted list this step reads is not valid
 
     // striped load into LDS: slot q holds element tile_base + q - 1
 #pragma unroll
@@ -432,8 +430,6 @@ __global__ __launch_bounds__(BLOCK) void smallsort_kernel(SmallSortArgs a)
     const u32 t = threadIdx.x;
     const long long t0 = (long long)blockIdx.x * TILE;
     const long long lo = t0 - MAXG; // list index of s_sec[0]
-    if (block_dev_failed(a.err))
-        return; // the active list is not valid
 
     u32 x[ITEMS], sec[ITEMS];
     // own elements (striped: consecutive lanes hold consecutive elements) and the two halos
@@ -693,8 +689,6 @@ __global__ __launch_bounds__(BLOCK) void apply_small_kernel(ApplySmallArgs a)
     const u32 tile = blockIdx.x;
     const u64 tile_base = (u64)tile * TILE;
     const u32 m = a.m;
-    if (block_dev_failed(a.err))
-        return; // the sorted list is not valid
     // striped loads; s_nr[q] holds place tile_base + q - 1
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
@@ -816,8 +810,11 @@ __global__ __launch_bounds__(BLOCK) void place_big_kernel(PlaceArgs a)
     const u32 t = threadIdx.x;
     const u32 lane = t & 63u;
     const u32 w = t >> 6;
-    if (t == 0)
-        s_tile = dev_failed(a.err) ? 0xFFFFFFFFu : atomicAdd(a.ticket, 1u);
+    if (t == 0) {
+        const bool failed = dev_failed(a.err); // read while the ticket is on its way
+        const u32 ticket = atomicAdd(a.ticket, 1u);
+        s_tile = failed ? 0xFFFFFFFFu : ticket;
+    }
     __syncthreads();
     const u32 tile = s_tile;
     if (tile == 0xFFFFFFFFu)

@@ -229,10 +229,9 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
     // caller that has declared the device its own. Tiles past the last whole group of 8 chunks, and every tile when
     // C = 0, are numbered by arrival, so that all predecessors have started.
     if (t == 0) {
+        const bool failed = dev_failed(a.err); // read while the ticket is on its way
         u32 tl;
-        if (dev_failed(a.err)) {
-            tl = 0xFFFFFFFFu; // the step is lost already: leave, and take no ticket
-        } else if (a.xcd_chunk == 0) {
+        if (a.xcd_chunk == 0) {
             tl = atomicAdd(a.ticket, 1u);
         } else {
             const u32 b = blockIdx.x;
@@ -244,6 +243,8 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
                 tl = ((q / a.xcd_chunk) * 8u + x) * a.xcd_chunk + q % a.xcd_chunk;
             }
         }
+        if (failed)
+            tl = 0xFFFFFFFFu; // the step is lost already: leave
         s_tile = tl;
     }
     for (int i = t; i < WAVES * RADIX_BINS; i += BLOCK)
