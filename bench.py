@@ -379,6 +379,8 @@ def main():
                     help="which step to measure: the partition sort (the headline, default) or one of the steps around it")
     ap.add_argument("--shared-device", action="store_true",
                     help="measure the headline with the default tile order (safe next to other launches) only")
+    ap.add_argument("--no-order-comparison", action="store_true",
+                    help="do not also time the default tile order after the headline (counter runs want one sort per run)")
     ap.add_argument("--partitions", type=int, default=256, help="partitions of --row partition_ids")
     args = ap.parse_args()
 
@@ -444,7 +446,7 @@ def main():
             print("[bench] the device verifier REJECTED the suffix array", file=sys.stderr)
 
     ms_by_arrival = ms_per_step
-    if not args.shared_device:
+    if not args.shared_device and not args.no_order_comparison:
         sorter.set_device_exclusive(False)
         sorter.sort(d_text, out=out)
         torch.cuda.synchronize()
