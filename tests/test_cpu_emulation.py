@@ -245,6 +245,20 @@ def test_multi_partition_pipeline_with_the_emulated_step_entries(emu, p, key_wor
     assert log == glue_log
 
 
+def test_step_entries_on_a_text_of_one_symbol(emu):
+    """One symbol: a single group that only sheds its last members each generation; every pivot is equal, so all but
+    one partition are empty. Closed form: the shorter suffix comes first."""
+    import multi_partition
+    T = np.full(100, 9, dtype=np.uint16)
+    h = C.c_void_p()
+    assert emu.csa_create(T.size, 1, C.byref(h)) == 0
+    try:
+        sa, gens = multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, 3, step_handle=h)
+    finally:
+        emu.csa_destroy(h)
+    assert np.array_equal(sa, np.arange(T.size - 1, -1, -1, dtype=np.uint64)), gens
+
+
 def test_chunked_tile_order_without_resident_workgroups_ends_in_an_error_not_a_hang(emu, monkeypatch):
     # The XCD-chunked tile order of the radix pass waits for tiles whose workgroups are dispatched later. The emulator
     # runs one workgroup at a time, the extreme case of a device shared with other launches: the wait must run into

@@ -55,3 +55,36 @@ def test_partitions_that_only_exchange_messages_build_the_oracles_suffix_array(g
     want, _ = oracle_lib.prefix_doubling(T, key_words)
     assert np.array_equal(sa, want)
     assert gens >= 10 and sum(step[5] for step in log if step[0] >= 1) > 0
+
+
+def _shape(name):
+    from cascade_amd import workloads
+    if name == "one_symbol":       # one group until the very end; every pivot equal, so all but one partition are empty
+        return np.full(50000, 7, dtype=np.uint16)
+    if name == "period_7":         # groups of n / 7 members for log2(n) generations
+        return np.tile(np.array([3, 1, 4, 1, 5, 9, 2], dtype=np.uint16), 9000)
+    if name == "zipf_duplicates":  # the headline construction, scaled down: long duplicated documents
+        return workloads.generate(3, 400000)
+    if name == "adversarial":      # a token run, a periodic stretch and Zipf text in one partition set
+        return workloads.generate(5, 300000)
+    raise KeyError(name)
+
+
+@pytest.mark.parametrize("shape,p", [("one_symbol", 5), ("period_7", 9), ("zipf_duplicates", 300), ("adversarial", 64)])
+def test_step_entries_on_hard_shapes(gpu, shape, p):
+    """csa_sort_init_dev / csa_sort_rerank_dev per partition and generation, on texts whose groups stay large for many
+    generations, with empty partitions and with hundreds of partitions."""
+    lib, to_dev, to_host = gpu
+    T = _shape(shape)
+    n = T.size
+    h = C.c_void_p()
+    assert lib.csa_create(n, 1, C.byref(h)) == 0
+    try:
+        print(f"  step entries on {shape}: n={n} p={p}", flush=True)
+        sa, gens = multi_partition.build_sa(lib, to_dev, to_host, T, p, step_handle=h)
+    finally:
+        lib.csa_destroy(h)
+    want, _ = oracle_lib.prefix_doubling(T, 1)
+    assert np.array_equal(sa, want), (shape, gens)
+    if shape == "one_symbol":
+        assert np.array_equal(sa, np.arange(n - 1, -1, -1, dtype=np.uint64))
