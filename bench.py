@@ -323,7 +323,7 @@ def bench_next_rows(args):
             # with several partitions the forward tag (the partition of the suffix one context further) refines the order
             ok = int(res.active) == resident if p == 1 else int(res.active) <= resident
             check.close()
-            alg = n * (8 + 5 + 4 + 2 * 2 * 24 + 8 * 2 * 24 + 41 + 41 + 9)  # tag sort, key sort, rank, split, narrow
+            alg = n * (8 + 5 + 4 + 2 * 2 * 24 + 8 * 2 * 24 + 41 + 41 + 9)  # unpack, two tag passes, eight key passes, rank, split, narrow (src/GPU_SACA.cu:1157-1331)
             res_row = _row_result("suffixes through a generation-0 partition step/sec at 1 GPU", workloads.NAMES[args.config], n, ms,
                                   "csa_sort_init_dev (10 radix passes + glue)", alg,
                                   {"partitions": p, "active_after": int(res.active), "messages": int(res.messages)}, args.steps, args.warmup, ok)
@@ -341,7 +341,7 @@ def bench_next_rows(args):
                                                                  C.byref(res)))
             ms, _ = _timed(torch, rer, args.steps, args.warmup)
             ok = int(res.active) <= a
-            alg = a * (5 * 2 * 24 + 29 + 8 * 2 * 24 + 90 + 9)  # suffix-order sort, join, key sort, re-rank, narrow (rows a8-a11)
+            alg = a * (5 * 2 * 24 + 29 + 8 * 2 * 24 + 90 + 9)  # suffix-order sort, join, key sort, re-rank, narrow (src/GPU_SACA.cu:1769-1995)
             res_row = _row_result("active suffixes through a later partition step/sec at 1 GPU", workloads.NAMES[args.config], a, ms,
                                   "csa_sort_rerank_dev (13 radix passes + join + glue)", alg,
                                   {"partitions": p, "inbox": total, "active_after": int(res.active)}, args.steps, args.warmup, ok)

@@ -10,6 +10,11 @@
  * Pointers named d_* are device (HBM) addresses, h_* are host addresses. `stream` is a
  * hipStream_t passed as void* (NULL = the default stream). A handle owns all device scratch
  * memory and serves one call at a time; use one handle per stream for concurrent partitions.
+ *
+ * Entry points that take a handle, and csa_pack_keys_u16_dev, return after the stream has finished
+ * (they read counters back). csa_partition_ids_u16_dev, csa_stage_slab_u16_dev, csa_count_messages_dev,
+ * csa_message_offsets_dev, csa_emit_messages_dev and csa_join_messages_dev only enqueue kernels on the
+ * stream and allocate nothing.
  */
 #ifndef CASCADE_HIP_H
 #define CASCADE_HIP_H
