@@ -137,8 +137,9 @@ struct csa_handle {
     u32* counts = nullptr; // [2] error flag; [3] verifier flag; [4] members of large groups
     u32* h_pinned = nullptr; // host mirror: [0..3] counts/err, [16 ..) histogram
     u32 epoch = 0;
-    u32 xcd_chunk = 0;         // tiles of a radix pass that one XCD takes in a row (0: numbered by arrival); in use
-    u32 xcd_chunk_exclusive = 0; // the value for a caller that has the device to itself (csa_set_device_exclusive)
+    u32 tile_order = TILES_BY_ARRIVAL;           // how the radix passes number their tiles (radix_sort.hpp), in use
+    u32 tile_order_exclusive = TILES_BY_ARRIVAL; // the order after csa_set_device_exclusive
+    u32 xcd_chunk = XCD_CHUNK;                   // tiles of a radix pass that one XCD takes in a row under TILES_STATIC_CHUNKS
     u32 defer_min = DEFER_MIN; // lists at least this long use the bucketed rank update (env CASCADE_DEFER_MIN overrides)
     u64* step64[2] = {nullptr, nullptr}; // two more 8-byte arrays of the capacity, for the per-generation partition steps
     u32 window_min_changed = WINDOW_MIN_CHANGED; // env CASCADE_WINDOW_MIN_CHANGED overrides (0xFFFFFFFF: never)
@@ -187,21 +188,28 @@ u32 hist_blocks(u64 items_per_block, u64 n)
     return (u32)(blocks ? blocks : 1);
 }
 
-template <int SRC>
-void launch_onesweep(const OnesweepArgs& a, hipStream_t s)
+// tile order of a pass over a.n pairs in tiles of `tile` pairs
+void set_tile_order(const csa_handle* h, OnesweepArgs& a, u32 tile)
 {
-    const u32 tiles = (u32)(((u64)a.n + SORT_TILE - 1) / SORT_TILE);
-    if (a.shift >= 32)
-        hipLaunchKernelGGL((onesweep_kernel<u64, SORT_BLOCK, SORT_ITEMS, SRC, 1>), dim3(tiles), dim3(SORT_BLOCK), 0, s, a);
-    else
-        hipLaunchKernelGGL((onesweep_kernel<u64, SORT_BLOCK, SORT_ITEMS, SRC, 0>), dim3(tiles), dim3(SORT_BLOCK), 0, s, a);
+    a.tiles = (u32)(((u64)a.n + tile - 1) / tile);
+    a.order = h->tile_order;
+    a.xcd_chunk = h->xcd_chunk ? h->xcd_chunk : 1u;
 }
 
-void launch_onesweep32(const OnesweepArgs& a, hipStream_t s)
+template <int SRC>
+void launch_onesweep(const csa_handle* h, OnesweepArgs& a, hipStream_t s)
 {
-    constexpr u32 TILE32 = SORT_BLOCK * SORT32_ITEMS;
-    const u32 tiles = (u32)(((u64)a.n + TILE32 - 1) / TILE32);
-    hipLaunchKernelGGL((onesweep_kernel<u32, SORT_BLOCK, SORT32_ITEMS, SRC_PAIRS, 0>), dim3(tiles), dim3(SORT_BLOCK), 0, s, a);
+    set_tile_order(h, a, SORT_TILE);
+    if (a.shift >= 32)
+        hipLaunchKernelGGL((onesweep_kernel<u64, SORT_BLOCK, SORT_ITEMS, SRC, 1>), dim3(a.tiles), dim3(SORT_BLOCK), 0, s, a);
+    else
+        hipLaunchKernelGGL((onesweep_kernel<u64, SORT_BLOCK, SORT_ITEMS, SRC, 0>), dim3(a.tiles), dim3(SORT_BLOCK), 0, s, a);
+}
+
+void launch_onesweep32(const csa_handle* h, OnesweepArgs& a, hipStream_t s)
+{
+    set_tile_order(h, a, SORT_BLOCK * SORT32_ITEMS);
+    hipLaunchKernelGGL((onesweep_kernel<u32, SORT_BLOCK, SORT32_ITEMS, SRC_PAIRS, 0>), dim3(a.tiles), dim3(SORT_BLOCK), 0, s, a);
 }
 
 // Sorts n pairs by the digits of `plan`. The first pass that runs takes its input as `src` says
@@ -279,7 +287,6 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
         a.lookback_groups = h->lookback + h->lookback_tile_words;
         a.epoch = next_epoch(h);
         a.err = h->counts + 2;
-        a.xcd_chunk = h->xcd_chunk;
         int rc = next_ticket(L, &a.ticket);
         if (rc)
             return rc;
@@ -288,11 +295,11 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
             HIP_TRY(hipEventRecord(h->events[L.events_used], s));
         const int use_src = first ? src : SRC_PAIRS;
         if (use_src == SRC_PAIRS)
-            launch_onesweep<SRC_PAIRS>(a, s);
+            launch_onesweep<SRC_PAIRS>(h, a, s);
         else if (use_src == SRC_TEXT)
-            launch_onesweep<SRC_TEXT>(a, s);
+            launch_onesweep<SRC_TEXT>(h, a, s);
         else
-            launch_onesweep<SRC_TEXT_IDX>(a, s);
+            launch_onesweep<SRC_TEXT_IDX>(h, a, s);
         if (timed) {
             HIP_TRY(hipEventRecord(h->events[L.events_used + 1], s));
             L.timed.push_back({L.events_used, (u64)n});
@@ -436,11 +443,10 @@ int deferred_rank_update(Launch& L, const u32* pos, const DeferBuffers& buf, u32
             a.lookback_groups = h->lookback + h->lookback_tile_words;
             a.epoch = next_epoch(h);
             a.err = h->counts + 2;
-            a.xcd_chunk = h->xcd_chunk;
-            int rc = next_ticket(L, &a.ticket);
+                int rc = next_ticket(L, &a.ticket);
             if (rc)
                 return rc;
-            launch_onesweep32(a, s);
+            launch_onesweep32(h, a, s);
             in_pos = out_pos[p];
             in_val = out_val[p];
         }
@@ -489,11 +495,10 @@ int windowed_rank_update(Launch& L, const u32* pos, const DeferBuffers& buf, u32
         a.lookback_groups = h->lookback + h->lookback_tile_words;
         a.epoch = next_epoch(h);
         a.err = h->counts + 2;
-        a.xcd_chunk = h->xcd_chunk;
         int rc = next_ticket(L, &a.ticket);
         if (rc)
             return rc;
-        launch_onesweep32(a, s);
+        launch_onesweep32(h, a, s);
         in_pos = buf.t1_pos;
         in_val = buf.t1_val;
     }
@@ -1364,17 +1369,22 @@ int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
     if (rank_tiles * 4 > h->lookback_words)
         h->lookback_words = rank_tiles * 4;
     hipError_t e = hipGetDevice(&h->device);
-    // The XCD-aware tile order of the radix pass needs 8 * (XCD_CHUNK - 1) + 1 workgroups resident at once; every
-    // CU holds at least one, so a full MI355X (256 CUs) qualifies and a small partition of it falls back.
     int cus = 0;
     if (e == hipSuccess)
         e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, h->device);
-    // XCD-chunked tile order needs 8 * XCD_CHUNK workgroups of a pass resident at once: offered only on a device with room
-    // for twice that many, and used only after csa_set_device_exclusive (the default numbers tiles by arrival)
-    h->xcd_chunk_exclusive = cus >= 2 * 8 * (int)XCD_CHUNK ? XCD_CHUNK : 0;
-    if (const char* c = getenv("CASCADE_XCD_CHUNK"))
-        h->xcd_chunk_exclusive = (u32)strtoul(c, nullptr, 10);
-    h->xcd_chunk = 0;
+    // Tile order of the radix passes: by arrival, unless the caller declares the device its own
+    // (csa_set_device_exclusive); the XCD-chunked order then needs 8 * XCD_CHUNK workgroups of a pass resident at once
+    // and is offered only on a device with room for twice that many. CASCADE_XCD_CHUNK overrides the chunk length
+    // (0: never chunked), for experiments and for the CPU emulation's test of the failure path.
+    h->tile_order = TILES_BY_ARRIVAL;
+    h->tile_order_exclusive = cus >= 2 * 8 * (int)XCD_CHUNK ? TILES_STATIC_CHUNKS : TILES_BY_ARRIVAL;
+    h->xcd_chunk = XCD_CHUNK;
+    if (const char* c = getenv("CASCADE_XCD_CHUNK")) {
+        const u32 v = (u32)strtoul(c, nullptr, 10);
+        h->tile_order_exclusive = v ? TILES_STATIC_CHUNKS : TILES_BY_ARRIVAL;
+        if (v)
+            h->xcd_chunk = v;
+    }
     auto alloc = [&](void** p, u64 bytes) {
         if (e == hipSuccess)
             e = hipMalloc(p, bytes ? bytes : 4);
@@ -1420,7 +1430,7 @@ int csa_set_device_exclusive(csa_handle* h, int exclusive)
 {
     if (!h)
         return fail(CSA_ERR_ARG, "csa_set_device_exclusive: null handle");
-    h->xcd_chunk = exclusive ? h->xcd_chunk_exclusive : 0u;
+    h->tile_order = exclusive ? h->tile_order_exclusive : TILES_BY_ARRIVAL;
     return CSA_OK;
 }
 

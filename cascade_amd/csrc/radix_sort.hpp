@@ -179,11 +179,48 @@ struct OnesweepArgs {
     const u32* digit_base; // [256] for this pass
     u64* lookback;         // [tiles][256]
     u64* lookback_groups;  // [ceil(tiles / LB_GROUP)][256]
-    u32* ticket;           // zero before the launch (used when xcd_chunk == 0)
-    u32 xcd_chunk;         // consecutive tiles given to one XCD, or 0: tiles numbered by arrival
+    u32* ticket;           // zero before the launch (TILES_BY_ARRIVAL)
+    u32 order;             // TILES_BY_ARRIVAL or TILES_STATIC_CHUNKS
+    u32 xcd_chunk;         // TILES_STATIC_CHUNKS: consecutive tiles given to one XCD
+    u32 tiles;             // tiles of the pass = workgroups of the launch
     u32 epoch;
     u32* err;
 };
+
+// How the workgroups of a radix pass come by their tiles (one each). Whatever the order, a tile waits for the tiles
+// before it.
+//  TILES_BY_ARRIVAL     numbered by an atomic ticket: every predecessor of a tile has started, so every wait ends
+//                       whatever else shares the device.
+//  TILES_STATIC_CHUNKS  numbered from the workgroup index so that XCD x (workgroup b runs on XCD b % 8) works on chunks
+//                       of xcd_chunk consecutive tiles: the runs of one digit written by neighbouring tiles then meet in
+//                       one L2 and leave it as full lines (measured 15% faster per pass at chunks of 16). A predecessor
+//                       may belong to a workgroup that is dispatched up to 8 (xcd_chunk - 1) places later: the waits only
+//                       end if that many workgroups of the launch are resident at once, which holds on a device that
+//                       runs nothing else and not, in general, next to other launches (their waiting workgroups can
+//                       fill the places this launch needs). The host selects it only for a caller that has declared the
+//                       device its own. Tiles past the last whole group of 8 chunks are numbered by workgroup index.
+constexpr u32 TILES_BY_ARRIVAL = 0, TILES_STATIC_CHUNKS = 1;
+constexpr u32 NO_TILE = 0xFFFFFFFFu;
+
+// Thread 0 of a workgroup: its tile, or NO_TILE when the step is lost already and the workgroup is to leave.
+__device__ __forceinline__ u32 onesweep_tile_number(const OnesweepArgs& a)
+{
+    const bool failed = dev_failed(a.err); // read while the ticket is on its way
+    u32 tl;
+    if (a.order == TILES_BY_ARRIVAL) {
+        tl = atomicAdd(a.ticket, 1u);
+    } else {
+        const u32 b = blockIdx.x;
+        const u32 span = 8u * a.xcd_chunk;
+        const u32 whole = (a.tiles / span) * span;
+        tl = b;
+        if (b < whole) {
+            const u32 x = b % 8u, q = b / 8u;
+            tl = ((q / a.xcd_chunk) * 8u + x) * a.xcd_chunk + q % a.xcd_chunk;
+        }
+    }
+    return failed || tl >= a.tiles ? NO_TILE : tl;
+}
 
 // predecessors a digit's look-back inspects per round
 #ifndef CSA_SORT_LB_W
@@ -219,39 +256,13 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
     const u32 lane = t & 63u;
     const u32 w = t >> 6;
 
-    // Tile numbering. The hardware deals workgroups to the 8 XCDs round-robin (workgroup b runs on XCD b % 8), and
-    // each XCD has an L2 of its own. With xcd_chunk = C, every XCD works on chunks of C consecutive tiles, so the
-    // runs of one digit written by neighbouring tiles meet in the same L2 and leave it as full lines; measured
-    // 15% faster per pass than arrival order at C = 16. The predecessor of a tile may then belong to a workgroup
-    // dispatched up to 8 (C - 1) places later: the waits only end if that many workgroups of this launch are
-    // resident at once, which holds on a device that runs nothing else and not, in general, next to other launches
-    // (their waiting workgroups can fill the places this launch needs). The host therefore passes C > 0 only for a
-    // caller that has declared the device its own. Tiles past the last whole group of 8 chunks, and every tile when
-    // C = 0, are numbered by arrival, so that all predecessors have started.
-    if (t == 0) {
-        const bool failed = dev_failed(a.err); // read while the ticket is on its way
-        u32 tl;
-        if (a.xcd_chunk == 0) {
-            tl = atomicAdd(a.ticket, 1u);
-        } else {
-            const u32 b = blockIdx.x;
-            const u32 span = 8u * a.xcd_chunk;
-            const u32 whole = (gridDim.x / span) * span;
-            tl = b;
-            if (b < whole) {
-                const u32 x = b % 8u, q = b / 8u;
-                tl = ((q / a.xcd_chunk) * 8u + x) * a.xcd_chunk + q % a.xcd_chunk;
-            }
-        }
-        if (failed)
-            tl = 0xFFFFFFFFu; // the step is lost already: leave
-        s_tile = tl;
-    }
+    if (t == 0)
+        s_tile = onesweep_tile_number(a);
     for (int i = t; i < WAVES * RADIX_BINS; i += BLOCK)
         s_whist[i] = 0;
     __syncthreads();
     const u32 tile = s_tile;
-    if (tile == 0xFFFFFFFFu)
+    if (tile == NO_TILE)
         return;
     const u64 base = (u64)tile * TILE;
     const u32 valid = (u32)((u64)a.n - base < (u64)TILE ? (u64)a.n - base : (u64)TILE);
@@ -284,8 +295,9 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
     };
 
     // ---- load: wave-striped, so that consecutive lanes read consecutive pairs ----
+    // (the values are fetched, or computed, only when they are needed: held from here they would cost ITEMS registers
+    // through the ranking, which is where the kernel is tightest)
     KeyT key[ITEMS];
-    u32 val[ITEMS];
     const u32 first_local = w * (WAVE * ITEMS) + lane;
     if (valid == (u32)TILE) { // every tile but the last: no bounds checks, all loads in flight at once
 #pragma unroll
@@ -293,13 +305,10 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
             const u64 i = base + first_local + k * WAVE;
             if (SRC == SRC_PAIRS) {
                 key[k] = keys_in[i];
-                val[k] = a.vals_in[i];
             } else if (SRC == SRC_TEXT) {
-                val[k] = virtual_to_suffix((u32)i, a.text_n, a.tail);
                 key[k] = (KeyT)text_key((u32)i);
             } else {
-                val[k] = a.vals_in[i];
-                key[k] = (KeyT)load_kgram(a.text, a.text_n, val[k], a.word);
+                key[k] = (KeyT)load_kgram(a.text, a.text_n, a.vals_in[i], a.word);
             }
         }
     } else {
@@ -308,18 +317,13 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
             const u32 local = first_local + k * WAVE;
             const u64 i = base + local;
             key[k] = ~(KeyT)0; // padding: largest digit, and behind every real pair of the tile
-            val[k] = 0;
             if (local < valid) {
-                if (SRC == SRC_PAIRS) {
+                if (SRC == SRC_PAIRS)
                     key[k] = keys_in[i];
-                    val[k] = a.vals_in[i];
-                } else if (SRC == SRC_TEXT) {
-                    val[k] = virtual_to_suffix((u32)i, a.text_n, a.tail);
+                else if (SRC == SRC_TEXT)
                     key[k] = (KeyT)text_key((u32)i);
-                } else {
-                    val[k] = a.vals_in[i];
-                    key[k] = (KeyT)load_kgram(a.text, a.text_n, val[k], a.word);
-                }
+                else
+                    key[k] = (KeyT)load_kgram(a.text, a.text_n, a.vals_in[i], a.word);
             }
         }
     }
@@ -411,6 +415,14 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
     }
     __syncthreads();
     u32* s_vals = reinterpret_cast<u32*>(s_keys);
+    u32 val[ITEMS];
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const u32 local = first_local + k * WAVE;
+        val[k] = 0;
+        if (local < valid)
+            val[k] = SRC == SRC_TEXT ? virtual_to_suffix((u32)(base + local), a.text_n, a.tail) : a.vals_in[base + local];
+    }
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k)
         s_vals[pos[k]] = val[k];
