@@ -609,24 +609,19 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     u32* V[2] = {h->idx[0], h->idx[1]};
     int cur; // the (K, V) set that holds the sorted pairs
     int rc;
-    if (h->key_words == 1) {
-        rc = radix_sort(L, SRC_TEXT, d_text, n, tail, 0, K[0], V[0], K[1], V[1], n, full, &in_out, &passes);
+    // A key of W words is sorted word by word, the least significant word first: the first sort builds its keys
+    // straight from the text, every following (stable) sort rebuilds its word from the text through the suffix
+    // indices the sort before it left.
+    cur = 0;
+    for (int word = h->key_words - 1; word >= 0; --word) {
+        const bool first_sort = word == h->key_words - 1;
+        rc = radix_sort(L, first_sort ? SRC_TEXT : SRC_TEXT_IDX, d_text, n, tail, (u32)word, K[cur], V[cur], K[cur ^ 1], V[cur ^ 1],
+                        n, full, &in_out, &p1);
         if (rc)
             return rc;
-        cur = in_out ? 1 : 0;
-    } else {
-        // 128-bit key: sort by the least significant word first, then stably by the most significant
-        // word, which is rebuilt from the text through the suffix indices of the first sort
-        rc = radix_sort(L, SRC_TEXT, d_text, n, tail, 1, K[0], V[0], K[1], V[1], n, full, &in_out, &p1);
-        if (rc)
-            return rc;
-        const int r1 = in_out ? 1 : 0;
-        rc = radix_sort(L, SRC_TEXT_IDX, d_text, n, tail, 0, K[r1], V[r1], K[r1 ^ 1], V[r1 ^ 1], n, full, &in_out,
-                        &passes);
-        if (rc)
-            return rc;
-        cur = in_out ? (r1 ^ 1) : r1;
         passes += p1;
+        if (in_out)
+            cur ^= 1;
     }
     u64* k_sorted = K[cur];
     u32* sa32 = V[cur]; // from here on the suffix array under construction
@@ -1349,8 +1344,8 @@ int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
     if (!out)
         return fail(CSA_ERR_ARG, "csa_create: out is null");
     *out = nullptr;
-    if (key_words != 1 && key_words != 2)
-        return fail(CSA_ERR_ARG, "csa_create: key_words must be 1 or 2, got %d", key_words);
+    if (key_words < 1 || key_words > 4)
+        return fail(CSA_ERR_ARG, "csa_create: key_words = %d is outside [1, 4]", key_words);
     if (max_part_sz > CSA_MAX_PART_SZ)
         return fail(CSA_ERR_TOO_LARGE, "csa_create: %llu suffixes exceed the partition limit %llu",
                     (unsigned long long)max_part_sz, (unsigned long long)CSA_MAX_PART_SZ);
@@ -1535,8 +1530,8 @@ int csa_sort_partition_u16(const uint16_t* h_text, uint64_t n, int key_words, ui
 
 int csa_pack_keys_u16_dev(const uint16_t* d_text, uint64_t n, int key_words, uint64_t* d_keys, void* stream)
 {
-    if (key_words != 1 && key_words != 2)
-        return fail(CSA_ERR_ARG, "csa_pack_keys_u16_dev: key_words must be 1 or 2, got %d", key_words);
+    if (key_words < 1 || key_words > 4)
+        return fail(CSA_ERR_ARG, "csa_pack_keys_u16_dev: key_words = %d is outside [1, 4]", key_words);
     if (n > CSA_MAX_PART_SZ)
         return fail(CSA_ERR_TOO_LARGE, "csa_pack_keys_u16_dev: %llu suffixes exceed the partition limit",
                     (unsigned long long)n);

@@ -26,7 +26,7 @@ struct RerankArgs {
     const u64* keys;
     const u32* sufs;
     u32 m;         // = n: generation 0 ranks every suffix
-    int key_words; // 1 or 2 (the low word is re-read from the text when 2)
+    int key_words; // 1..4 (the words after the first are re-read from the text where the first words tie)
     u32 n;         // partition size
     u32 ell;       // symbols in the generation-0 key
     const u16* text;
@@ -107,8 +107,8 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
     for (int k = 0; k < ITEMS + 1; ++k) {
         const u64 c = base + k; // right element of the pair
         bool e = c >= 1 && c < m && key[k] == key[k + 1];
-        if (e && a.key_words == 2)
-            e = load_kgram(a.text, a.n, suf[k], 1) == load_kgram(a.text, a.n, suf[k + 1], 1);
+        for (int word = 1; e && word < a.key_words; ++word)
+            e = load_kgram(a.text, a.n, suf[k], (u32)word) == load_kgram(a.text, a.n, suf[k + 1], (u32)word);
         // a suffix that runs off the text inside its key ties with nobody (include/bit-layout.hpp:99-100)
         if (e && ((u64)suf[k] + a.ell >= a.n || (u64)suf[k + 1] + a.ell >= a.n))
             e = false;

@@ -69,6 +69,20 @@ def test_fixtures_through_the_emulated_kernels(emu, key_words):
         assert active == counts, name
 
 
+@pytest.mark.parametrize("key_words", [3, 4])
+def test_keys_of_three_and_four_words(emu, key_words):
+    # the reference's default key is 4 words (16 symbols): generation 0 sorts word by word and compares the later words
+    # through the text; texts shorter than a key, and runs that tie over a whole key, are the edge cases
+    suite = dict(texts.fixture_suite())
+    for name, T in [(n_, suite[n_]) for n_ in ("rand_n17_s2", "rand_n1000_s2", "hand_15")] + [
+            ("run", np.concatenate([np.full(40, 3, dtype=np.uint16), texts.random_text(300, 2, 9, sep_every=0)])),
+            ("short", np.array([2, 1, 2, 1, 2], dtype=np.uint16))]:
+        got, active, _ = emu_sort(emu, T, key_words)
+        assert np.array_equal(got, oracle_lib.build_sa40(T)), name
+        _, counts = oracle_lib.prefix_doubling(T, key_words)
+        assert active == counts, name
+
+
 @pytest.mark.parametrize("key_words", [1, 2])
 def test_text_at_every_alignment_inside_an_eight_byte_word(emu, key_words):
     # the first pass stages the text with aligned 8-byte loads: the text may start anywhere inside such a word, and

@@ -57,7 +57,7 @@ def gpu_sa40(torch, s, T, index_base=0):
 
 # ---- stage: K-gram key packing ---------------------------------------------------------------------
 
-@pytest.mark.parametrize("key_words", [1, 2])
+@pytest.mark.parametrize("key_words", [1, 2, 3, 4])
 def test_pack_keys_matches_oracle(torch_mod, key_words):
     from cascade_amd import pack_keys
     for n, sigma, seed in ((1, 4, 0), (3, 4, 1), (4, 4, 2), (5, 65536, 3), (1000, 65536, 4), (100003, 65536, 5)):
@@ -256,7 +256,7 @@ def test_sixteen_million_symbols_pass_the_oracle_verifier(torch_mod, config):
 
 
 def test_random_small_texts_against_the_oracle(torch_mod):
-    """Many short texts over tiny alphabets (long ties, groups that straddle tiles, tails of zeros), both key widths,
+    """Many short texts over tiny alphabets (long ties, groups that straddle tiles, tails of zeros), all four key widths,
     on exact-size handles: byte-equal to the oracle's comparison sort."""
     from cascade_amd import PartitionSorter
     rng = np.random.default_rng(2024)
@@ -268,11 +268,26 @@ def test_random_small_texts_against_the_oracle(torch_mod):
             T[-int(rng.integers(1, min(n, 40) + 1)):] = 0
         if case % 4 == 1 and n > 600:
             T[n // 2:n // 2 + 256] = T[:256]  # a long repeat
-        kw = 1 + case % 2
+        kw = 1 + case % 4
         with PartitionSorter(n, key_words=kw) as s:
             print(f"  random case={case} n={n} sigma={sigma} key_words={kw}", flush=True)
             got = s.sort(to_dev(torch_mod, T)).cpu().numpy()
         assert np.array_equal(got, oracle_lib.build_sa40(T)), (case, n, sigma, kw)
+
+
+@pytest.mark.parametrize("key_words", [3, 4])
+def test_keys_of_three_and_four_words_on_deep_repeats(torch_mod, key_words):
+    """The reference's default key is 4 words (include/Packed_Prefix.hpp:20-24): the same suffix array, fewer and
+    smaller generations, whose sizes must be the oracle's for that key width."""
+    from cascade_amd import PartitionSorter, workloads
+    with PartitionSorter(1 << 19, key_words=key_words) as s:
+        for config in (3, 5, 4):
+            T = workloads.generate(config, 1 << 19)
+            got = gpu_sa40(torch_mod, s, T)
+            sa, counts = oracle_lib.prefix_doubling(T, key_words)
+            assert np.array_equal(got, oracle_lib.u64_to_sa40(sa)), config
+            assert s.last_stats["active"] == counts, config
+            assert s.last_stats["passes"][0] >= 1
 
 
 def test_three_dispatcher_threads_with_their_own_handles_and_streams(torch_mod):
