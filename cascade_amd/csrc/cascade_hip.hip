@@ -1064,8 +1064,8 @@ namespace {
 // Shared tail of the two partition steps: the list (keys, suffix words, routing tags) sorted by key is ranked and split
 // into active / retired, the cohort's messages are emitted, ranks and lanes are narrowed for the caller.
 template <bool GEN0>
-int finish_partition_step(Launch& L, const u64* sorted_key0, const u64* sorted_key1, const u64* sorted_words, const u32* sorted_beta,
-                          u64 m, u64 ctx, u32 p, u64* key_r, u64* words_r, u32* beta_r, u32* d_rank_out, u8* d_suf40_out,
+int finish_partition_step(Launch& L, const u64* sorted_key0, const u64* sorted_key1, const u64* keys_src, const u32* perm, int key_words,
+                          const u64* sorted_words, const u32* sorted_beta, u64 m, u64 ctx, u32 p, u64* key_r, u64* words_r, u32* beta_r, u32* d_rank_out, u8* d_suf40_out,
                           u8* d_msg_target, u32* d_msg_rank, u32* d_msg_off, csa_step_result* res)
 {
     csa_handle* h = L.h;
@@ -1075,6 +1075,9 @@ int finish_partition_step(Launch& L, const u64* sorted_key0, const u64* sorted_k
     StepRankArgs ra;
     ra.key0 = sorted_key0;
     ra.key1 = sorted_key1;
+    ra.keys_src = keys_src;
+    ra.perm = perm;
+    ra.key_words = key_words;
     ra.words = sorted_words;
     ra.beta = sorted_beta;
     ra.m = m;
@@ -1150,8 +1153,8 @@ int csa_sort_init_dev(csa_handle* h, const uint64_t* d_keys, int key_words, cons
                       uint64_t m, uint32_t p, uint32_t* d_rank_out, uint8_t* d_suf40_out, uint8_t* d_msg_target,
                       uint32_t* d_msg_rank, uint32_t* d_msg_off, void* stream, csa_step_result* res)
 {
-    if (key_words != 1 && key_words != 2)
-        return fail(CSA_ERR_ARG, "csa_sort_init_dev: key_words must be 1 or 2");
+    if (key_words < 1 || key_words > 4)
+        return fail(CSA_ERR_ARG, "csa_sort_init_dev: key_words = %d is outside [1, 4]", key_words);
     int rc = check_step_args(h, "csa_sort_init_dev", m, p, d_keys, d_suf40, d_beta, d_msg_off);
     if (rc)
         return rc;
@@ -1194,16 +1197,17 @@ int csa_sort_init_dev(csa_handle* h, const uint64_t* d_keys, int key_words, cons
     }
     // sorted: key word 0 in K[kc], the permutation in P[pc]
     u64* sorted_key1 = nullptr;
-    if (key_words == 2) {
+    if (key_words >= 2) {
         sorted_key1 = K[kc ^ 1];
-        hipLaunchKernelGGL(gather_u64_kernel, dim3(blocks), dim3(256), 0, s, (const u64*)d_keys, (const u32*)P[pc], m, 2u, 1u, sorted_key1);
+        hipLaunchKernelGGL(gather_u64_kernel, dim3(blocks), dim3(256), 0, s, (const u64*)d_keys, (const u32*)P[pc], m, (u32)key_words, 1u,
+                           sorted_key1);
     }
     u64* sorted_words = h->key[2];
     u32* sorted_beta = h->idx[2];
     hipLaunchKernelGGL(unpack_words_kernel, dim3(blocks), dim3(256), 0, s, d_suf40, d_beta, (const u32*)P[pc], m, 1, sorted_words,
                        sorted_beta);
     HIP_TRY(hipGetLastError());
-    return finish_partition_step<true>(L, K[kc], sorted_key1, sorted_words, sorted_beta, m, 4ull * (u64)key_words, p, h->step64[0],
+    return finish_partition_step<true>(L, K[kc], sorted_key1, d_keys, P[pc], key_words, sorted_words, sorted_beta, m, 4ull * (u64)key_words, p, h->step64[0],
                                        h->step64[1], h->idx[3], d_rank_out, d_suf40_out, d_msg_target, d_msg_rank, d_msg_off, res);
 }
 
@@ -1279,7 +1283,7 @@ int csa_sort_rerank_dev(csa_handle* h, const uint32_t* d_rank, const uint8_t* d_
     hipLaunchKernelGGL(gather_u32_kernel, dim3(blocks), dim3(256), 0, s, (const u32*)beta_by_suffix, (const u32*)perm, m, sorted_beta);
     HIP_TRY(hipGetLastError());
     // 4. refine, split, messages, narrow
-    return finish_partition_step<false>(L, sorted_keys, nullptr, sorted_words, sorted_beta, m, ctx, p, h->step64[1], spare64,
+    return finish_partition_step<false>(L, sorted_keys, nullptr, nullptr, nullptr, 1, sorted_words, sorted_beta, m, ctx, p, h->step64[1], spare64,
                                         primary_by_suffix, d_rank_out, d_suf40_out, d_msg_target, d_msg_rank, d_msg_off, res);
 }
 

@@ -78,7 +78,10 @@ __global__ __launch_bounds__(256) void unpack_words_kernel(const u8* __restrict_
 // order; retired ones follow (reference: cub::DevicePartition::Flagged, which reverses them: their order carries nothing).
 struct StepRankArgs {
     const u64* key0;  // generation 0: sorted key word 0; generation t: sorted composite keys
-    const u64* key1;  // generation 0 with 128-bit keys: sorted key word 1, else null
+    const u64* key1;  // generation 0 with keys of two or more words: sorted key word 1, else null
+    const u64* keys_src; // generation 0 with keys of three or four words: the caller's keys (key_words per suffix) ...
+    const u32* perm;     // ... and the permutation that sorted them: words 2 and 3 are compared through it where words 0
+    int key_words;       //     and 1 tie
     const u64* words; // suffix words in the same order (generation 0: forward tag in the top 16 bits)
     const u32* beta;
     u64 m;
@@ -97,8 +100,12 @@ struct StepRankArgs {
 template <bool GEN0>
 __device__ __forceinline__ bool step_same_key(const StepRankArgs& a, u64 i, u64 j)
 {
-    if (GEN0)
-        return a.key0[i] == a.key0[j] && (!a.key1 || a.key1[i] == a.key1[j]) && (a.words[i] >> 48) == (a.words[j] >> 48);
+    if (GEN0) {
+        bool same = a.key0[i] == a.key0[j] && (!a.key1 || a.key1[i] == a.key1[j]) && (a.words[i] >> 48) == (a.words[j] >> 48);
+        for (int w = 2; same && w < a.key_words; ++w)
+            same = a.keys_src[(u64)a.perm[i] * a.key_words + w] == a.keys_src[(u64)a.perm[j] * a.key_words + w];
+        return same;
+    }
     return a.key0[i] == a.key0[j]; // whole words: tied entries agree on the pill receipt
 }
 

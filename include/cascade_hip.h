@@ -208,7 +208,7 @@ typedef struct csa_step_result {
 } csa_step_result;
 
 /* Generation 0 of one partition of m suffixes (m <= the handle's capacity), everything resident in HBM:
- *   in : d_keys[i * key_words + w] packed K-gram words, d_suf40 5-byte lanes, d_beta routing-tag pairs (forward tag in
+ *   in : d_keys[i * key_words + w] packed K-gram words (key_words 1 to 4), d_suf40 5-byte lanes, d_beta routing-tag pairs (forward tag in
  *        the high half), in any order: what csa_stage_slab_u16_dev (or the reference's stage_slab) produces;
  *   out: d_rank_out[i] partition-local ranks (offset of the head of the run of equal (key, forward tag)) and
  *        d_suf40_out lanes, the tied ("active") suffixes first, in sorted order, the retired ones after them;

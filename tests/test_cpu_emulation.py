@@ -236,7 +236,7 @@ def test_multi_partition_pipeline_through_the_emulated_stage_kernels(emu, p, key
         assert gens >= 6 and sum(step[5] for step in log if step[0] >= 1) > 0  # pills travelled in later generations
 
 
-@pytest.mark.parametrize("p,key_words,sigma,n", [(5, 2, 2, 900), (4, 1, 2, 1300)])
+@pytest.mark.parametrize("p,key_words,sigma,n", [(5, 4, 2, 900), (4, 1, 2, 1300)])
 def test_multi_partition_pipeline_with_the_emulated_step_entries(emu, p, key_words, sigma, n):
     """The same pipeline with each partition step as one call of csa_sort_init_dev / csa_sort_rerank_dev."""
     import multi_partition

@@ -34,7 +34,8 @@ def gpu():
 
 
 @pytest.mark.parametrize("p,key_words,sorted_join,steps", [(3, 1, False, False), (16, 1, True, False), (33, 2, False, False),
-                                                           (3, 1, False, True), (16, 2, False, True), (40, 1, False, True)])
+                                                           (3, 1, False, True), (16, 2, False, True), (40, 1, False, True),
+                                                           (9, 3, False, True), (16, 4, False, True), (5, 4, False, False)])
 def test_partitions_that_only_exchange_messages_build_the_oracles_suffix_array(gpu, p, key_words, sorted_join, steps):
     """steps = False: numpy glue between the exported stage kernels; True: each partition step is one call of
     csa_sort_init_dev / csa_sort_rerank_dev."""
