@@ -2,6 +2,7 @@
 
   libcascade_hip.so        hand-written HIP for gfx950 behind the C ABI of include/cascade_hip.h
   libcascade_workloads.so  host-only generator of the synthetic benchmark partitions
+  cascade_sa               the reference's command-line builder (text file in, sa40 file out) over the C ABI
 
 Run as `python -m cascade_amd.build`. hipcc cross-compiles for gfx950 without a GPU.
 """
@@ -13,6 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 HIP_LIB = os.path.join(HERE, "libcascade_hip.so")
 WORKLOADS_LIB = os.path.join(HERE, "libcascade_workloads.so")
+CLI = os.path.join(HERE, "cascade_sa")
 
 HIPCC_FLAGS = [
     "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared", "-Wall",
@@ -42,9 +44,19 @@ def build_workloads():
     return WORKLOADS_LIB
 
 
+def build_cli():
+    """The host-side mirror of the reference's builder (include/cascade_gpu_saca.hpp) as a program: plain g++, linked
+    against libcascade_hip.so next to it."""
+    cxx = os.environ.get("CXX", "g++")
+    _run([cxx, "-std=c++17", "-O2", "-Wall", "-Wextra", "-Werror", "-o", CLI, os.path.join(CSRC, "cascade_sa.cpp"),
+          "-L" + HERE, "-lcascade_hip", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath-link,/opt/rocm/lib"])
+    return CLI
+
+
 def build_all():
     build_hip()
     build_workloads()
+    build_cli()
 
 
 if __name__ == "__main__":

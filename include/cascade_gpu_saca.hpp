@@ -1,0 +1,191 @@
+// cascade_gpu_saca.hpp : the reference's builder surface over the C ABI of cascade_hip.h, header only, plain C++17
+// (no HIP header: device pointers and streams travel as plain pointers, as in the C ABI).
+//
+// Names, argument meaning and error behaviour follow gpu_saca::GPU_SACA<T_sym_> (reference: include/GPU_SACA.hpp:39-310):
+//   GPU_SACA(ip_path, op_path) / build_SA()        include/GPU_SACA.hpp:304-310, src/main.cu:27-30
+//   partition_size_upper_bound()                   include/GPU_SACA.hpp:209
+//   allocate_device_space()                        include/GPU_SACA.hpp:221
+//   set_context(ctx, gen)                          include/GPU_SACA.hpp:236
+//   sort_and_init_rank_and_filter(p_id, ., buf_id) include/GPU_SACA.hpp:272
+//   sort_and_re_rank_and_filter(p_id, ., buf_id)   include/GPU_SACA.hpp:279
+//   scatter_to_rank_order(p_id, ., buf_id)         include/GPU_SACA.hpp:288
+// Where the reference passes a Partition_Assembly (pinned host slabs that its pipeline uploads and downloads around the
+// call, include/Staging_Slab.hpp:20-119), the members here take a Device_Partition: the same columns, already in HBM.
+// A failure prints the library's message and ends the process, as CUDA_CHECK does (include/utility.cuh:19-29); code
+// that wants the status instead calls the C ABI directly.
+#ifndef CASCADE_GPU_SACA_HPP
+#define CASCADE_GPU_SACA_HPP
+
+#include "cascade_hip.h"
+
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <fstream>
+#include <iostream>
+#include <string>
+#include <vector>
+
+namespace cascade_hip {
+
+using idx_t = std::uint64_t;  // text positions, sizes (reference: include/types.hpp:12-16)
+using p_id_t = std::uint16_t; // partition ids
+using p_sz_t = std::uint32_t; // partition-local ranks
+using beta_t = std::uint32_t; // pair of routing tags
+
+// One partition's columns on the device, before and after a step (the device-side image of a Partition_Assembly).
+struct Device_Partition {
+    idx_t sz = 0;                         // suffixes in the cohort handed to the step
+    const std::uint64_t* key = nullptr;   // generation 0: packed K-gram words, key_words per suffix (Staging_Slab::key())
+    const p_sz_t* rank = nullptr;         // later generations: the partition-local ranks kept from the step before
+    const std::uint8_t* suf = nullptr;    // 5-byte lanes (Staging_Slab::suf())
+    const beta_t* beta = nullptr;         // routing tags (Staging_Slab::beta())
+    const std::uint8_t* inbox_target = nullptr; // later generations: the messages delivered to this partition
+    const p_sz_t* inbox_rank = nullptr;
+    std::uint32_t inbox_sz = 0;
+    p_sz_t* rank_out = nullptr;           // outputs: ranks and lanes, active suffixes first
+    std::uint8_t* suf_out = nullptr;
+    std::uint8_t* msg_target = nullptr;   // outbox, grouped by destination partition
+    p_sz_t* msg_rank = nullptr;
+    p_sz_t* msg_off = nullptr;            // p + 1 counters: exclusive end of every destination's group
+    idx_t active_sz = 0;                  // filled by the step: the new active-set size (active_set_sz[p_id])
+    idx_t msg_c = 0;                      // filled by the step: messages in the outbox
+};
+
+template <typename T_sym_> class GPU_SACA {
+    static_assert(sizeof(T_sym_) == 2, "the partition sort is built for uint16 symbols");
+
+public:
+    static constexpr idx_t STREAM_C = 3; // buffer sets, one dispatcher thread each (include/GPU_SACA.hpp:90)
+
+    // The reference's command-line use: the text at ip_path is one partition, its suffix array goes to op_path.
+    GPU_SACA(const std::string& ip_path, const std::string& op_path, int key_words = 1)
+        : ip_path_(ip_path), op_path_(op_path), key_words_(key_words)
+    {
+    }
+
+    // For a pipeline that drives partitions itself: p partitions of at most max_part_sz suffixes.
+    GPU_SACA(idx_t max_part_sz, p_id_t p, int key_words = 1) : key_words_(key_words), p_(p), max_part_sz_(max_part_sz) {}
+
+    GPU_SACA(const GPU_SACA&) = delete;
+    GPU_SACA& operator=(const GPU_SACA&) = delete;
+
+    ~GPU_SACA()
+    {
+        for (idx_t b = 0; b < STREAM_C; ++b)
+            if (csa_[b])
+                csa_destroy(csa_[b]);
+    }
+
+    // Largest partition that STREAM_C buffer sets of the library's floor plan fit into free_device_bytes (the
+    // reference balances three partitions over the device memory the same way, src/GPU_SACA.cu:372,557).
+    idx_t partition_size_upper_bound(std::size_t free_device_bytes) const
+    {
+        const idx_t by_memory = free_device_bytes / (STREAM_C * csa_bytes_per_suffix(key_words_));
+        return by_memory < CSA_MAX_PART_SZ ? by_memory : CSA_MAX_PART_SZ;
+    }
+
+    // One handle per buffer set; false if the device has no room (the reference returns the same way).
+    bool allocate_device_space()
+    {
+        for (idx_t b = 0; b < STREAM_C; ++b)
+            if (!csa_[b] && csa_create(max_part_sz_, key_words_, &csa_[b]) != CSA_OK) {
+                std::cerr << csa_last_error() << "\n";
+                return false;
+            }
+        return true;
+    }
+
+    // The stream (a hipStream_t) of a buffer set; the default stream otherwise.
+    void set_stream(idx_t buf_id, void* stream) { stream_[buf_id] = stream; }
+
+    // Context the coming generation resolves to, and its index (src/GPU_SACA.cu:1043-1049).
+    void set_context(idx_t ctx, idx_t gen)
+    {
+        ctx_ = ctx;
+        gen_ = gen;
+    }
+
+    void sort_and_init_rank_and_filter(p_id_t /*p_id*/, Device_Partition& part, idx_t buf_id)
+    {
+        csa_step_result r{};
+        check(csa_sort_init_dev(csa_[buf_id], part.key, key_words_, part.suf, part.beta, part.sz, p_, part.rank_out, part.suf_out,
+                                part.msg_target, part.msg_rank, part.msg_off, stream_[buf_id], &r));
+        part.active_sz = r.active;
+        part.msg_c = r.messages;
+    }
+
+    void sort_and_re_rank_and_filter(p_id_t /*p_id*/, Device_Partition& part, idx_t buf_id)
+    {
+        csa_step_result r{};
+        check(csa_sort_rerank_dev(csa_[buf_id], part.rank, part.suf, part.beta, part.sz, part.inbox_target, part.inbox_rank,
+                                  part.inbox_sz, ctx_, p_, part.rank_out, part.suf_out, part.msg_target, part.msg_rank,
+                                  part.msg_off, stream_[buf_id], &r));
+        part.active_sz = r.active;
+        part.msg_c = r.messages;
+    }
+
+    // part_sz suffixes (lanes) with their final partition-local ranks -> the partition's stretch of the suffix array.
+    void scatter_to_rank_order(p_id_t /*p_id*/, const std::uint8_t* suf, const p_sz_t* rank, idx_t part_sz, std::uint8_t* sa40,
+                               idx_t buf_id)
+    {
+        check(csa_scatter_to_rank_order_dev(csa_[buf_id], suf, rank, part_sz, sa40, stream_[buf_id]));
+    }
+
+    // A partition whose symbols are a window of the text resident in HBM: every generation inside one call.
+    void sort_partition(const T_sym_* d_text, idx_t part_sz, idx_t index_base, std::uint8_t* d_sa40, idx_t buf_id,
+                        csa_stats* stats = nullptr)
+    {
+        check(csa_sort_partition_u16_dev(csa_[buf_id], reinterpret_cast<const std::uint16_t*>(d_text), part_sz, index_base, d_sa40,
+                                         stream_[buf_id], 0, stats));
+    }
+
+    // Builds the suffix array of the text file as one partition and writes it as 5-byte entries (src/main.cu:27-30).
+    void build_SA()
+    {
+        std::ifstream in(ip_path_, std::ios::binary | std::ios::ate);
+        if (!in)
+            fail("cannot open " + ip_path_);
+        const std::streamoff bytes = in.tellg();
+        if (bytes % 2 != 0)
+            fail(ip_path_ + " does not hold whole 16-bit symbols");
+        std::vector<std::uint16_t> text(static_cast<std::size_t>(bytes / 2));
+        in.seekg(0);
+        in.read(reinterpret_cast<char*>(text.data()), bytes);
+        if (!in && bytes)
+            fail("cannot read " + ip_path_);
+        std::vector<std::uint8_t> sa40(5 * text.size());
+        check(csa_sort_partition_u16(text.data(), text.size(), key_words_, sa40.data(), &stats_));
+        std::ofstream out(op_path_, std::ios::binary | std::ios::trunc);
+        out.write(reinterpret_cast<const char*>(sa40.data()), static_cast<std::streamsize>(sa40.size()));
+        if (!out)
+            fail("cannot write " + op_path_);
+    }
+
+    const csa_stats& stats() const { return stats_; } // generations and their sizes of the last build_SA()
+
+private:
+    [[noreturn]] static void fail(const std::string& what)
+    {
+        std::cerr << what << ". Aborting.\n";
+        std::exit(EXIT_FAILURE);
+    }
+    static void check(int status)
+    {
+        if (status != CSA_OK)
+            fail(csa_last_error());
+    }
+
+    std::string ip_path_, op_path_;
+    int key_words_ = 1;
+    p_id_t p_ = 1;
+    idx_t max_part_sz_ = 0;
+    idx_t ctx_ = 0, gen_ = 0;
+    csa_handle* csa_[STREAM_C] = {};
+    void* stream_[STREAM_C] = {};
+    csa_stats stats_{};
+};
+
+} // namespace cascade_hip
+
+#endif

@@ -35,10 +35,23 @@ def test_argument_errors_need_no_gpu():
     lib = _native.load()
     assert lib.csa_bytes_per_suffix(1) == 60
     h = C.c_void_p()
-    assert lib.csa_create(10, 3, C.byref(h)) == _native.CSA_ERR_ARG
+    assert lib.csa_create(10, 5, C.byref(h)) == _native.CSA_ERR_ARG
     assert b"key_words" in lib.csa_last_error()
     assert lib.csa_create(1 << 31, 1, C.byref(h)) == _native.CSA_ERR_TOO_LARGE
     assert lib.csa_sort_partition_u16(None, 1 << 31, 1, None, None) == _native.CSA_ERR_TOO_LARGE
     assert lib.csa_sort_partition_u16_dev(None, None, 0, 0, None, None, 0, None) == _native.CSA_ERR_ARG
     with pytest.raises(_native.CascadeError):
         _native.check(lib.csa_radix_sort_pairs_dev(None, None, None, 0, 0, 64, None))
+
+
+def test_builder_mirror_compiles_as_plain_cpp_and_the_program_is_built():
+    """include/cascade_gpu_saca.hpp (the reference's builder surface over the C ABI) needs no HIP header, and
+    cascade_amd/cascade_sa, the command-line builder made from it, refuses a call without arguments as the reference's
+    program does (src/main.cu:15-19)."""
+    import subprocess
+    hdr = os.path.join(ROOT, "include", "cascade_gpu_saca.hpp")
+    subprocess.run(["g++", "-std=c++17", "-fsyntax-only", "-Wall", "-Wextra", "-Werror", "-x", "c++", hdr], check=True)
+    exe = os.path.join(ROOT, "cascade_amd", "cascade_sa")
+    assert os.path.exists(exe), "run python -m cascade_amd.build"
+    r = subprocess.run([exe], capture_output=True, text=True)
+    assert r.returncode == 1 and "Usage:" in r.stderr

@@ -325,3 +325,23 @@ def test_three_dispatcher_threads_with_their_own_handles_and_streams(torch_mod):
     for th in threads:
         th.join()
     assert not errors, errors
+
+
+def test_command_line_builder_writes_the_oracles_suffix_array(tmp_path):
+    """cascade_amd/cascade_sa <text-file> <suffix-array-file>: the reference's program (src/main.cu:12-46) through the
+    C++ mirror of its builder class; the file it writes is the oracle's, byte for byte; a missing input ends it with
+    an error message and status 1, as the reference's error policy does."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "cascade_amd", "cascade_sa")
+    for name, T in (("c1", texts.random_text(200000, 50257, 1, sep_every=1000)), ("ties", texts.random_text(50000, 2, 2, sep_every=0)),
+                    ("empty", np.zeros(0, dtype=np.uint16))):
+        ip, op = tmp_path / f"{name}.u16", tmp_path / f"{name}.sa40"
+        T.astype("<u2").tofile(ip)
+        print(f"  cascade_sa {name} n={T.size}", flush=True)
+        for key_words in (1, 4):
+            r = subprocess.run([exe, str(ip), str(op), str(key_words)], capture_output=True, text=True, timeout=100)
+            assert r.returncode == 0 and "Time taken" in r.stderr, r.stderr
+            assert np.array_equal(np.fromfile(op, dtype=np.uint8), oracle_lib.build_sa40(T)), (name, key_words)
+    r = subprocess.run([exe, str(tmp_path / "missing.u16"), str(tmp_path / "x.sa40")], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 1 and "cannot open" in r.stderr
