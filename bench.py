@@ -350,15 +350,21 @@ def bench_next_rows(args):
     else:  # scatter
         rank = torch.randperm(n, device=dev).to(torch.int32)
         lanes = torch.randint(0, 256, (5 * n,), dtype=torch.uint8, device=dev)
-        s = PartitionSorter(16)
         out = torch.empty(5 * n + 128, dtype=torch.uint8, device=dev)
-        ms, _ = _timed(torch, lambda: s.scatter_to_rank_order(lanes, rank, out=out), args.steps, args.warmup)
         h_rank = rank[:cs].cpu().numpy().view(np.uint32).astype(np.int64)
-        got = out[:5 * n].view(n, 5)[torch.from_numpy(h_rank).to(dev)].cpu().numpy()
-        ok = bool(np.array_equal(got, lanes[:5 * cs].view(cs, 5).cpu().numpy()))
-        s.close()
-        res = _row_result("suffixes scattered to rank order/sec at 1 GPU", "random permutation of ranks", n, ms, "scatter_lanes_kernel",
-                          n * 14, {}, args.steps, args.warmup, ok)
+
+        def run(capacity):  # a handle smaller than the partition scatters directly, one that holds it buckets by windows first
+            s = PartitionSorter(capacity)
+            out.zero_()
+            ms, _ = _timed(torch, lambda: s.scatter_to_rank_order(lanes, rank, out=out), args.steps, args.warmup)
+            got = out[:5 * n].view(n, 5)[torch.from_numpy(h_rank).to(dev)].cpu().numpy()
+            s.close()
+            return ms, bool(np.array_equal(got, lanes[:5 * cs].view(cs, 5).cpu().numpy()))
+        ms_direct, ok_direct = run(16)
+        ms, ok = run(n)
+        res = _row_result("suffixes scattered to rank order/sec at 1 GPU", "random permutation of ranks", n, ms,
+                          "scatter_window_keys_kernel + one radix pass + scatter_window_lanes_kernel", n * 14,
+                          {"ms_direct_scatter": round(ms_direct, 3)}, args.steps, args.warmup, ok and ok_direct)
     print(json.dumps(res), flush=True)
     if not res["config"]["checked_against_oracle"]:
         sys.exit(1)

@@ -96,6 +96,16 @@ constexpr u32 DEFER_MIN = CSA_DEFER_MIN;
 #endif
 constexpr int WINDOW_LOG2 = CSA_WINDOW_LOG2;
 constexpr u32 WINDOW_MIN_CHANGED = CSA_WINDOW_MIN_CHANGED;
+// rank-order scatter of a whole partition: partitions of at least SCATTER_WINDOW_MIN suffixes are first grouped by
+// windows of 2^SCATTER_WINDOW_LOG2 ranks (40 MB of output, which the last-level cache holds)
+#ifndef CSA_SCATTER_WINDOW_LOG2
+#define CSA_SCATTER_WINDOW_LOG2 23
+#endif
+#ifndef CSA_SCATTER_WINDOW_MIN
+#define CSA_SCATTER_WINDOW_MIN (1u << 25)
+#endif
+constexpr u32 SCATTER_WINDOW_LOG2 = CSA_SCATTER_WINDOW_LOG2;
+constexpr u64 SCATTER_WINDOW_MIN = CSA_SCATTER_WINDOW_MIN;
 // smallest cohort for which the message join builds a directory over the suffix-ordered cohort first
 #ifndef CSA_JOIN_DIR_MIN
 #define CSA_JOIN_DIR_MIN 4096u
@@ -1299,15 +1309,38 @@ int csa_scatter_to_rank_order_dev(csa_handle* h, const uint8_t* d_suf, const uin
     if (part_sz > CSA_MAX_PART_SZ)
         return fail(CSA_ERR_TOO_LARGE, "csa_scatter_to_rank_order_dev: %llu suffixes exceed a partition", (unsigned long long)part_sz);
     hipStream_t s = (hipStream_t)stream;
-    HIP_TRY(hipMemsetAsync(h->counts + 3, 0, sizeof(u32), s));
-    hipLaunchKernelGGL(scatter_lanes_kernel, dim3((u32)((part_sz + 255) / 256)), dim3(256), 0, s, d_suf, d_rank, part_sz, d_sa40,
-                       h->counts + 3);
+    HIP_TRY(hipMemsetAsync(h->counts, 0, 4 * sizeof(u32), s));
+    const u32 blocks = (u32)((part_sz + 255) / 256);
+    if (part_sz >= SCATTER_WINDOW_MIN && part_sz <= h->cap) {
+        // large partition: group the pairs by the window of the output their rank falls into, then write window by window
+        Launch L;
+        L.h = h;
+        L.stream = s;
+        L.flags = 0;
+        L.stats = nullptr;
+        hipLaunchKernelGGL(scatter_window_keys_kernel, dim3(blocks), dim3(256), 0, s, d_suf, d_rank, part_sz, (int)SCATTER_WINDOW_LOG2,
+                           h->key[0], h->idx[0], h->counts + 3);
+        const int window_bits = bit_length((part_sz - 1) >> SCATTER_WINDOW_LOG2);
+        int in_out = 0, passes = 0;
+        const int rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, h->key[0], h->idx[0], h->key[1], h->idx[1], (u32)part_sz,
+                                  make_plan(40, 40 + window_bits), &in_out, &passes);
+        if (rc)
+            return rc;
+        hipLaunchKernelGGL(scatter_window_lanes_kernel, dim3(blocks), dim3(256), 0, s, (const u64*)h->key[in_out],
+                           (const u32*)h->idx[in_out], part_sz, d_sa40);
+    } else {
+        hipLaunchKernelGGL(scatter_lanes_kernel, dim3(blocks), dim3(256), 0, s, d_suf, d_rank, part_sz, d_sa40, h->counts + 3);
+    }
     HIP_TRY(hipGetLastError());
-    HIP_TRY(hipMemcpyAsync(h->h_pinned + 3, h->counts + 3, sizeof(u32), hipMemcpyDeviceToHost, s));
-    HIP_TRY(hipStreamSynchronize(s));
+    Launch R;
+    R.h = h;
+    R.stream = s;
+    R.flags = 0;
+    R.stats = nullptr;
+    const int rc_counts = read_counts(R, nullptr); // waits for the stream; a failed wait of the bucket pass ends here
     if (h->h_pinned[3])
         return fail(CSA_ERR_ARG, "csa_scatter_to_rank_order_dev: a rank lies outside [0, %llu)", (unsigned long long)part_sz);
-    return CSA_OK;
+    return rc_counts;
 }
 
 void csa_output_cut(uint64_t lo, uint64_t hi, uint64_t chunk_bytes, uint64_t c, uint64_t chunk_c, uint64_t out[6])

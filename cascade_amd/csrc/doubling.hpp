@@ -914,6 +914,14 @@ __global__ __launch_bounds__(256) void emit_sa40_kernel(const u32* __restrict__ 
 
 __device__ __forceinline__ u64 load_sa40(const u8* sa, u64 r);
 
+// One 5-byte entry to its place (plain byte stores: a 4 + 1 byte split measured the same).
+__device__ __forceinline__ void store_sa40(u8* __restrict__ out, u64 r, u64 v)
+{
+#pragma unroll
+    for (int b = 0; b < 5; ++b)
+        out[5 * r + b] = (u8)(v >> (8 * b));
+}
+
 // Rank-order scatter of a partition that arrives as (suffix lane, local rank) pairs in any order:
 // out lane[rank[i]] = lane[i]. The reference scatters into 8-byte words and packs the lanes in a second kernel
 // (include/GPU_SACA.cuh:167-182 and :126-133, src/GPU_SACA.cu:2133-2143); here the 5 bytes go straight to their place.
@@ -929,10 +937,39 @@ __global__ __launch_bounds__(256) void scatter_lanes_kernel(const u8* __restrict
         atomicExch(bad, 1u);
         return;
     }
-    const u64 v = load_sa40(suf, i);
-#pragma unroll
-    for (int b = 0; b < 5; ++b)
-        out[5 * r + b] = (u8)(v >> (8 * b));
+    store_sa40(out, r, load_sa40(suf, i));
+}
+
+// The same scatter for large partitions, bucketed: 5-byte writes spread over gigabytes run at the rate of scattered
+// write requests, writes confined to a window that the last-level cache holds run about four times faster (the same
+// finding as for the rank updates above). Step 1 turns every pair into key = (window of its rank) << 40 | suffix and
+// value = rank; one radix pass on the window bits groups the pairs by window, in the order of the windows; step 3
+// writes the lanes of one window after the other.
+__global__ __launch_bounds__(256) void scatter_window_keys_kernel(const u8* __restrict__ suf, const u32* __restrict__ rank, u64 n,
+                                                                 int window_log2, u64* __restrict__ keys, u32* __restrict__ vals,
+                                                                 u32* bad)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n)
+        return;
+    u32 r = rank[i];
+    if (r >= n) {
+        atomicExch(bad, 1u);
+        r = 0; // keeps the pass in range; the call fails anyway
+    }
+    keys[i] = load_sa40(suf, i) | ((u64)(r >> window_log2) << 40);
+    vals[i] = r;
+}
+
+__global__ __launch_bounds__(256) void scatter_window_lanes_kernel(const u64* __restrict__ keys, const u32* __restrict__ vals, u64 n,
+                                                                  u8* __restrict__ out)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n)
+        return;
+    const u64 v = keys[i];
+    const u64 r = vals[i];
+    store_sa40(out, r, v);
 }
 
 // Standalone K-gram packing (reference: include/utility.hpp:147-162, include/Packed_Prefix.hpp:91-104).

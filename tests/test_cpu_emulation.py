@@ -69,8 +69,8 @@ def test_fixtures_through_the_emulated_kernels(emu, key_words):
         assert active == counts, name
 
 
-@pytest.mark.parametrize("key_words", [3, 4])
-def test_keys_of_three_and_four_words(emu, key_words):
+@pytest.mark.parametrize("key_words", [4])
+def test_keys_of_four_words(emu, key_words):
     # the reference's default key is 4 words (16 symbols): generation 0 sorts word by word and compares the later words
     # through the text; texts shorter than a key, and runs that tie over a whole key, are the edge cases
     suite = dict(texts.fixture_suite())
@@ -171,11 +171,13 @@ def test_emulated_slab_staging_and_rank_order_scatter(emu, generation0, ctx, key
     # and the way back: the same lanes scattered to a random rank order
     rank = rng.permutation(suf.size).astype(np.uint32)
     out = np.zeros(5 * suf.size, dtype=np.uint8)
-    h = C.c_void_p()
-    assert emu.csa_create(16, 1, C.byref(h)) == 0
-    rc = emu.csa_scatter_to_rank_order_dev(h, lanes.ctypes.data, rank.ctypes.data, suf.size, out.ctypes.data, None)
-    emu.csa_destroy(h)
-    assert rc == 0 and np.array_equal(out, oracle_lib.scatter_to_rank_order(lanes, rank)[1])
+    for capacity in (16, suf.size):  # a small handle scatters directly, one that holds the partition buckets it by windows
+        out[:] = 0
+        h = C.c_void_p()
+        assert emu.csa_create(capacity, 1, C.byref(h)) == 0
+        rc = emu.csa_scatter_to_rank_order_dev(h, lanes.ctypes.data, rank.ctypes.data, suf.size, out.ctypes.data, None)
+        emu.csa_destroy(h)
+        assert rc == 0 and np.array_equal(out, oracle_lib.scatter_to_rank_order(lanes, rank)[1]), capacity
 
 
 class HostArray:

@@ -72,17 +72,20 @@ def test_oracle_scatter_is_the_inverse_permutation():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("m", [1, 5, 255, 256, 257, 100003, 1 << 22])
-def test_gpu_scatter_to_rank_order_matches_the_oracle(m):
+@pytest.mark.parametrize("m,capacity", [(1, 16), (5, 16), (255, 16), (256, 16), (257, 16), (100003, 16), (1 << 22, 16),
+                                        ((1 << 25) + 12345, (1 << 25) + 12345), (1 << 26, 1 << 27)])
+def test_gpu_scatter_to_rank_order_matches_the_oracle(m, capacity):
+    """A handle smaller than the partition scatters directly; one that holds it buckets large partitions by windows of
+    the output first (same result)."""
     import torch
     from cascade_amd import PartitionSorter, _native
     rng = np.random.default_rng(m)
     suf = rng.integers(0, 1 << 40, m).astype(np.uint64)
     rank = rng.permutation(m).astype(np.uint32)
     lanes = oracle_lib.u64_to_sa40(suf)[:5 * m]
-    s = PartitionSorter(16)
+    s = PartitionSorter(capacity)
     try:
-        print(f"  scatter m={m}", flush=True)
+        print(f"  scatter m={m} capacity={capacity}", flush=True)
         out = s.scatter_to_rank_order(torch.from_numpy(lanes).cuda(), torch.from_numpy(rank.view(np.int32)).cuda())
         assert np.array_equal(out.cpu().numpy(), oracle_lib.scatter_to_rank_order(lanes, rank)[1])
         if m > 5:
