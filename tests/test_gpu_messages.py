@@ -75,12 +75,19 @@ def test_count_offsets_and_emit_match_the_oracle(gpu, packed, ctx):
 def test_join_matches_the_oracle(gpu):
     lib, to_dev, to_host = gpu
     rng = np.random.default_rng(3)
-    for n, hits, misses in ((1, 1, 3), (1000, 400, 100), (1 << 20, 300000, 50000)):
-        suf = np.sort(rng.choice(1 << 30, n, replace=False)).astype(np.uint64)
+    for n, hits, misses in ((1, 1, 3), (1000, 400, 100), (1 << 20, 300000, 50000), (200001, 5000, 3000), (150000, 60, 40)):
+        if n == 200001:    # 40-bit suffixes in two far-apart clusters: most buckets of the join's directory are empty
+            suf = np.unique(np.concatenate([rng.integers(0, 1 << 20, n // 2), (1 << 40) - 1 - rng.integers(0, 1 << 22, n // 2)])
+                            .astype(np.uint64))
+            n = suf.size
+        elif n == 150000:  # few messages: the handle of the sorted variant has room for a small directory only
+            suf = np.sort(rng.choice(1 << 36, n, replace=False)).astype(np.uint64)
+        else:
+            suf = np.sort(rng.choice(1 << 30, n, replace=False)).astype(np.uint64)
         sa = suf | (rng.integers(0, 1 << 16, n).astype(np.uint64) << np.uint64(48))
         primary = rng.integers(0, 1 << 31, n).astype(np.uint32)
         tgt = np.concatenate([suf[rng.choice(n, hits, replace=False)],
-                              np.setdiff1d(rng.integers(0, 1 << 30, misses).astype(np.uint64), suf)])
+                              np.setdiff1d(rng.integers(0, int(suf[-1]) + 1000, misses).astype(np.uint64), suf)])
         rank = rng.integers(0, 1 << 32, tgt.size, dtype=np.uint64).astype(np.uint32)
         order = rng.permutation(tgt.size)
         tgt, rank = tgt[order], rank[order]
