@@ -28,6 +28,51 @@ def _run_heads(*cols):
     return np.maximum.accumulate(idx), head
 
 
+def validate_messages(m_tgt, m_rank, end, q, pid, psz, n, ctx):
+    """The reference's check of a partition's outbox (gpu_saca::test::validate_messages, test/rank-propagation.cpp:23-107):
+    every message's sender lies in partition q (directly, one context after the target, or as the forwarder of a pill,
+    half a context after it); every message sits in the group of its target's partition; every rank is below the
+    partition's size (a forwarded pill carries another partition's rank: below the largest partition's size)."""
+    total = m_tgt.size
+    if total == 0:
+        return
+    pill = (m_rank >> np.uint32(31)) != 0
+    rank = (m_rank & np.uint32(0x7FFFFFFF)).astype(np.uint64)
+    direct, forwarder = m_tgt + np.uint64(ctx), m_tgt + np.uint64(ctx // 2)
+    assert not ((direct >= n) & (forwarder >= n)).any(), "a message has no sender inside the text"
+    assert not ((direct >= n) & (forwarder < n) & ~pill).any(), "only a pill can come from half a context away"
+    pid_direct = pid[np.minimum(direct, np.uint64(n - 1)).astype(np.int64)]
+    pid_forwarder = pid[np.minimum(forwarder, np.uint64(n - 1)).astype(np.int64)]
+    in_place = ((direct < n) & (pid_direct == q)) | (pill & (forwarder < n) & (pid_forwarder == q))
+    assert in_place.all(), "a message's sender does not belong to the partition that produced it"
+    dest = pid[m_tgt.astype(np.int64)].astype(np.int64)
+    ends = end.astype(np.int64)
+    beg = np.where(dest > 0, ends[np.maximum(dest - 1, 0)], 0)
+    slot = np.arange(total, dtype=np.int64)
+    assert ((beg <= slot) & (slot < ends[dest])).all(), "a message lies outside the group of its destination partition"
+    bound = np.where(pill, np.uint64(psz.max()), np.uint64(psz[q]))
+    assert (rank < bound).all(), "a message carries a rank beyond its sender's partition"
+
+
+def validate_inbox_routing(tgt, t, pid, n):
+    """gpu_saca::test::validate_inbox_routing (test/rank-propagation.cpp:176-188): every message delivered to partition t
+    is addressed to a suffix of partition t."""
+    assert (tgt < n).all() and (pid[tgt.astype(np.int64)] == t).all(), f"partition {t} received a message for another partition"
+
+
+def validate_coherent_targets(suf, rank, pid, n, stride, ell):
+    """gpu_saca::test::validate_coherent_targets as stage_slab applies it to neighbouring cohort entries
+    (test/rank-propagation.cpp:14-19, src/GPU_SACA.cu:1621-1633): suffixes tied after the generation before draw their
+    secondaries of this generation from the same partition (equal forward tags, include/bit-layout.hpp:99-100)."""
+    if suf.size < 2:
+        return
+    src = suf + np.uint64(stride)
+    tag = np.where(src < n, pid[np.minimum(src, np.uint64(n - 1)).astype(np.int64)].astype(np.uint64) + np.uint64(ell),
+                   np.uint64(n + ell - 1) - src)
+    tied = rank[1:] == rank[:-1]
+    assert (tag[1:][tied] == tag[:-1][tied]).all(), "target coherence invariant broken"
+
+
 def build_sa(lib, to_dev, to_host, T, p, key_words=1, pivot_words=2, seed=0, max_generations=64, log=None, join_handle=None,
              step_handle=None):
     """Returns (sa uint64[n], generations run). `to_dev(np array)` gives an object with .ptr; `to_host(obj)` the array back.
@@ -72,6 +117,10 @@ def build_sa(lib, to_dev, to_host, T, p, key_words=1, pivot_words=2, seed=0, max
             if a == 0:
                 continue
             suf, prim = pt["suf"][:a].copy(), pt["rank"][:a].copy()
+            if gen > 0:  # the reference's checks of a cohort at staging time (src/GPU_SACA.cu:1621-1640, :1475)
+                validate_coherent_targets(suf, prim, pid, n, ctx // 2, ell)
+                assert not oracle_lib.retired(words, bits, suf).any(), "a retired suffix is in the cohort"
+                validate_inbox_routing(inbox[q][0], q, pid, n)
             # ---- staging (src/GPU_SACA.cu:1611-1692): keys at generation 0, routing tags always ----
             d_keys = to_dev(np.zeros(a * key_words, dtype=np.uint64))
             d_beta = to_dev(np.zeros(a, dtype=np.uint32))
@@ -103,6 +152,7 @@ def build_sa(lib, to_dev, to_host, T, p, key_words=1, pivot_words=2, seed=0, max
                 end = to_host(d_off)
                 assert total == int(end[p - 1])
                 m_tgt, m_rank = oracle_lib.sa40_to_u64(to_host(d_mt))[:total], to_host(d_mr)[:total]
+                validate_messages(m_tgt, m_rank, end, q, pid, psz, n, ctx)
                 start = 0
                 for dest in range(p):
                     e = int(end[dest])
@@ -171,6 +221,7 @@ def build_sa(lib, to_dev, to_host, T, p, key_words=1, pivot_words=2, seed=0, max
                                              None) == 0
             end = to_host(d_off)
             m_tgt, m_rank = oracle_lib.sa40_to_u64(to_host(d_mt))[:total], to_host(d_mr)[:total]
+            validate_messages(m_tgt, m_rank, end, q, pid, psz, n, ctx)
             start = 0
             for dest in range(p):  # the host splits the outbox by the end offsets (src/Partition_Backend.cpp:516-554)
                 e = int(end[dest])

@@ -282,9 +282,14 @@ def stage_slab(T, suf, key_words, pid, retired, ctx, generation0):
 
 def set_retired(words, bits, positions):
     """Marks text positions retired in a packed map: the top bit of their entries (include/Partition_ID_Map.hpp:55,198-202)."""
-    for x in positions:
-        bit = int(x) * bits + bits - 1
-        words[bit // 64] |= np.uint64(1) << np.uint64(bit % 64)
+    bit = np.asarray(positions, dtype=np.uint64) * np.uint64(bits) + np.uint64(bits - 1)
+    np.bitwise_or.at(words, (bit // np.uint64(64)).astype(np.int64), np.uint64(1) << (bit % np.uint64(64)))
+
+
+def retired(words, bits, positions):
+    """The retirement flags of text positions in a packed map (Partition_ID_Map::retired, include/Partition_ID_Map.hpp:180)."""
+    bit = np.asarray(positions, dtype=np.uint64) * np.uint64(bits) + np.uint64(bits - 1)
+    return ((words[(bit // np.uint64(64)).astype(np.int64)] >> (bit % np.uint64(64))) & np.uint64(1)).astype(bool)
 
 
 def count_messages(sa, keys, beta, ctx, packed, p):
