@@ -150,6 +150,13 @@ __device__ __forceinline__ u32 lb2_wait_exclusive(u64* tile_chain, u64* group_ch
 #pragma unroll
     for (u32 k = 1; k < LB_GROUP; ++k)
         word[k - 1] = k <= j ? lb_load(tile_chain + (u64)(tile - k) * stride) : 0ull;
+    // the words of the two groups before this one travel together with the tile words: the walk over the groups below
+    // then starts from words that are already here, instead of paying a round trip of its own for each
+    constexpr u32 PROBES = 2;
+    u64 probe[PROBES];
+#pragma unroll
+    for (u32 k = 0; k < PROBES; ++k)
+        probe[k] = g > k ? lb_load(group_chain + (u64)(g - 1 - k) * stride) : 0ull;
     u32 within = 0;
 #pragma unroll
     for (u32 k = 1; k < LB_GROUP; ++k) {
@@ -168,7 +175,9 @@ __device__ __forceinline__ u32 lb2_wait_exclusive(u64* tile_chain, u64* group_ch
     u32 gexcl = 0;
     for (u32 gi = g; gi > 0;) {
         --gi;
-        const u64 w = lb_wait_word(group_chain + (u64)gi * stride, epoch, err);
+        u64 w = g - 1 - gi < PROBES ? probe[g - 1 - gi] : 0ull;
+        if ((u32)(w >> 34) != epoch || ((w >> 32) & 3u) == 0)
+            w = lb_wait_word(group_chain + (u64)gi * stride, epoch, err);
         gexcl += (u32)w;
         if (((w >> 32) & 3u) == LB_INCL || w == 0)
             break;

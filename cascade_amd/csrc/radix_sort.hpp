@@ -402,6 +402,16 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
     }
     __syncthreads();
 
+    // the values are asked for now: their way from HBM overlaps the writes of the keys below (asked for before the
+    // look-back they would delay its words, which come back in the order of issue)
+    u32 val[ITEMS];
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const u32 local = first_local + k * WAVE;
+        val[k] = 0;
+        if (local < valid)
+            val[k] = SRC == SRC_TEXT ? virtual_to_suffix((u32)(base + local), a.text_n, a.tail) : a.vals_in[base + local];
+    }
     // ---- write runs of equal digits to their global places ----
     u32 dst[ITEMS];
 #pragma unroll
@@ -415,14 +425,6 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
     }
     __syncthreads();
     u32* s_vals = reinterpret_cast<u32*>(s_keys);
-    u32 val[ITEMS];
-#pragma unroll
-    for (int k = 0; k < ITEMS; ++k) {
-        const u32 local = first_local + k * WAVE;
-        val[k] = 0;
-        if (local < valid)
-            val[k] = SRC == SRC_TEXT ? virtual_to_suffix((u32)(base + local), a.text_n, a.tail) : a.vals_in[base + local];
-    }
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k)
         s_vals[pos[k]] = val[k];
