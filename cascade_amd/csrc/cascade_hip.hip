@@ -52,6 +52,19 @@ constexpr int SORT_ITEMS = CSA_SORT_ITEMS;
 constexpr int SORT32_ITEMS = CSA_SORT32_ITEMS; // pairs per thread when the keys are 32-bit (same LDS bytes at twice the items)
 constexpr int SORT_TILE = SORT_BLOCK * SORT_ITEMS;
 static_assert(SORT32_ITEMS >= SORT_ITEMS, "the look-back words are sized for tiles of SORT_TILE pairs or more");
+// Under arrival order (the default, where neighbouring tiles run on different XCDs) long passes use workgroups of twice the
+// threads: the runs of a digit a tile writes are twice as long, so fewer of the lines it writes are shared with a tile
+// whose L2 is another one. One such workgroup fills a CU's LDS; measured 125.3 -> 121.4 ms per sort of the 1B-token
+// workload. The chunked order keeps the smaller workgroup (two per CU), which is faster there (119.5 against 121.6 ms).
+#ifndef CSA_SORT_WIDE_BLOCK
+#define CSA_SORT_WIDE_BLOCK 1024
+#endif
+#ifndef CSA_SORT_WIDE_MIN
+#define CSA_SORT_WIDE_MIN (1u << 24)
+#endif
+constexpr int SORT_WIDE_BLOCK = CSA_SORT_WIDE_BLOCK;
+constexpr u32 SORT_WIDE_MIN = CSA_SORT_WIDE_MIN; // fewest pairs of a pass that uses the wide workgroups
+static_assert(SORT_WIDE_BLOCK >= SORT_BLOCK, "the look-back words are sized for tiles of SORT_TILE pairs or more");
 #ifndef CSA_RANK_BLOCK
 #define CSA_RANK_BLOCK 256
 #endif
@@ -206,20 +219,39 @@ void set_tile_order(const csa_handle* h, OnesweepArgs& a, u32 tile)
     a.xcd_chunk = h->xcd_chunk ? h->xcd_chunk : 1u;
 }
 
+bool wide_workgroups(const csa_handle* h, const OnesweepArgs& a)
+{
+    return h->tile_order == TILES_BY_ARRIVAL && SORT_WIDE_BLOCK > SORT_BLOCK && a.n >= SORT_WIDE_MIN;
+}
+
+template <int SRC, int BLOCK>
+void launch_onesweep_shape(const csa_handle* h, OnesweepArgs& a, hipStream_t s)
+{
+    set_tile_order(h, a, BLOCK * SORT_ITEMS);
+    if (a.shift >= 32)
+        hipLaunchKernelGGL((onesweep_kernel<u64, BLOCK, SORT_ITEMS, SRC, 1>), dim3(a.tiles), dim3(BLOCK), 0, s, a);
+    else
+        hipLaunchKernelGGL((onesweep_kernel<u64, BLOCK, SORT_ITEMS, SRC, 0>), dim3(a.tiles), dim3(BLOCK), 0, s, a);
+}
+
 template <int SRC>
 void launch_onesweep(const csa_handle* h, OnesweepArgs& a, hipStream_t s)
 {
-    set_tile_order(h, a, SORT_TILE);
-    if (a.shift >= 32)
-        hipLaunchKernelGGL((onesweep_kernel<u64, SORT_BLOCK, SORT_ITEMS, SRC, 1>), dim3(a.tiles), dim3(SORT_BLOCK), 0, s, a);
+    if (wide_workgroups(h, a))
+        launch_onesweep_shape<SRC, SORT_WIDE_BLOCK>(h, a, s);
     else
-        hipLaunchKernelGGL((onesweep_kernel<u64, SORT_BLOCK, SORT_ITEMS, SRC, 0>), dim3(a.tiles), dim3(SORT_BLOCK), 0, s, a);
+        launch_onesweep_shape<SRC, SORT_BLOCK>(h, a, s);
 }
 
 void launch_onesweep32(const csa_handle* h, OnesweepArgs& a, hipStream_t s)
 {
-    set_tile_order(h, a, SORT_BLOCK * SORT32_ITEMS);
-    hipLaunchKernelGGL((onesweep_kernel<u32, SORT_BLOCK, SORT32_ITEMS, SRC_PAIRS, 0>), dim3(a.tiles), dim3(SORT_BLOCK), 0, s, a);
+    if (wide_workgroups(h, a)) {
+        set_tile_order(h, a, SORT_WIDE_BLOCK * SORT32_ITEMS);
+        hipLaunchKernelGGL((onesweep_kernel<u32, SORT_WIDE_BLOCK, SORT32_ITEMS, SRC_PAIRS, 0>), dim3(a.tiles), dim3(SORT_WIDE_BLOCK), 0, s, a);
+    } else {
+        set_tile_order(h, a, SORT_BLOCK * SORT32_ITEMS);
+        hipLaunchKernelGGL((onesweep_kernel<u32, SORT_BLOCK, SORT32_ITEMS, SRC_PAIRS, 0>), dim3(a.tiles), dim3(SORT_BLOCK), 0, s, a);
+    }
 }
 
 // Sorts n pairs by the digits of `plan`. The first pass that runs takes its input as `src` says
