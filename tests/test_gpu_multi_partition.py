@@ -89,3 +89,30 @@ def test_step_entries_on_hard_shapes(gpu, shape, p):
     assert np.array_equal(sa, want), (shape, gens)
     if shape == "one_symbol":
         assert np.array_equal(sa, np.arange(n - 1, -1, -1, dtype=np.uint64))
+
+
+def test_random_pipelines_through_the_step_entries(gpu):
+    """Random texts (tiny alphabets, long repeats, zero tails), 1 to 200 partitions, all four key widths: every step
+    passes the reference's validators inside the harness and the suffix array is the oracle's."""
+    lib, to_dev, to_host = gpu
+    rng = np.random.default_rng(99)
+    for case in range(40):
+        n = int(rng.integers(50, 30000))
+        sigma = int(rng.choice([1, 2, 3, 5, 40, 65536]))
+        T = rng.integers(0, sigma, n).astype(np.uint16)
+        if case % 3 == 1 and n > 200:
+            length = int(rng.integers(10, n // 2))
+            T[n - length:] = T[:length]
+        if case % 3 == 2:
+            T[-int(rng.integers(1, 30)):] = 0
+        p = int(rng.choice([1, 2, 3, 7, 16, 50, 200]))
+        key_words = 1 + case % 4
+        h = C.c_void_p()
+        assert lib.csa_create(n, 1, C.byref(h)) == 0
+        try:
+            print(f"  random pipeline case={case} n={n} sigma={sigma} p={p} key_words={key_words}", flush=True)
+            sa, _ = multi_partition.build_sa(lib, to_dev, to_host, T, p, key_words=key_words, seed=case, step_handle=h)
+        finally:
+            lib.csa_destroy(h)
+        want, _ = oracle_lib.prefix_doubling(T, 1)
+        assert np.array_equal(sa, want), (case, n, sigma, p, key_words)
