@@ -638,7 +638,15 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     hipStream_t s = L.stream;
     csa_stats* st = L.stats;
     const u32 n = (u32)n64;
-    const u32 ell = 4u * (u32)h->key_words;
+    // Keys of 2 and 4 words are not sorted word by word: a generation that resolves 8 or 16 symbols is what one or two
+    // doubling generations on one-word keys resolve (4 -> 8 -> 16 symbols; the order of suffixes that run off the text is
+    // the same: the shorter first), so the sort runs on one-word keys and reports those generations as its generation 0.
+    // Every later generation then has the context, the ranks and the active set of the wide-key generation it stands
+    // for. A 4-word key sorted word by word costs 32 radix passes over all suffixes (316 ms on the 1B-token workload);
+    // this way it costs what the one-word key costs. Three words (12 symbols) are no power of two times 4: word by word.
+    const int folded = h->key_words == 2 ? 1 : (h->key_words == 4 ? 2 : 0);
+    const int sort_words = folded ? 1 : h->key_words;
+    const u32 ell = 4u * (u32)sort_words;
     const u32 tail = n < ell ? n : ell;
 
     HIP_TRY(hipMemsetAsync(h->counts, 0, 4 * sizeof(u32), s));
@@ -655,8 +663,8 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     // straight from the text, every following (stable) sort rebuilds its word from the text through the suffix
     // indices the sort before it left.
     cur = 0;
-    for (int word = h->key_words - 1; word >= 0; --word) {
-        const bool first_sort = word == h->key_words - 1;
+    for (int word = sort_words - 1; word >= 0; --word) {
+        const bool first_sort = word == sort_words - 1;
         rc = radix_sort(L, first_sort ? SRC_TEXT : SRC_TEXT_IDX, d_text, n, tail, (u32)word, K[cur], V[cur], K[cur ^ 1], V[cur ^ 1],
                         n, full, &in_out, &p1);
         if (rc)
@@ -680,7 +688,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     ra.keys = k_sorted;
     ra.sufs = sa32;
     ra.m = n;
-    ra.key_words = h->key_words;
+    ra.key_words = sort_words;
     ra.n = n;
     ra.ell = ell;
     ra.text = d_text;
@@ -846,6 +854,29 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
         st->radix_ms += ms;
         st->radix_pairs += tl.second;
         st->radix_launches++;
+    }
+    // wide keys: the first generations that ran stand for generation 0
+    const int merged = folded < gen - 1 ? folded : gen - 1;
+    if (merged > 0) {
+        for (int g = 1; g <= merged; ++g) {
+            st->ms[0] += st->ms[g];
+            st->passes[0] += st->passes[g];
+        }
+        for (int g = 1; g + merged < gen; ++g) {
+            st->active[g] = st->active[g + merged];
+            st->groups[g] = st->groups[g + merged];
+            st->big[g] = st->big[g + merged];
+            st->passes[g] = st->passes[g + merged];
+            st->rank_update[g] = st->rank_update[g + merged];
+            st->small_only[g] = st->small_only[g + merged];
+            st->ms[g] = st->ms[g + merged];
+        }
+        for (int g = gen - merged; g < gen; ++g) {
+            st->active[g] = st->groups[g] = st->big[g] = 0;
+            st->passes[g] = st->rank_update[g] = st->small_only[g] = 0;
+            st->ms[g] = 0.0f;
+        }
+        st->generations = gen - merged;
     }
     return CSA_OK;
 }

@@ -69,10 +69,12 @@ def test_fixtures_through_the_emulated_kernels(emu, key_words):
         assert active == counts, name
 
 
-@pytest.mark.parametrize("key_words", [4])
-def test_keys_of_four_words(emu, key_words):
-    # the reference's default key is 4 words (16 symbols): generation 0 sorts word by word and compares the later words
-    # through the text; texts shorter than a key, and runs that tie over a whole key, are the edge cases
+@pytest.mark.parametrize("key_words", [3, 4])
+def test_keys_of_three_and_four_words(emu, key_words):
+    # three words are sorted word by word, the later words compared through the text; four words (the reference's
+    # default, 16 symbols) run as one-word keys whose first two doubling generations stand for generation 0. Either way
+    # the generation sizes must be the oracle's for that key width; texts shorter than a key, and runs that tie over a
+    # whole key, are the edge cases
     suite = dict(texts.fixture_suite())
     for name, T in [(n_, suite[n_]) for n_ in ("rand_n17_s2", "rand_n1000_s2", "hand_15")] + [
             ("run", np.concatenate([np.full(40, 3, dtype=np.uint16), texts.random_text(300, 2, 9, sep_every=0)])),
