@@ -338,10 +338,8 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
         const int use_src = first ? src : SRC_PAIRS;
         if (use_src == SRC_PAIRS)
             launch_onesweep<SRC_PAIRS>(h, a, s);
-        else if (use_src == SRC_TEXT)
-            launch_onesweep<SRC_TEXT>(h, a, s);
         else
-            launch_onesweep<SRC_TEXT_IDX>(h, a, s);
+            launch_onesweep<SRC_TEXT>(h, a, s);
         if (timed) {
             HIP_TRY(hipEventRecord(h->events[L.events_used + 1], s));
             L.timed.push_back({L.events_used, (u64)n});
@@ -638,15 +636,18 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     hipStream_t s = L.stream;
     csa_stats* st = L.stats;
     const u32 n = (u32)n64;
-    // Keys of 2 and 4 words are not sorted word by word: a generation that resolves 8 or 16 symbols is what one or two
-    // doubling generations on one-word keys resolve (4 -> 8 -> 16 symbols; the order of suffixes that run off the text is
-    // the same: the shorter first), so the sort runs on one-word keys and reports those generations as its generation 0.
-    // Every later generation then has the context, the ranks and the active set of the wide-key generation it stands
-    // for. A 4-word key sorted word by word costs 32 radix passes over all suffixes (316 ms on the 1B-token workload);
-    // this way it costs what the one-word key costs. Three words (12 symbols) are no power of two times 4: word by word.
-    const int folded = h->key_words == 2 ? 1 : (h->key_words == 4 ? 2 : 0);
-    const int sort_words = folded ? 1 : h->key_words;
-    const u32 ell = 4u * (u32)sort_words;
+    // Wide keys are not sorted word by word. A generation 0 that resolves 4 W symbols is what doubling on one-word keys
+    // reaches after one or two more generations (4 -> 8 -> 16 symbols; 4 -> 8 -> 12 with the second step looking only 4
+    // symbols ahead; the order of suffixes that run off the text is the same: the shorter first). So the sort always
+    // starts from one-word keys, steps up to the context of the wide key, reports those generations as its generation 0
+    // and doubles from there. Every reported generation then has the context, the ranks and the active set of the wide-key
+    // generation it stands for. A 4-word key sorted word by word costs 32 radix passes over all suffixes (316 ms on the
+    // 1B-token workload); this way it costs what the one-word key costs.
+    const u32 ell = 4u;
+    const u64 wide_ell = 4ull * (u64)h->key_words;
+    int folded = 0; // generations after the first that still belong to the reported generation 0
+    for (u64 c = ell; c < wide_ell; c += (c < wide_ell - c ? c : wide_ell - c))
+        ++folded;
     const u32 tail = n < ell ? n : ell;
 
     HIP_TRY(hipMemsetAsync(h->counts, 0, 4 * sizeof(u32), s));
@@ -659,20 +660,13 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     u32* V[2] = {h->idx[0], h->idx[1]};
     int cur; // the (K, V) set that holds the sorted pairs
     int rc;
-    // A key of W words is sorted word by word, the least significant word first: the first sort builds its keys
-    // straight from the text, every following (stable) sort rebuilds its word from the text through the suffix
-    // indices the sort before it left.
     cur = 0;
-    for (int word = sort_words - 1; word >= 0; --word) {
-        const bool first_sort = word == sort_words - 1;
-        rc = radix_sort(L, first_sort ? SRC_TEXT : SRC_TEXT_IDX, d_text, n, tail, (u32)word, K[cur], V[cur], K[cur ^ 1], V[cur ^ 1],
-                        n, full, &in_out, &p1);
-        if (rc)
-            return rc;
-        passes += p1;
-        if (in_out)
-            cur ^= 1;
-    }
+    rc = radix_sort(L, SRC_TEXT, d_text, n, tail, 0, K[0], V[0], K[1], V[1], n, full, &in_out, &p1);
+    if (rc)
+        return rc;
+    passes += p1;
+    if (in_out)
+        cur = 1;
     u64* k_sorted = K[cur];
     u32* sa32 = V[cur]; // from here on the suffix array under construction
     // roles of the remaining arrays in generations t >= 1
@@ -688,7 +682,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     ra.keys = k_sorted;
     ra.sufs = sa32;
     ra.m = n;
-    ra.key_words = sort_words;
+    ra.key_words = 1;
     ra.n = n;
     ra.ell = ell;
     ra.text = d_text;
@@ -714,7 +708,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     int gp = 0; // gprim[gp] / gstart[gp] describe the current groups
     bool all_small = false; // no group of the current list exceeds SMALL_MAXG members
     const int sec_bits = bit_length(n > 1 ? n - 1 : 1);
-    u64 h_ctx = ell;
+    u64 ctx = ell; // symbols resolved so far; the next generation looks hop symbols ahead
     while (m > 0) {
         if (gen >= CSA_MAX_GENERATIONS)
             return fail(CSA_ERR_INTERNAL, "generation cap reached with %u suffixes still active", m);
@@ -733,7 +727,8 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
         sa.rank = h->rank;
         sa.m = m_in;
         sa.n = n;
-        sa.h = (u32)h_ctx;
+        const u64 hop = ctx < wide_ell ? (ctx < wide_ell - ctx ? ctx : wide_ell - ctx) : ctx;
+        sa.h = (u32)hop;
         sa.sec_bits = sec_bits;
         sa.groups = groups;
         sa.err = h->counts + 2;
@@ -829,7 +824,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
         st->passes[gen] = passes;
         HIP_TRY(hipEventRecord(h->ev_gen[gen + 1], s));
         gen++;
-        h_ctx *= 2;
+        ctx += hop;
     }
     st->generations = gen;
 

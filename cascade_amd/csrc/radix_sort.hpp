@@ -26,8 +26,7 @@ struct PassPlan {
 // How a pass obtains its input pairs.
 enum : int {
     SRC_PAIRS = 0, // keys_in[i], vals_in[i]
-    SRC_TEXT = 1,  // generation 0, first pass: the pair of virtual position i is built from the text
-    SRC_TEXT_IDX = 2 // key word `word` of suffix vals_in[i], rebuilt from the text (128-bit keys, second phase)
+    SRC_TEXT = 1   // generation 0, first pass: the pair of virtual position i is built from the text
 };
 
 // Generation 0 feeds the suffixes in the order (n-1, n-2, ..., n-tail, 0, 1, ..., n-tail-1): the last
@@ -171,9 +170,9 @@ struct OnesweepArgs {
     u32* vals_out;
     const u16* text;
     u32 n;      // pairs
-    u32 text_n; // symbols in the text (SRC_TEXT*)
+    u32 text_n; // symbols in the text (SRC_TEXT)
     u32 tail;   // suffixes that run off the text inside their key (SRC_TEXT)
-    u32 word;   // key word to build (SRC_TEXT*)
+    u32 word;   // key word to build (SRC_TEXT)
     int shift;
     int bits;
     const u32* digit_base; // [256] for this pass
@@ -303,13 +302,10 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) {
             const u64 i = base + first_local + k * WAVE;
-            if (SRC == SRC_PAIRS) {
+            if (SRC == SRC_PAIRS)
                 key[k] = keys_in[i];
-            } else if (SRC == SRC_TEXT) {
+            else
                 key[k] = (KeyT)text_key((u32)i);
-            } else {
-                key[k] = (KeyT)load_kgram(a.text, a.text_n, a.vals_in[i], a.word);
-            }
         }
     } else {
 #pragma unroll
@@ -320,10 +316,8 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
             if (local < valid) {
                 if (SRC == SRC_PAIRS)
                     key[k] = keys_in[i];
-                else if (SRC == SRC_TEXT)
-                    key[k] = (KeyT)text_key((u32)i);
                 else
-                    key[k] = (KeyT)load_kgram(a.text, a.text_n, a.vals_in[i], a.word);
+                    key[k] = (KeyT)text_key((u32)i);
             }
         }
     }

@@ -75,8 +75,8 @@ uint64_t csa_bytes_per_suffix(int key_words);
 /* Allocates the scratch for partitions of up to max_part_sz suffixes on the current device.
  * key_words: 64-bit words of the generation-0 key, 1 to 4 (4 to 16 uint16 symbols; the reference's
  * PREF_KEY_WORDS, include/Packed_Prefix.hpp:20-24, whose default is 4). The suffix array does not depend on it,
- * only the number of generations and their sizes do; 1, 2 and 4 words cost the same time (wide keys are resolved by
- * doubling on one-word keys and reported as generation 0), 3 words are sorted word by word.
+ * only the number of generations and their sizes do; every width costs the same time (wide keys are resolved by
+ * doubling steps on one-word keys, which are reported as generation 0).
  * Replaces GPU_SACA::allocate_device_space (src/GPU_SACA.cu:535-590). */
 int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out);
 

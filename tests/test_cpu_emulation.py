@@ -71,10 +71,10 @@ def test_fixtures_through_the_emulated_kernels(emu, key_words):
 
 @pytest.mark.parametrize("key_words", [3, 4])
 def test_keys_of_three_and_four_words(emu, key_words):
-    # three words are sorted word by word, the later words compared through the text; four words (the reference's
-    # default, 16 symbols) run as one-word keys whose first two doubling generations stand for generation 0. Either way
-    # the generation sizes must be the oracle's for that key width; texts shorter than a key, and runs that tie over a
-    # whole key, are the edge cases
+    # wide keys (four words, 16 symbols, are the reference's default) run as one-word keys whose first generations stand
+    # for generation 0: 4 -> 8 -> 16 symbols, or 4 -> 8 -> 12 with a second step that looks only 4 symbols ahead. The
+    # generation sizes must be the oracle's for that key width; texts shorter than a key, and runs that tie over a whole
+    # key, are the edge cases
     suite = dict(texts.fixture_suite())
     for name, T in [(n_, suite[n_]) for n_ in ("rand_n17_s2", "rand_n1000_s2", "hand_15")] + [
             ("run", np.concatenate([np.full(40, 3, dtype=np.uint16), texts.random_text(300, 2, 9, sep_every=0)])),
