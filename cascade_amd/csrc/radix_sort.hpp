@@ -271,8 +271,10 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
 #define CSA_DIGIT(kk) __builtin_amdgcn_ubfe(HI ? (u32)((u64)(kk) >> 32) : (u32)(kk), sh, bits)
 #ifdef __HIP_DEVICE_COMPILE__
 #define CSA_LDS_ORDER() asm volatile("" ::: "memory")
+#define CSA_OPAQUE(x) asm volatile("" : "+v"(x))
 #else
 #define CSA_LDS_ORDER() __builtin_amdgcn_wave_barrier() /* CPU emulation: lanes are threads, order them for real */
+#define CSA_OPAQUE(x) ((void)0)
 #endif
     // ---- first pass of generation 0: stage the tile's stretch of the text in LDS ----
     // The tile covers consecutive virtual positions, i.e. (after the few tail suffixes of tile 0) consecutive text
@@ -324,7 +326,7 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
 
     // ---- rank each pair among the pairs of its wave that share its digit ----
     // For every digit bit, (ballot of "bit set") XOR (all-ones if my own bit is set) has a 0 exactly at the lanes
-    // that agree with me on that bit; OR-ed over the bits, `differ` marks the lanes whose digit is not mine.
+    // that agree with me on that bit; `same` keeps the lanes that agree on every bit, i.e. whose digit is mine.
     // The per-wave counters are plain LDS words: a wave executes its LDS instructions in order, so the counter
     // update of one item is seen by the next item's read; the empty asm statements only keep the compiler from
     // moving those accesses across each other.
@@ -333,15 +335,16 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         const u32 d = CSA_DIGIT(key[k]);
-        u32 differ_lo = 0, differ_hi = 0;
+        u32 same_lo = ~0u, same_hi = ~0u;
 #pragma unroll
         for (int b = 0; b < RADIX_BITS; ++b) {
-            const u32 mine = (u32)__builtin_amdgcn_sbfe(d, b, 1); // 0 or 0xFFFFFFFF
-            const u64 bal = __ballot(mine != 0);
-            differ_lo |= (u32)bal ^ mine;
-            differ_hi |= (u32)(bal >> 32) ^ mine;
+            u32 mine = (u32)__builtin_amdgcn_sbfe(d, b, 1); // 0 or 0xFFFFFFFF
+            CSA_OPAQUE(mine); // the ballot tests this register (one compare), not a second extraction of the bit
+            const u64 bal = __ballot((int)mine < 0);
+            // same &= ~(bal ^ mine): one three-input bit operation per half (table of a & ~(b ^ c): 0x90)
+            same_lo = __builtin_amdgcn_bitop3_b32(same_lo, (u32)bal, mine, 0x90);
+            same_hi = __builtin_amdgcn_bitop3_b32(same_hi, (u32)(bal >> 32), mine, 0x90);
         }
-        const u32 same_lo = ~differ_lo, same_hi = ~differ_hi;
         const u32 before = __builtin_amdgcn_mbcnt_hi(same_hi, __builtin_amdgcn_mbcnt_lo(same_lo, 0u));
         const u32 prev = whist[d];
         CSA_LDS_ORDER();
@@ -431,6 +434,7 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
     }
 #undef CSA_DIGIT
 #undef CSA_LDS_ORDER
+#undef CSA_OPAQUE
 }
 
 } // namespace csa

@@ -171,6 +171,17 @@ inline int __builtin_amdgcn_sbfe(unsigned src, unsigned off, unsigned width)
     return (int)((v ^ sign) - sign);
 }
 
+// three-input bit operation: bit i of the result is bit ((a_i << 2) | (b_i << 1) | c_i) of the table
+inline unsigned __builtin_amdgcn_bitop3_b32(unsigned a, unsigned b, unsigned c, unsigned table)
+{
+    unsigned r = 0;
+    for (int i = 0; i < 32; ++i) {
+        const unsigned sel = (((a >> i) & 1u) << 2) | (((b >> i) & 1u) << 1) | ((c >> i) & 1u);
+        r |= ((table >> sel) & 1u) << i;
+    }
+    return r;
+}
+
 inline unsigned __builtin_amdgcn_mbcnt_lo(unsigned mask, unsigned add)
 {
     const unsigned l = hipemu::lane;
