@@ -52,10 +52,11 @@ constexpr int SORT_ITEMS = CSA_SORT_ITEMS;
 constexpr int SORT32_ITEMS = CSA_SORT32_ITEMS; // pairs per thread when the keys are 32-bit (same LDS bytes at twice the items)
 constexpr int SORT_TILE = SORT_BLOCK * SORT_ITEMS;
 static_assert(SORT32_ITEMS >= SORT_ITEMS, "the look-back words are sized for tiles of SORT_TILE pairs or more");
-// Under arrival order (the default, where neighbouring tiles run on different XCDs) long passes use workgroups of twice the
-// threads: the runs of a digit a tile writes are twice as long, so fewer of the lines it writes are shared with a tile
-// whose L2 is another one. One such workgroup fills a CU's LDS; measured 125.3 -> 121.4 ms per sort of the 1B-token
-// workload. The chunked order keeps the smaller workgroup (two per CU), which is faster there (119.5 against 121.6 ms).
+// Long passes use workgroups of twice the threads: the runs of a digit a tile writes are twice as long, so fewer of the
+// lines it writes are shared with a tile whose L2 is another one. One such workgroup fills a CU's LDS. Measured per
+// sort of the 1B-token workload: 125.3 -> 121.4 ms by arrival (the default order, where neighbouring tiles run on
+// different XCDs), 119.3 -> 117.4 ms under the chunked order, whose chunks keep their length in pairs (half as many
+// of the larger tiles: with the full count the wide workgroups gained nothing there).
 #ifndef CSA_SORT_WIDE_BLOCK
 #define CSA_SORT_WIDE_BLOCK 1024
 #endif
@@ -216,12 +217,14 @@ void set_tile_order(const csa_handle* h, OnesweepArgs& a, u32 tile)
 {
     a.tiles = (u32)(((u64)a.n + tile - 1) / tile);
     a.order = h->tile_order;
-    a.xcd_chunk = h->xcd_chunk ? h->xcd_chunk : 1u;
+    // the chunk length is meant in tiles of SORT_TILE pairs: larger tiles, proportionally fewer per chunk
+    const u32 chunk = (u32)((u64)h->xcd_chunk * SORT_TILE / tile);
+    a.xcd_chunk = chunk ? chunk : 1u;
 }
 
-bool wide_workgroups(const csa_handle* h, const OnesweepArgs& a)
+bool wide_workgroups(const OnesweepArgs& a)
 {
-    return h->tile_order == TILES_BY_ARRIVAL && SORT_WIDE_BLOCK > SORT_BLOCK && a.n >= SORT_WIDE_MIN;
+    return SORT_WIDE_BLOCK > SORT_BLOCK && a.n >= SORT_WIDE_MIN;
 }
 
 template <int SRC, int BLOCK>
@@ -237,7 +240,7 @@ void launch_onesweep_shape(const csa_handle* h, OnesweepArgs& a, hipStream_t s)
 template <int SRC>
 void launch_onesweep(const csa_handle* h, OnesweepArgs& a, hipStream_t s)
 {
-    if (wide_workgroups(h, a))
+    if (wide_workgroups(a))
         launch_onesweep_shape<SRC, SORT_WIDE_BLOCK>(h, a, s);
     else
         launch_onesweep_shape<SRC, SORT_BLOCK>(h, a, s);
@@ -245,7 +248,7 @@ void launch_onesweep(const csa_handle* h, OnesweepArgs& a, hipStream_t s)
 
 void launch_onesweep32(const csa_handle* h, OnesweepArgs& a, hipStream_t s)
 {
-    if (wide_workgroups(h, a)) {
+    if (wide_workgroups(a)) {
         set_tile_order(h, a, SORT_WIDE_BLOCK * SORT32_ITEMS);
         hipLaunchKernelGGL((onesweep_kernel<u32, SORT_WIDE_BLOCK, SORT32_ITEMS, SRC_PAIRS, 0>), dim3(a.tiles), dim3(SORT_WIDE_BLOCK), 0, s, a);
     } else {
