@@ -75,9 +75,19 @@ static_assert(SORT_WIDE_BLOCK >= SORT_BLOCK, "the look-back words are sized for 
 constexpr int RANK_BLOCK = CSA_RANK_BLOCK;
 constexpr int RANK_ITEMS = CSA_RANK_ITEMS;
 constexpr int RANK_TILE = RANK_BLOCK * RANK_ITEMS;
-// groups of up to SMALL_MAXG suffixes are sorted inside one tile of the small-group kernel
+// Groups of up to SMALL_MAXG suffixes are sorted inside one tile of the small-group kernel; the larger ones go through
+// the radix sort. A list of mostly short groups (at most SMALL_AVG_LIMIT members per group on average: token corpora)
+// takes the higher limit SMALL_MAXG_HI, which leaves fewer members to the radix passes (1B-token workload: 117.5 ->
+// 115.4 ms per sort). A list of long groups (small alphabets, runs) keeps the lower one: the tile's halo of SMALL_MAXG
+// elements on either side and the longer member loops only cost there (4-letter workload: +6 % with the higher limit).
 #ifndef CSA_SMALL_MAXG
 #define CSA_SMALL_MAXG 64
+#endif
+#ifndef CSA_SMALL_MAXG_HI
+#define CSA_SMALL_MAXG_HI 256
+#endif
+#ifndef CSA_SMALL_AVG_LIMIT
+#define CSA_SMALL_AVG_LIMIT 16
 #endif
 #ifndef CSA_SMALL_BLOCK
 #define CSA_SMALL_BLOCK 256
@@ -89,6 +99,9 @@ constexpr int SMALL_BLOCK = CSA_SMALL_BLOCK;
 constexpr int SMALL_ITEMS = CSA_SMALL_ITEMS;
 constexpr int SMALL_TILE = SMALL_BLOCK * SMALL_ITEMS;
 constexpr int SMALL_MAXG = CSA_SMALL_MAXG;
+constexpr int SMALL_MAXG_HI = CSA_SMALL_MAXG_HI;
+constexpr u32 SMALL_AVG_LIMIT = CSA_SMALL_AVG_LIMIT;
+static_assert(SMALL_MAXG_HI >= SMALL_MAXG, "the higher group limit is the higher one");
 constexpr u32 TICKET_POOL = 4096;
 constexpr int EVENT_POOL = 2 * CSA_MAX_GENERATIONS * MAX_PASSES * 2;
 
@@ -412,18 +425,19 @@ int read_counts(Launch& L, u32* big)
 
 
 struct DeferBuffers {
-    u32* vals;    // [m] new ranks in sorted-list order (written by the rerank kernel)
+    u64* recs[2]; // generation 0: [n] (position << 32 | rank) records in sorted-list order, and their ping-pong partner
+    u32* vals;    // later generations: [m] new ranks in sorted-list order
     u32* t1_pos;  // ping
     u32* t1_val;
     u32* t2_pos;  // pong
     u32* t2_val;
 };
 
-// After a rerank launched with rank_vals = buf.vals: rank[pos[c]] = vals[c] for all c < m.
-// pos[0, n) is a permutation of the text positions [0, n) (the sorted suffixes of generation 0), which makes the
-// digit counts of the passes a closed form. The pairs are sorted on the position bits above the window size
+// After a rerank launched with rank_recs = buf.recs[0]: rank[x] = r for each of the n records (x << 32) | r.
+// The positions x are a permutation of the text positions [0, n) (the sorted suffixes of generation 0), which makes
+// the digit counts of the passes a closed form. The records are sorted on the position bits above the window size
 // (windows of at most 1 << 14 positions, 1 << 15 for the largest partitions), then placed window by window.
-int deferred_rank_update(Launch& L, const u32* pos, const DeferBuffers& buf, u32 n)
+int deferred_rank_update(Launch& L, const DeferBuffers& buf, u32 n)
 {
     csa_handle* h = L.h;
     hipStream_t s = L.stream;
@@ -446,8 +460,7 @@ int deferred_rank_update(Launch& L, const u32* pos, const DeferBuffers& buf, u32
         xbits[0] = top;
         n_pass = 1;
     }
-    const u32* in_pos = pos;
-    const u32* in_val = buf.vals;
+    const u64* in_recs = buf.recs[0];
     if (n_pass > 0) {
         u32* h_hist = h->h_pinned + 16;
         for (int p = 0; p < n_pass; ++p) {
@@ -466,20 +479,18 @@ int deferred_rank_update(Launch& L, const u32* pos, const DeferBuffers& buf, u32
         }
         HIP_TRY(hipMemcpyAsync(h->ghist, h_hist, n_pass * RADIX_BINS * sizeof(u32), hipMemcpyHostToDevice, s));
         hipLaunchKernelGGL(radix_scan_hist_kernel, dim3(1), dim3(256), 0, s, h->ghist, h->digit_base, n_pass);
-        u32* out_pos[2] = {buf.t1_pos, buf.t2_pos};
-        u32* out_val[2] = {buf.t1_val, buf.t2_val};
         for (int p = 0; p < n_pass; ++p) {
             OnesweepArgs a;
-            a.keys_in = in_pos;
-            a.vals_in = in_val;
-            a.keys_out = out_pos[p];
-            a.vals_out = out_val[p];
+            a.keys_in = in_recs;
+            a.vals_in = nullptr; // the records travel alone
+            a.keys_out = buf.recs[(p + 1) & 1];
+            a.vals_out = nullptr;
             a.text = nullptr;
             a.n = n;
             a.text_n = n;
             a.tail = 0;
             a.word = 0;
-            a.shift = xshift[p];
+            a.shift = 32 + xshift[p]; // the position is the high half of a record
             a.bits = xbits[p];
             a.digit_base = h->digit_base + p * RADIX_BINS;
             a.lookback = h->lookback;
@@ -489,16 +500,15 @@ int deferred_rank_update(Launch& L, const u32* pos, const DeferBuffers& buf, u32
                 int rc = next_ticket(L, &a.ticket);
             if (rc)
                 return rc;
-            launch_onesweep32(h, a, s);
-            in_pos = out_pos[p];
-            in_val = out_val[p];
+            launch_onesweep<SRC_PAIRS>(h, a, s);
+            in_recs = buf.recs[(p + 1) & 1];
         }
     }
     const u32 windows = (u32)((((u64)n - 1) >> window_log2) + 1);
     if (window_log2 <= 14)
-        hipLaunchKernelGGL((place_ranks_kernel<14>), dim3(windows), dim3(1024), 0, s, in_pos, in_val, n, window_log2, h->rank);
+        hipLaunchKernelGGL((place_ranks_kernel<14>), dim3(windows), dim3(1024), 0, s, in_recs, n, window_log2, h->rank);
     else
-        hipLaunchKernelGGL((place_ranks_kernel<15>), dim3(windows), dim3(1024), 0, s, in_pos, in_val, n, window_log2, h->rank);
+        hipLaunchKernelGGL((place_ranks_kernel<15>), dim3(windows), dim3(1024), 0, s, in_recs, n, window_log2, h->rank);
     HIP_TRY(hipGetLastError());
     return CSA_OK;
 }
@@ -619,17 +629,17 @@ int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivo
     ra.slab_total = r.slab_total;
     ra.slab = r.slab;
     ra.err = h->counts + 2;
-    ra.rank_vals = nullptr;
+    ra.rank_recs = nullptr;
     hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS, false>), dim3(r.tiles), dim3(RANK_BLOCK), 0, s, ra);
     int rc = rank_totals(L, r, true, ra.m, ra.n, false, survivors, groups, rank_update);
     if (rc)
         return rc;
     if (*rank_update != 0)
-        ra.rank_vals = buf.vals;
+        ra.rank_recs = buf.recs[0];
     hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS, true>), dim3(r.tiles), dim3(RANK_BLOCK), 0, s, ra);
     HIP_TRY(hipGetLastError());
     if (*rank_update == 1)
-        return deferred_rank_update(L, ra.sufs, buf, ra.n);
+        return deferred_rank_update(L, buf, ra.n);
     return CSA_OK;
 }
 
@@ -695,7 +705,9 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     ra.gprim_out = h->gprim[0];
     ra.gstart_out = h->gstart[0];
     // scratch of the bucketed rank update: all free while (and after) a list is being ranked
-    const DeferBuffers defer_buf = {bx[0], bx[1], reinterpret_cast<u32*>(bkey[0]), reinterpret_cast<u32*>(bkey[1]),
+    // (the records of generation 0 start in the third key array and swap with the sort's other output array; the sorted
+    // keys themselves are still being read when the first records are written)
+    const DeferBuffers defer_buf = {{bkey[0], key_out}, bx[0], bx[1], reinterpret_cast<u32*>(bkey[0]), reinterpret_cast<u32*>(bkey[1]),
                                     reinterpret_cast<u32*>(bkey[1]) + h->cap};
     u32 m = 0, groups = 0, big = 0;
     rc = rerank_step(L, ra, defer_buf, &m, &groups, &st->rank_update[0]);
@@ -709,7 +721,8 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     // ---- generations t >= 1 (reference loop: src/GPU_SACA.cu:1999-2103) ----
     int gen = 1;
     int gp = 0; // gprim[gp] / gstart[gp] describe the current groups
-    bool all_small = false; // no group of the current list exceeds SMALL_MAXG members
+    bool all_small = false; // no group of the current list exceeds the limit of the generation that found it so
+    bool high_limit = false; // that generation's limit was SMALL_MAXG_HI (groups only split: the limit stays from there on)
     const int sec_bits = bit_length(n > 1 ? n - 1 : 1);
     u64 ctx = ell; // symbols resolved so far; the next generation looks hop symbols ahead
     while (m > 0) {
@@ -748,14 +761,23 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
             // kernel then also counts for the apply step, and nothing else runs before it.
             HIP_TRY(hipMemsetAsync(r.tile_agg, 0, (u64)r.tiles * 4 * sizeof(u32), s));
             HIP_TRY(hipMemsetAsync(r.tile_splits, 0, (u64)r.tiles * sizeof(u32), s));
-            hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG, true>), dim3(r.tiles), dim3(SMALL_BLOCK), 0, s,
-                               sa);
+            if (high_limit)
+                hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG_HI, true>), dim3(r.tiles), dim3(SMALL_BLOCK), 0,
+                                   s, sa);
+            else
+                hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG, true>), dim3(r.tiles), dim3(SMALL_BLOCK), 0, s,
+                                   sa);
             HIP_TRY(hipGetLastError());
             st->small_only[gen] = 1;
         } else {
             HIP_TRY(hipMemsetAsync(h->counts + 4, 0, sizeof(u32), s));
-            hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG, false>), dim3(r.tiles), dim3(SMALL_BLOCK), 0, s,
-                               sa);
+            high_limit = (u64)m_in <= (u64)groups * SMALL_AVG_LIMIT;
+            if (high_limit)
+                hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG_HI, false>), dim3(r.tiles), dim3(SMALL_BLOCK), 0,
+                                   s, sa);
+            else
+                hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG, false>), dim3(r.tiles), dim3(SMALL_BLOCK), 0, s,
+                                   sa);
             HIP_TRY(hipGetLastError());
             rc = read_counts(L, &big);
             if (rc)

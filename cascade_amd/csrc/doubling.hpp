@@ -31,11 +31,10 @@ struct RerankArgs {
     u32 ell;       // symbols in the generation-0 key
     const u16* text;
     u32* rank;     // [n] by text position
-    // Deferred rank update: instead of the scattered write rank[x] = r, the new rank of the suffix at sorted
-    // index c is stored at rank_vals[c] (a coalesced stream; the suffix itself is sufs[c]). The (x, r) pairs then go
-    // through radix passes on the high bits of x before they are written to rank[], so that those writes fall into
-    // one window of rank[] at a time. (Later generations mark unchanged ranks with NO_RANK in such a stream.)
-    u32* rank_vals; // null: write rank[x] directly
+    // Deferred rank update: instead of the scattered write rank[x] = r, the suffix at sorted index c leaves the record
+    // (x << 32) | r at rank_recs[c] (a coalesced stream). The records then go through radix passes on the high bits of
+    // x before they are written to rank[], so that those writes fall into one window of rank[] at a time.
+    u64* rank_recs; // null: write rank[x] directly
     u32* sufs_out;  // first active list
     u32* gids_out;
     u32* gprim_out;
@@ -62,7 +61,6 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
     constexpr int PADDED = SLOTS + SLOTS / ITEMS + 1;
     __shared__ u64 s_key[PADDED]; // later: compacted survivors (suffixes, group ids)
     __shared__ u32 s_suf[PADDED]; // later: tables of the groups (first rank, start)
-    __shared__ u32 s_rv[TILE];    // ranks in list order (deferred rank update only)
     __shared__ u32 s_wagg[WAVES][3];
 #define CSA_PAD(q) ((q) + (q) / ITEMS)
 
@@ -182,9 +180,11 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
     u32* s_oprim = s_suf;                        // [TILE / 2] first rank of each group of the tile
     u32* s_ostart = s_suf + TILE / 2;            // [TILE / 2] and its start in the active list
 
+    u64 rec[ITEMS]; // (position << 32 | rank) records of the thread's elements (deferred rank update)
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         const u64 c = base + k;
+        rec[k] = 0;
         if (c < m) {
             const bool ka = !eq[k];
             const bool single = ka && !eq[k + 1];
@@ -196,8 +196,8 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
                 atomicExch(a.err, DEV_ERR_RERANK_RANGE);
                 continue;
             }
-            if (a.rank_vals)
-                s_rv[t * ITEMS + k] = nr;
+            if (a.rank_recs)
+                rec[k] = ((u64)x << 32) | nr;
             else
                 a.rank[x] = nr;
             if (!single) {
@@ -212,6 +212,20 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
             }
         }
     }
+    // a thread's ITEMS records are neighbours in memory: whole 16-byte stores where the tile is full
+    if (a.rank_recs) {
+        if (ITEMS % 2 == 0 && tile_base + TILE <= m) {
+            uint4* out = reinterpret_cast<uint4*>(a.rank_recs + base); // base is a multiple of ITEMS: 16-byte aligned
+#pragma unroll
+            for (int k = 0; k < ITEMS; k += 2)
+                out[k / 2] = make_uint4((u32)rec[k], (u32)(rec[k] >> 32), (u32)rec[k + 1], (u32)(rec[k + 1] >> 32));
+        } else {
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k)
+                if (base + k < m)
+                    a.rank_recs[base + k] = rec[k];
+        }
+    }
     __syncthreads();
     // striped write-out of what the tile produced
     const u32 n_surv = tile_total_surv, n_heads = tile_total_heads;
@@ -223,9 +237,6 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
         a.gprim_out[tile_rh + i] = s_oprim[i];
         a.gstart_out[tile_rh + i] = s_ostart[i];
     }
-    if (a.rank_vals)
-        for (u32 i = t; i < (u32)TILE && tile_base + i < m; i += BLOCK)
-            a.rank_vals[tile_base + i] = s_rv[i];
 #undef CSA_PAD
 }
 
@@ -308,23 +319,23 @@ __global__ __launch_bounds__(1024) void rerank_scan_kernel(const u32* __restrict
     }
 }
 
-// Last step of the deferred rank update. The (text position, rank) pairs of generation 0 arrive sorted by the
-// high bits of the position; the positions are a permutation of [0, n), so the pairs of window w (positions
-// [w * S, (w + 1) * S), S = 1 << window_log2) are exactly pairs [w * S, (w + 1) * S) of the list. One workgroup
+// Last step of the deferred rank update. The (text position << 32 | rank) records of generation 0 arrive sorted by
+// the high bits of the position; the positions are a permutation of [0, n), so the records of window w (positions
+// [w * S, (w + 1) * S), S = 1 << window_log2) are exactly records [w * S, (w + 1) * S) of the list. One workgroup
 // per window scatters the ranks into an LDS image of the window and writes the image out in full lines.
 template <int MAX_LOG2>
-__global__ __launch_bounds__(1024) void place_ranks_kernel(const u32* __restrict__ pos, const u32* __restrict__ val, u32 n,
-                                                           int window_log2, u32* __restrict__ rank)
+__global__ __launch_bounds__(1024) void place_ranks_kernel(const u64* __restrict__ recs, u32 n, int window_log2,
+                                                           u32* __restrict__ rank)
 {
     __shared__ u32 s_win[1 << MAX_LOG2];
     const u32 S = 1u << window_log2;
     const u64 first = (u64)blockIdx.x << window_log2;
     const u32 count = (u32)((u64)n - first < S ? (u64)n - first : S);
     for (u32 i = threadIdx.x; i < count; i += 1024) {
-        const u32 x = pos[first + i];
-        const u32 off = x - (u32)first;
+        const u64 r = recs[first + i];
+        const u32 off = (u32)(r >> 32) - (u32)first;
         if (off < count) // always, for a permutation sorted by window
-            s_win[off] = val[first + i];
+            s_win[off] = (u32)r;
     }
     __syncthreads();
     for (u32 i = threadIdx.x; i < count; i += 1024)
@@ -662,7 +673,7 @@ struct ApplySmallArgs {
     const u32* nr; // bit 31: the rank changed
     u32 m, n;
     u32* rank;
-    u32* rank_vals; // null: write rank[x] directly (see RerankArgs::rank_vals)
+    u32* rank_vals; // null: write rank[x] directly; else the rank of list place c goes to rank_vals[c] (NO_RANK where unchanged)
     u32* sa32;      // suffix array under construction
     u32* sufs_out;
     u32* gids_out;

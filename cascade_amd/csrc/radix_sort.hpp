@@ -165,7 +165,7 @@ __global__ __launch_bounds__(256) void radix_scan_hist_kernel(const u32* ghist, 
 
 struct OnesweepArgs {
     const void* keys_in; // u64 keys, or u32 keys for the narrow instantiation
-    const u32* vals_in;
+    const u32* vals_in;  // null (SRC_PAIRS only): the keys travel alone, vals_out is not written
     void* keys_out;
     u32* vals_out;
     const u16* text;
@@ -401,12 +401,13 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
 
     // the values are asked for now: their way from HBM overlaps the writes of the keys below (asked for before the
     // look-back they would delay its words, which come back in the order of issue)
+    const bool has_vals = SRC == SRC_TEXT || a.vals_in != nullptr;
     u32 val[ITEMS];
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         const u32 local = first_local + k * WAVE;
         val[k] = 0;
-        if (local < valid)
+        if (has_vals && local < valid)
             val[k] = SRC == SRC_TEXT ? virtual_to_suffix((u32)(base + local), a.text_n, a.tail) : a.vals_in[base + local];
     }
     // ---- write runs of equal digits to their global places ----
@@ -420,6 +421,8 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
             keys_out[dst[k]] = kk;
         }
     }
+    if (!has_vals) // the same for every thread of the launch
+        return;
     __syncthreads();
     u32* s_vals = reinterpret_cast<u32*>(s_keys);
 #pragma unroll
