@@ -240,23 +240,23 @@ bool wide_workgroups(const OnesweepArgs& a)
     return SORT_WIDE_BLOCK > SORT_BLOCK && a.n >= SORT_WIDE_MIN;
 }
 
-template <int SRC, int BLOCK>
+template <int SRC, int BLOCK, bool VALS>
 void launch_onesweep_shape(const csa_handle* h, OnesweepArgs& a, hipStream_t s)
 {
     set_tile_order(h, a, BLOCK * SORT_ITEMS);
     if (a.shift >= 32)
-        hipLaunchKernelGGL((onesweep_kernel<u64, BLOCK, SORT_ITEMS, SRC, 1>), dim3(a.tiles), dim3(BLOCK), 0, s, a);
+        hipLaunchKernelGGL((onesweep_kernel<u64, BLOCK, SORT_ITEMS, SRC, 1, VALS>), dim3(a.tiles), dim3(BLOCK), 0, s, a);
     else
-        hipLaunchKernelGGL((onesweep_kernel<u64, BLOCK, SORT_ITEMS, SRC, 0>), dim3(a.tiles), dim3(BLOCK), 0, s, a);
+        hipLaunchKernelGGL((onesweep_kernel<u64, BLOCK, SORT_ITEMS, SRC, 0, VALS>), dim3(a.tiles), dim3(BLOCK), 0, s, a);
 }
 
-template <int SRC>
+template <int SRC, bool VALS = true>
 void launch_onesweep(const csa_handle* h, OnesweepArgs& a, hipStream_t s)
 {
     if (wide_workgroups(a))
-        launch_onesweep_shape<SRC, SORT_WIDE_BLOCK>(h, a, s);
+        launch_onesweep_shape<SRC, SORT_WIDE_BLOCK, VALS>(h, a, s);
     else
-        launch_onesweep_shape<SRC, SORT_BLOCK>(h, a, s);
+        launch_onesweep_shape<SRC, SORT_BLOCK, VALS>(h, a, s);
 }
 
 void launch_onesweep32(const csa_handle* h, OnesweepArgs& a, hipStream_t s)
@@ -500,7 +500,7 @@ int deferred_rank_update(Launch& L, const DeferBuffers& buf, u32 n)
                 int rc = next_ticket(L, &a.ticket);
             if (rc)
                 return rc;
-            launch_onesweep<SRC_PAIRS>(h, a, s);
+            launch_onesweep<SRC_PAIRS, false>(h, a, s);
             in_recs = buf.recs[(p + 1) & 1];
         }
     }

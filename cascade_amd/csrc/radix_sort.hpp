@@ -165,7 +165,7 @@ __global__ __launch_bounds__(256) void radix_scan_hist_kernel(const u32* ghist, 
 
 struct OnesweepArgs {
     const void* keys_in; // u64 keys, or u32 keys for the narrow instantiation
-    const u32* vals_in;  // null (SRC_PAIRS only): the keys travel alone, vals_out is not written
+    const u32* vals_in;  // unused by the instantiations without values, like vals_out
     void* keys_out;
     u32* vals_out;
     const u16* text;
@@ -234,9 +234,11 @@ __device__ __forceinline__ u32 onesweep_tile_number(const OnesweepArgs& a)
 // KeyT is u64 (the suffix-sort keys) or u32 (the (text position, rank) pairs of the bucketed rank update).
 // HI selects the 32-bit half of a 64-bit key that holds this pass's digit (digits never straddle the halves),
 // so that the digit is one bit-field extract of a 32-bit register.
-template <typename KeyT, int BLOCK, int ITEMS, int SRC, int HI>
+// VALS = false: the keys travel alone (records whose payload sits in the key bits that are not sorted on).
+template <typename KeyT, int BLOCK, int ITEMS, int SRC, int HI, bool VALS = true>
 __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(OnesweepArgs a)
 {
+    static_assert(VALS || SRC == SRC_PAIRS, "the text pass makes the suffix indices");
     constexpr int TILE = BLOCK * ITEMS;
     constexpr int WAVES = BLOCK / WAVE;
     static_assert(BLOCK >= RADIX_BINS, "one thread per digit is assumed");
@@ -401,13 +403,12 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
 
     // the values are asked for now: their way from HBM overlaps the writes of the keys below (asked for before the
     // look-back they would delay its words, which come back in the order of issue)
-    const bool has_vals = SRC == SRC_TEXT || a.vals_in != nullptr;
     u32 val[ITEMS];
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         const u32 local = first_local + k * WAVE;
         val[k] = 0;
-        if (has_vals && local < valid)
+        if (VALS && local < valid)
             val[k] = SRC == SRC_TEXT ? virtual_to_suffix((u32)(base + local), a.text_n, a.tail) : a.vals_in[base + local];
     }
     // ---- write runs of equal digits to their global places ----
@@ -421,7 +422,7 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
             keys_out[dst[k]] = kk;
         }
     }
-    if (!has_vals) // the same for every thread of the launch
+    if (!VALS)
         return;
     __syncthreads();
     u32* s_vals = reinterpret_cast<u32*>(s_keys);
