@@ -111,6 +111,14 @@ constexpr int EVENT_POOL = 2 * CSA_MAX_GENERATIONS * MAX_PASSES * 2;
 #define CSA_DEFER_MIN (1u << 23)
 #endif
 constexpr u32 XCD_CHUNK = 16;
+// Windows of rank[] that the last step of generation 0's bucketed update assembles in LDS (1 << 14 positions; twice
+// that on the largest partitions, whose two passes cover 16 position bits at most). Smaller in test builds, so that
+// short lists go through the passes too.
+#ifndef CSA_PLACE_WINDOW_LOG2
+#define CSA_PLACE_WINDOW_LOG2 14
+#endif
+constexpr int PLACE_WINDOW_LOG2 = CSA_PLACE_WINDOW_LOG2;
+static_assert(PLACE_WINDOW_LOG2 >= 1 && PLACE_WINDOW_LOG2 <= 14, "the placement kernel holds a window of 1 << 14 or 1 << 15 ranks");
 constexpr u32 DEFER_MIN = CSA_DEFER_MIN;
 // Later generations: when at least half of the sorted list changes its rank, and at least WINDOW_MIN_CHANGED
 // suffixes in all, the rank writes of the generation are bucketed into windows of 1 << WINDOW_LOG2 positions of
@@ -442,7 +450,7 @@ int deferred_rank_update(Launch& L, const DeferBuffers& buf, u32 n)
     csa_handle* h = L.h;
     hipStream_t s = L.stream;
     const int nb = bit_length(n - 1); // <= 31
-    int top = nb - 14;                // position bits to sort on
+    int top = nb - PLACE_WINDOW_LOG2; // position bits to sort on
     if (top < 0)
         top = 0;
     if (top > 16)

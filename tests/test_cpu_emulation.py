@@ -108,8 +108,9 @@ def test_small_and_large_groups_take_both_paths(emu):
     got, active, big = emu_sort(emu, T, 1)
     assert np.array_equal(got, oracle_lib.build_sa40(T))
     assert big[1] > 0 and any(b == 0 and a > 0 for a, b in zip(active[2:], big[2:]))
-    # generation 0 takes the two-pass bucketed rank update here and later ones the one-pass kind (the emulation
-    # library is built with tiny thresholds for both); the short fixtures above write their ranks directly
+    # generation 0 takes the bucketed rank update here (records through one value-less radix pass on 4 position bits,
+    # then windows of 512 ranks) and later ones the one-pass kind (the emulation library is built with tiny thresholds
+    # and windows for both); the short fixtures above write their ranks directly
     assert emu_sort.rank_update[0] == 1 and 2 in emu_sort.rank_update[1:]
     # once a generation had no large group, the following ones run as the fused small-group generation
     first_small = big.index(0, 1)

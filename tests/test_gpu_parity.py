@@ -275,6 +275,36 @@ def test_random_small_texts_against_the_oracle(torch_mod):
         assert np.array_equal(got, oracle_lib.build_sa40(T)), (case, n, sigma, kw)
 
 
+def test_bucketed_rank_updates_at_small_and_ragged_sizes(torch_mod, monkeypatch):
+    """The bucketed rank updates normally serve lists of millions of suffixes: generation 0 sends (position, rank)
+    records through value-less radix passes and a window placement, later generations (position, rank) pairs through one
+    pass and a windowed scatter. With their thresholds at 1 (read when a handle is made) every list takes them: sizes
+    around the tile, window and pass boundaries, checked against the oracle, and the library must report that it went
+    that way."""
+    from cascade_amd import PartitionSorter, workloads
+    monkeypatch.setenv("CASCADE_DEFER_MIN", "1")
+    monkeypatch.setenv("CASCADE_WINDOW_MIN_CHANGED", "1")
+    rng = np.random.default_rng(77)
+    sizes = [1, 2, 5, 255, 1024, 1025, 8191, 8193, (1 << 14) - 1, 1 << 14, (1 << 14) + 1, 16385 * 3, (1 << 16) + 7,
+             (1 << 18) - 3, (1 << 20) + 11]
+    for case, n in enumerate(sizes):
+        if case % 3 == 0:
+            T = workloads.generate(3, n) if n >= 64 else rng.integers(0, 3, n).astype(np.uint16)
+        elif case % 3 == 1:
+            T = rng.integers(0, 4, n).astype(np.uint16)
+        else:
+            T = workloads.generate(5, n) if n >= 64 else np.zeros(n, dtype=np.uint16)
+        with PartitionSorter(n, key_words=1 + case % 2) as s:
+            print(f"  bucketed case={case} n={n} key_words={s.key_words}", flush=True)
+            got = s.sort(to_dev(torch_mod, T)).cpu().numpy()
+            how = s.last_stats["rank_update"]
+        if n <= 1 << 16:
+            assert np.array_equal(got, oracle_lib.build_sa40(T)), (case, n)
+        else:  # the oracle's O(n) verifier: pass = byte-equal to the one correct suffix array
+            assert oracle_lib.is_correct_sa40(got, T), (case, n)
+        assert how[0] == 1, (case, n, how)
+
+
 @pytest.mark.parametrize("key_words", [3, 4])
 def test_keys_of_three_and_four_words_on_deep_repeats(torch_mod, key_words):
     """The reference's default key is 4 words (include/Packed_Prefix.hpp:20-24): the same suffix array, fewer and
