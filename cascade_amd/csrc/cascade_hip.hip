@@ -810,14 +810,18 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
                 pa.gprim = h->gprim[gp];
                 pa.sufs_out = x_out;
                 pa.nr_out = nr_list;
-                pa.lookback = h->lookback;
-                pa.epoch = next_epoch(h);
                 pa.err = h->counts + 2;
-                rc = next_ticket(L, &pa.ticket);
-                if (rc)
-                    return rc;
-                hipLaunchKernelGGL((place_big_kernel<RANK_BLOCK, RANK_ITEMS>), dim3((big + RANK_TILE - 1) / RANK_TILE),
-                                   dim3(RANK_BLOCK), 0, s, pa);
+                // (the tile tables are free between the small-group kernel and the counting pass below)
+                const RankTables pr = rank_tables(h, big, RANK_TILE);
+                pa.tile_agg = pr.tile_agg;
+                pa.tile_splits = pr.tile_splits;
+                pa.tile_prefix = pr.tile_prefix;
+                pa.slab_total = pr.slab_total;
+                pa.slab = pr.slab;
+                hipLaunchKernelGGL((place_big_kernel<RANK_BLOCK, RANK_ITEMS, false>), dim3(pr.tiles), dim3(RANK_BLOCK), 0, s, pa);
+                hipLaunchKernelGGL(rerank_scan_kernel, dim3(pr.slabs), dim3(1024), 0, s, pr.tile_agg, pr.tile_prefix, pr.tiles, pr.slab,
+                                   pr.slab_total, pr.tile_splits);
+                hipLaunchKernelGGL((place_big_kernel<RANK_BLOCK, RANK_ITEMS, true>), dim3(pr.tiles), dim3(RANK_BLOCK), 0, s, pa);
                 HIP_TRY(hipGetLastError());
             }
             // 3. per-tile counts of the sorted list (4 bytes read per member)

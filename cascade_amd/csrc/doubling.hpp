@@ -790,7 +790,9 @@ __global__ __launch_bounds__(BLOCK) void apply_small_kernel(ApplySmallArgs a)
 // Brings the radix-sorted members of the large groups back into the sorted active list, in the (suffix, refined
 // rank) form of the small groups: the k-th sorted member of group g goes to place gstart[g] + (k - index of g's first
 // member in the sorted large-group list), and its refined rank is gprim[g] + (index of the head of its key run -
-// index of g's first member). Two max look-back chains find the two heads; wave 0 walks one, wave 1 the other.
+// index of g's first member). The two heads are running maxima over the list; like the rank step of generation 0
+// they are found in three launches (per-tile maxima, rerank_scan_kernel over the tiles, the pass that applies them),
+// which on this part beats one launch with look-back chains by a wide margin when the list is long.
 struct PlaceArgs {
     const u64* big_keys; // sorted by (group id, rank[x + h])
     const u32* big_sufs;
@@ -803,33 +805,25 @@ struct PlaceArgs {
     const u32* gprim;
     u32* sufs_out;
     u32* nr_out;
-    u64* lookback; // [tiles][2]
-    u32* ticket;
-    u32 epoch;
+    u32* tile_agg;    // [tiles][4]: last group head, last key-run head of the tile (0: none, or element 0), 0, 0
+    u32* tile_splits; // [tiles]: zeroed for the scan
+    const u32* tile_prefix; // [tiles][4]: the maxima over the earlier tiles of the tile's slab
+    const u32* slab_total;  // [RERANK_SLABS][5]
+    u32 slab;               // tiles per slab
     u32* err;
 };
 
-template <int BLOCK, int ITEMS>
+// APPLY = false: writes the tile's maxima to tile_agg. APPLY = true: reads their exclusive prefix and does the work.
+template <int BLOCK, int ITEMS, bool APPLY>
 __global__ __launch_bounds__(BLOCK) void place_big_kernel(PlaceArgs a)
 {
     constexpr int TILE = BLOCK * ITEMS;
     constexpr int WAVES = BLOCK / WAVE;
-    static_assert(WAVES >= 2, "one wave per look-back chain");
     __shared__ u32 s_wagg[WAVES][2];
-    __shared__ u32 s_prefix[2];
-    __shared__ u32 s_tile;
     const u32 t = threadIdx.x;
     const u32 lane = t & 63u;
     const u32 w = t >> 6;
-    if (t == 0) {
-        const bool failed = dev_failed(a.err); // read while the ticket is on its way
-        const u32 ticket = atomicAdd(a.ticket, 1u);
-        s_tile = failed ? 0xFFFFFFFFu : ticket;
-    }
-    __syncthreads();
-    const u32 tile = s_tile;
-    if (tile == 0xFFFFFFFFu)
-        return; // the step is lost already
+    const u32 tile = blockIdx.x;
     const u64 base = (u64)tile * TILE + (u64)t * ITEMS;
 
     u64 key[ITEMS + 1]; // element base - 1 first
@@ -855,6 +849,21 @@ __global__ __launch_bounds__(BLOCK) void place_big_kernel(PlaceArgs a)
         s_wagg[w][1] = ik;
     }
     __syncthreads();
+    if (!APPLY) {
+        if (t == 0) {
+            u32 ag = 0, ak = 0;
+            for (int ww = 0; ww < WAVES; ++ww) {
+                ag = ag > s_wagg[ww][0] ? ag : s_wagg[ww][0];
+                ak = ak > s_wagg[ww][1] ? ak : s_wagg[ww][1];
+            }
+            a.tile_agg[(u64)tile * 4 + 0] = ag;
+            a.tile_agg[(u64)tile * 4 + 1] = ak;
+            a.tile_agg[(u64)tile * 4 + 2] = 0;
+            a.tile_agg[(u64)tile * 4 + 3] = 0;
+            a.tile_splits[tile] = 0;
+        }
+        return;
+    }
     u32 xg = __shfl_up(ig, 1), xk = __shfl_up(ik, 1);
     if (lane == 0)
         xg = xk = 0;
@@ -862,17 +871,15 @@ __global__ __launch_bounds__(BLOCK) void place_big_kernel(PlaceArgs a)
         xg = xg > s_wagg[ww][0] ? xg : s_wagg[ww][0];
         xk = xk > s_wagg[ww][1] ? xk : s_wagg[ww][1];
     }
-    if (w < 2) {
-        u32 agg = 0;
-        for (int ww = 0; ww < WAVES; ++ww)
-            agg = agg > s_wagg[ww][w] ? agg : s_wagg[ww][w];
-        const u32 prefix = lb_wave_exclusive<true>(a.lookback + w, 2, tile, a.epoch, agg, a.err);
-        if (lane == 0)
-            s_prefix[w] = prefix;
+    // prefix of the tile = totals of the slabs before its slab, combined with its prefix inside the slab
+    u32 pre_g = a.tile_prefix[(u64)tile * 4 + 0], pre_k = a.tile_prefix[(u64)tile * 4 + 1];
+    for (u32 sl = 0; sl < tile / a.slab; ++sl) {
+        const u32 sg = a.slab_total[sl * 5 + 0], sk = a.slab_total[sl * 5 + 1];
+        pre_g = pre_g > sg ? pre_g : sg;
+        pre_k = pre_k > sk ? pre_k : sk;
     }
-    __syncthreads();
-    u32 ghead = xg > s_prefix[0] ? xg : s_prefix[0];
-    u32 khead = xk > s_prefix[1] ? xk : s_prefix[1];
+    u32 ghead = xg > pre_g ? xg : pre_g;
+    u32 khead = xk > pre_k ? xk : pre_k;
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         const u64 c = base + k;
