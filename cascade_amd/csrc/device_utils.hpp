@@ -97,7 +97,7 @@ __device__ __forceinline__ u64 lb_load(const u64* p)
 
 // Publishes `aggregate` of `tile` on the chain whose word for tile t lives at chain[t * stride] (tile 0's aggregate is
 // its inclusive prefix). A kernel publishes as soon as the aggregate is known and waits for its predecessors as late
-// as possible; the two walks below do the waiting.
+// as possible; the walk below does the waiting.
 __device__ __forceinline__ void lb_publish(u64* chain, u32 stride, u32 tile, u32 epoch, u32 aggregate)
 {
     lb_store(chain + (u64)tile * stride, lb_pack(epoch, tile == 0 ? LB_INCL : LB_AGG, aggregate));
@@ -187,13 +187,7 @@ __device__ __forceinline__ u32 lb2_wait_exclusive(u64* tile_chain, u64* group_ch
     return gexcl + within;
 }
 
-// ---- wave-wide look-back ----
-// The same protocol walked by a whole wave: each round every lane loads the word of one predecessor (LOADS words
-// per lane, 64 * LOADS predecessors per round), ballots find the run of published words nearest to the tile and
-// the first inclusive word inside it, and a wave reduction combines that run. The number of tiles a launch can
-// resolve per unit time is (predecessors inspected per round) / (memory round trip); with one word per round
-// trip the kernels stall with every resident tile waiting in its look-back.
-// Must be called by all 64 lanes of a wave, converged; returns the same value in every lane.
+// ---- wave-wide reduction ----
 
 __device__ __forceinline__ u32 wave_reduce_sum(u32 v)
 {
@@ -201,83 +195,6 @@ __device__ __forceinline__ u32 wave_reduce_sum(u32 v)
     for (int o = 32; o > 0; o >>= 1)
         v += __shfl_xor(v, o);
     return v;
-}
-
-__device__ __forceinline__ u32 wave_reduce_max(u32 v)
-{
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const u32 t = __shfl_xor(v, o);
-        v = v > t ? v : t;
-    }
-    return v;
-}
-
-#ifndef CSA_LB_LOADS
-#define CSA_LB_LOADS 2
-#endif
-
-template <bool IS_MAX, int LOADS = CSA_LB_LOADS>
-__device__ __forceinline__ u32 lb_wave_exclusive(u64* chain, u32 stride, u32 tile, u32 epoch, u32 aggregate, u32* err)
-{
-    const u32 lane = lane_id();
-    if (lane == 0)
-        lb_publish(chain, stride, tile, epoch, aggregate);
-    if (tile == 0)
-        return 0;
-    u32 excl = 0;
-    long long next = (long long)tile - 1; // nearest predecessor not yet consumed
-    u32 idle = 0;
-    bool done = false;
-    while (!done) {
-        u64 word[LOADS];
-#pragma unroll
-        for (int j = 0; j < LOADS; ++j) {
-            const long long idx = next - (long long)(j * WAVE + lane);
-            word[j] = idx >= 0 ? lb_load(chain + (u64)idx * stride) : 0ull;
-        }
-        u32 consumed = 0;
-#pragma unroll
-        for (int j = 0; j < LOADS; ++j) {
-            // words of this batch, nearest predecessor in lane 0; a batch is looked at only if every earlier one
-            // of the round was consumed whole
-            const bool look = !done && consumed == (u32)(j * WAVE);
-            const long long idx = next - (long long)(j * WAVE + lane);
-            const u32 status = (idx >= 0 && (u32)(word[j] >> 34) == epoch) ? ((u32)(word[j] >> 32) & 3u) : 0u;
-            const u64 ready = __ballot(status != 0);
-            const u64 incl = __ballot(status == LB_INCL);
-            if (look) {
-                const u32 lead = ready == ~0ull ? 64u : (u32)__builtin_ctzll(~ready);
-                const u64 lead_mask = lead == 64u ? ~0ull : ((1ull << lead) - 1ull);
-                const u64 incl_in = incl & lead_mask;
-                const u32 take = incl_in ? (u32)__builtin_ctzll(incl_in) + 1u : lead;
-                const u32 mine = lane < take ? (u32)word[j] : 0u;
-                const u32 part = IS_MAX ? wave_reduce_max(mine) : wave_reduce_sum(mine);
-                excl = IS_MAX ? (excl > part ? excl : part) : excl + part;
-                consumed += take;
-                if (incl_in)
-                    done = true;
-            }
-        }
-        next -= consumed;
-        if (!done && consumed == 0) {
-            if (++idle >= LB_SPIN_LIMIT) {
-                if (lane == 0)
-                    atomicExch(err, DEV_ERR_LOOKBACK_TIMEOUT);
-                return excl;
-            }
-            if ((idle & 1023u) == 0u && __ballot(dev_failed(err)) != 0ull)
-                return excl; // another wait has failed: the launch is lost
-            __builtin_amdgcn_s_sleep(1);
-        } else {
-            idle = 0;
-        }
-    }
-    if (lane == 0) {
-        const u32 inclusive = IS_MAX ? (excl > aggregate ? excl : aggregate) : excl + aggregate;
-        lb_store(chain + (u64)tile * stride, lb_pack(epoch, LB_INCL, inclusive));
-    }
-    return excl;
 }
 
 // ---- K-gram key: four uint16 symbols of the zero-padded text, the first one most significant ----
