@@ -83,7 +83,7 @@ int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out);
 /* Declares whether calls on this handle have the device to themselves (exclusive != 0): no other handle, stream or
  * process launches work on it while such a call runs. Only then may the radix passes number their tiles by
  * workgroup index in XCD-sized chunks (about 1.5% faster on the 1B-token workload): that order waits for workgroups
- * which are dispatched later and needs 128 workgroups of a pass resident together, which launches that share the
+ * which are dispatched later and needs up to 128 workgroups of a pass resident together, which launches that share the
  * device do not guarantee; an unfulfilled wait ends in CSA_ERR_INTERNAL ("look-back wait ran into its spin limit"),
  * not in a hang. The default (0) numbers tiles by arrival and is safe next to any other work, e.g. the three
  * dispatcher threads of the reference (STREAM_C, include/GPU_SACA.hpp:90-91), each with a handle of its own.
