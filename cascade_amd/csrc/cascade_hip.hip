@@ -638,13 +638,13 @@ int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivo
     ra.slab = r.slab;
     ra.err = h->counts + 2;
     ra.rank_recs = nullptr;
-    hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS, false>), dim3(r.tiles), dim3(RANK_BLOCK), 0, s, ra);
+    hipLaunchKernelGGL((rerank_count_kernel<RANK_BLOCK, RANK_ITEMS>), dim3(r.tiles), dim3(RANK_BLOCK), 0, s, ra);
     int rc = rank_totals(L, r, true, ra.m, ra.n, false, survivors, groups, rank_update);
     if (rc)
         return rc;
     if (*rank_update != 0)
         ra.rank_recs = buf.recs[0];
-    hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS, true>), dim3(r.tiles), dim3(RANK_BLOCK), 0, s, ra);
+    hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS>), dim3(r.tiles), dim3(RANK_BLOCK), 0, s, ra);
     HIP_TRY(hipGetLastError());
     if (*rank_update == 1)
         return deferred_rank_update(L, buf, ra.n);

@@ -47,22 +47,127 @@ struct RerankArgs {
     u32* err;
 };
 
-// APPLY = false: writes the tile's aggregates to tile_agg. APPLY = true: reads the tile's exclusive prefix from
-// tile_prefix (rerank_scan_kernel in between) and does the work.
-template <int BLOCK, int ITEMS, bool APPLY>
+// Elements base - 1 .. base + ITEMS of the sorted (key, suffix) list, m elements long, for the thread that owns
+// elements base .. base + ITEMS - 1 (base a multiple of ITEMS): its own in whole 16-byte loads where they all exist,
+// zeros outside the list.
+template <int ITEMS>
+__device__ __forceinline__ void load_with_neighbours(const u64* __restrict__ keys, const u32* __restrict__ sufs, u64 base, u32 m,
+                                                     u64 (&key)[ITEMS + 2], u32 (&suf)[ITEMS + 2])
+{
+    if (ITEMS % 4 == 0 && base + ITEMS <= m) {
+        const uint4* k4 = reinterpret_cast<const uint4*>(keys + base);
+        const uint4* s4 = reinterpret_cast<const uint4*>(sufs + base);
+#pragma unroll
+        for (int k = 0; k < ITEMS; k += 2) {
+            const uint4 v = k4[k / 2];
+            key[k + 1] = (u64)v.x | ((u64)v.y << 32);
+            key[k + 2] = (u64)v.z | ((u64)v.w << 32);
+        }
+#pragma unroll
+        for (int k = 0; k < ITEMS; k += 4) {
+            const uint4 v = s4[k / 4];
+            suf[k + 1] = v.x;
+            suf[k + 2] = v.y;
+            suf[k + 3] = v.z;
+            suf[k + 4] = v.w;
+        }
+        key[0] = base >= 1 ? keys[base - 1] : 0;
+        suf[0] = base >= 1 ? sufs[base - 1] : 0;
+        const bool last_in = base + ITEMS < m;
+        key[ITEMS + 1] = last_in ? keys[base + ITEMS] : 0;
+        suf[ITEMS + 1] = last_in ? sufs[base + ITEMS] : 0;
+    } else {
+#pragma unroll
+        for (int k = 0; k < ITEMS + 2; ++k) {
+            const u64 c = base + k; // element c - 1
+            const bool in = c >= 1 && c - 1 < m;
+            key[k] = in ? keys[c - 1] : 0;
+            suf[k] = in ? sufs[c - 1] : 0;
+        }
+    }
+}
+
+// The counting pass of generation 0 on its own: the per-tile aggregates need no ordering inside the tile, so every
+// thread reads its ITEMS elements and their two neighbours straight from the arrays (no exchange through LDS, one
+// barrier) and the tile reduces instead of scanning. Same run and tail rules as rerank_kernel below.
+template <int BLOCK, int ITEMS>
+__global__ __launch_bounds__(BLOCK) void rerank_count_kernel(RerankArgs a)
+{
+    constexpr int TILE = BLOCK * ITEMS;
+    constexpr int WAVES = BLOCK / WAVE;
+    __shared__ u32 s_wagg[WAVES][3];
+    const u32 t = threadIdx.x;
+    const u32 lane = t & 63u;
+    const u32 w = t >> 6;
+    const u32 tile = blockIdx.x;
+    const u64 base = (u64)tile * TILE + (u64)t * ITEMS;
+    const u32 m = a.m;
+    u64 key[ITEMS + 2]; // elements base - 1 .. base + ITEMS
+    u32 suf[ITEMS + 2];
+    load_with_neighbours<ITEMS>(a.keys, a.sufs, base, m, key, suf);
+    u32 la = 0, lcnt = 0, lheads = 0;
+    bool prev_eq = false;
+#pragma unroll
+    for (int k = 0; k < ITEMS + 1; ++k) {
+        const u64 c = base + k; // right element of the pair (c - 1, c)
+        bool e = c >= 1 && c < m && key[k] == key[k + 1];
+        for (int word = 1; e && word < a.key_words; ++word)
+            e = load_kgram(a.text, a.n, suf[k], (u32)word) == load_kgram(a.text, a.n, suf[k + 1], (u32)word);
+        // a suffix that runs off the text inside its key ties with nobody (include/bit-layout.hpp:99-100)
+        if (e && ((u64)suf[k] + a.ell >= a.n || (u64)suf[k + 1] + a.ell >= a.n))
+            e = false;
+        if (k >= 1 && c - 1 < m) { // element c - 1 = base + k - 1: prev_eq ties it to its left, e to its right
+            const bool ka = !prev_eq;
+            const bool single = ka && !e;
+            if (ka)
+                la = (u32)(c - 1) + 1u;
+            lcnt += single ? 0u : 1u;
+            lheads += (ka && !single) ? 1u : 0u;
+        }
+        prev_eq = e;
+    }
+    u32 ra = la, rc = lcnt, rh = lheads;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const u32 oa = __shfl_xor(ra, o);
+        ra = ra > oa ? ra : oa;
+        rc += __shfl_xor(rc, o);
+        rh += __shfl_xor(rh, o);
+    }
+    if (lane == 0) {
+        s_wagg[w][0] = ra;
+        s_wagg[w][1] = rc;
+        s_wagg[w][2] = rh;
+    }
+    __syncthreads();
+    if (t == 0) {
+        u32 ta = 0, tc = 0, th = 0;
+        for (int ww = 0; ww < WAVES; ++ww) {
+            ta = ta > s_wagg[ww][0] ? ta : s_wagg[ww][0];
+            tc += s_wagg[ww][1];
+            th += s_wagg[ww][2];
+        }
+        a.tile_agg[(u64)tile * 4 + 0] = ta;
+        a.tile_agg[(u64)tile * 4 + 1] = 0;
+        a.tile_agg[(u64)tile * 4 + 2] = tc;
+        a.tile_agg[(u64)tile * 4 + 3] = th;
+        a.tile_splits[tile] = 0;
+    }
+}
+
+// The applying pass: reads the tile's exclusive prefix from tile_prefix (rerank_count_kernel and rerank_scan_kernel
+// before it) and does the work. What the tile produces is collected in LDS and leaves in striped order (consecutive
+// lanes, consecutive elements).
+template <int BLOCK, int ITEMS>
 __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
 {
     constexpr int TILE = BLOCK * ITEMS;
     constexpr int WAVES = BLOCK / WAVE;
-    // The tile is read from and written to HBM in striped order (consecutive lanes, consecutive elements) and
-    // exchanged through LDS with the blocked order (each thread, ITEMS consecutive elements) the scans want.
-    // One pad slot per ITEMS elements keeps the blocked LDS accesses off a single bank.
-    constexpr int SLOTS = TILE + 2;               // element tile_base - 1, the tile, element tile_base + TILE
-    constexpr int PADDED = SLOTS + SLOTS / ITEMS + 1;
-    __shared__ u64 s_key[PADDED]; // later: compacted survivors (suffixes, group ids)
-    __shared__ u32 s_suf[PADDED]; // later: tables of the groups (first rank, start)
+    __shared__ u32 s_osuf[TILE];       // survivors of the tile, compacted
+    __shared__ u32 s_ogid[TILE];       // their group ids
+    __shared__ u32 s_oprim[TILE / 2];  // first rank of each group of the tile
+    __shared__ u32 s_ostart[TILE / 2]; // and its start in the active list
     __shared__ u32 s_wagg[WAVES][3];
-#define CSA_PAD(q) ((q) + (q) / ITEMS)
 
     const u32 t = threadIdx.x;
     const u32 lane = t & 63u;
@@ -72,33 +177,11 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
     const u64 base = tile_base + (u64)t * ITEMS;
     const u32 m = a.m;
 
-    // striped load into LDS: slot q holds element tile_base + q - 1
-#pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-        const u32 q = j * BLOCK + t + 1;
-        const u64 c = tile_base + q - 1;
-        const bool in = c < m;
-        s_key[CSA_PAD(q)] = in ? a.keys[c] : 0;
-        s_suf[CSA_PAD(q)] = in ? a.sufs[c] : 0;
-    }
-    if (t < 2) {
-        const u32 q = t == 0 ? 0u : (u32)TILE + 1u;
-        const bool in = t == 0 ? tile_base >= 1 : tile_base + TILE < m;
-        const u64 c = tile_base + q - 1;
-        s_key[CSA_PAD(q)] = in ? a.keys[c] : 0;
-        s_suf[CSA_PAD(q)] = in ? a.sufs[c] : 0;
-    }
-    __syncthreads();
-
-    // blocked read: elements base - 1 .. base + ITEMS
+    // every thread reads its ITEMS elements (whole 16-byte loads where the tile is full) and their two neighbours
+    // straight from the arrays: elements base - 1 .. base + ITEMS
     u64 key[ITEMS + 2];
     u32 suf[ITEMS + 2];
-#pragma unroll
-    for (int k = 0; k < ITEMS + 2; ++k) {
-        const u32 q = t * ITEMS + k;
-        key[k] = s_key[CSA_PAD(q)];
-        suf[k] = s_suf[CSA_PAD(q)];
-    }
+    load_with_neighbours<ITEMS>(a.keys, a.sufs, base, m, key, suf);
     // eq[k]: elements (base+k-1) and (base+k) exist and belong to one run of equal keys
     bool eq[ITEMS + 1];
 #pragma unroll
@@ -135,30 +218,19 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
         s_wagg[w][1] = ic;
         s_wagg[w][2] = ih;
     }
-    __syncthreads(); // also: every thread holds its elements in registers, the staging arrays may be reused
+    __syncthreads();
     u32 xa = __shfl_up(ia, 1), xc = __shfl_up(ic, 1), xh = __shfl_up(ih, 1);
     if (lane == 0)
         xa = xc = xh = 0;
-    u32 tile_a = 0, tile_total_surv = 0, tile_total_heads = 0;
+    u32 tile_total_surv = 0, tile_total_heads = 0;
     for (u32 ww = 0; ww < WAVES; ++ww) {
         if (ww < w) {
             xa = xa > s_wagg[ww][0] ? xa : s_wagg[ww][0];
             xc += s_wagg[ww][1];
             xh += s_wagg[ww][2];
         }
-        tile_a = tile_a > s_wagg[ww][0] ? tile_a : s_wagg[ww][0];
         tile_total_surv += s_wagg[ww][1];
         tile_total_heads += s_wagg[ww][2];
-    }
-    if (!APPLY) {
-        if (t == 0) {
-            a.tile_agg[(u64)tile * 4 + 0] = tile_a;
-            a.tile_agg[(u64)tile * 4 + 1] = 0;
-            a.tile_agg[(u64)tile * 4 + 2] = tile_total_surv;
-            a.tile_agg[(u64)tile * 4 + 3] = tile_total_heads;
-            a.tile_splits[tile] = 0;
-        }
-        return;
     }
     // prefix of the tile = totals of the slabs before its slab, combined with its prefix inside the slab
     u32 pre_a = a.tile_prefix[(u64)tile * 4 + 0];
@@ -174,12 +246,6 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
     u32 ra = xa > pre_a ? xa : pre_a;
     u32 rc = xc; // tile-local from here on
     u32 rh = xh;
-    __syncthreads(); // every thread has read s_wagg and holds its elements in registers: the staging arrays are free
-    u32* s_osuf = reinterpret_cast<u32*>(s_key); // [TILE] survivors of the tile, compacted
-    u32* s_ogid = s_osuf + TILE;                 // [TILE] their group ids
-    u32* s_oprim = s_suf;                        // [TILE / 2] first rank of each group of the tile
-    u32* s_ostart = s_suf + TILE / 2;            // [TILE / 2] and its start in the active list
-
     u64 rec[ITEMS]; // (position << 32 | rank) records of the thread's elements (deferred rank update)
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
@@ -237,7 +303,6 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
         a.gprim_out[tile_rh + i] = s_oprim[i];
         a.gstart_out[tile_rh + i] = s_ostart[i];
     }
-#undef CSA_PAD
 }
 
 // Exclusive combination of the tile aggregates (max, max, sum, sum) over the tiles of one slab: workgroup s handles
