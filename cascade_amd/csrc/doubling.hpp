@@ -755,41 +755,52 @@ __global__ __launch_bounds__(BLOCK) void apply_small_kernel(ApplySmallArgs a)
 {
     constexpr int TILE = BLOCK * ITEMS;
     constexpr int WAVES = BLOCK / WAVE;
-    // one pad word per ITEMS elements keeps the blocked accesses (stride ITEMS) off a single LDS bank
-    constexpr int PADDED = TILE + 2 + (TILE + 2) / ITEMS + 1;
-    __shared__ u32 s_nr[PADDED];
-    __shared__ u32 s_x[PADDED];
-#define CSA_PADI(q) ((q) + (q) / ITEMS)
     __shared__ u32 s_w[WAVES][2];
     const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
     const u32 tile = blockIdx.x;
     const u64 tile_base = (u64)tile * TILE;
     const u32 m = a.m;
-    // striped loads; s_nr[q] holds place tile_base + q - 1
-#pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-        const u32 q = j * BLOCK + t;
-        const u64 c = tile_base + q;
-        s_nr[CSA_PADI(q + 1)] = c < m ? a.nr[c] : 0u;
-        s_x[CSA_PADI(q)] = c < m ? a.sufs[c] : 0u;
-    }
-    if (t == 0)
-        s_nr[CSA_PADI(0)] = tile_base >= 1 ? a.nr[tile_base - 1] : 0u;
-    if (t == 1)
-        s_nr[CSA_PADI(TILE + 1)] = tile_base + TILE < m ? a.nr[tile_base + TILE] : 0u;
-    __syncthreads();
-    // blocked: thread t owns places tile_base + t * ITEMS + k
+    // blocked: thread t owns places tile_base + t * ITEMS + k and reads them, with the refined ranks of the two places
+    // next to them, straight from the lists (whole 16-byte loads where the tile is full)
     const u64 base = tile_base + (u64)t * ITEMS;
+    u32 nrw[ITEMS + 2]; // places base - 1 .. base + ITEMS
+    u32 xs[ITEMS];
+    if (ITEMS % 4 == 0 && base + ITEMS <= m) {
+        const uint4* n4 = reinterpret_cast<const uint4*>(a.nr + base); // base is a multiple of ITEMS
+        const uint4* x4 = reinterpret_cast<const uint4*>(a.sufs + base);
+#pragma unroll
+        for (int k = 0; k < ITEMS; k += 4) {
+            const uint4 v = n4[k / 4], xv = x4[k / 4];
+            nrw[k + 1] = v.x;
+            nrw[k + 2] = v.y;
+            nrw[k + 3] = v.z;
+            nrw[k + 4] = v.w;
+            xs[k] = xv.x;
+            xs[k + 1] = xv.y;
+            xs[k + 2] = xv.z;
+            xs[k + 3] = xv.w;
+        }
+        nrw[0] = base >= 1 ? a.nr[base - 1] : 0u;
+        nrw[ITEMS + 1] = base + ITEMS < m ? a.nr[base + ITEMS] : 0u;
+    } else {
+#pragma unroll
+        for (int k = 0; k < ITEMS + 2; ++k) {
+            const u64 c = base + k; // place c - 1
+            nrw[k] = (c >= 1 && c - 1 < m) ? a.nr[c - 1] : 0u;
+        }
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k)
+            xs[k] = base + k < m ? a.sufs[base + k] : 0u;
+    }
     u32 flags = 0; // 2 bits per item: bit 0 survivor, bit 1 head of a new group
     u32 lsurv = 0, lhead = 0;
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         const u64 c = base + k;
         if (c < m) {
-            const u32 q = t * ITEMS + k + 1;
-            const u32 me = s_nr[CSA_PADI(q)] & 0x7FFFFFFFu;
-            const bool head = c == 0 || (s_nr[CSA_PADI(q - 1)] & 0x7FFFFFFFu) != me;
-            const bool last = c + 1 == m || (s_nr[CSA_PADI(q + 1)] & 0x7FFFFFFFu) != me;
+            const u32 me = nrw[k + 1] & 0x7FFFFFFFu;
+            const bool head = c == 0 || (nrw[k] & 0x7FFFFFFFu) != me;
+            const bool last = c + 1 == m || (nrw[k + 2] & 0x7FFFFFFFu) != me;
             const bool surv = !(head && last);
             flags |= (surv ? 1u : 0u) << (2 * k);
             flags |= ((head && surv) ? 2u : 0u) << (2 * k);
@@ -825,8 +836,7 @@ __global__ __launch_bounds__(BLOCK) void apply_small_kernel(ApplySmallArgs a)
         const u64 c = base + k;
         if (c >= m)
             continue;
-        const u32 q = t * ITEMS + k;
-        const u32 word = s_nr[CSA_PADI(q + 1)], nr = word & 0x7FFFFFFFu, x = s_x[CSA_PADI(q)];
+        const u32 word = nrw[k + 1], nr = word & 0x7FFFFFFFu, x = xs[k];
         const u32 f = (flags >> (2 * k)) & 3u;
         if (nr >= a.n || x >= a.n) {
             atomicExch(a.err, DEV_ERR_RERANK_RANGE);
@@ -850,7 +860,6 @@ __global__ __launch_bounds__(BLOCK) void apply_small_kernel(ApplySmallArgs a)
         }
     }
 }
-#undef CSA_PADI
 
 // Brings the radix-sorted members of the large groups back into the sorted active list, in the (suffix, refined
 // rank) form of the small groups: the k-th sorted member of group g goes to place gstart[g] + (k - index of g's first
