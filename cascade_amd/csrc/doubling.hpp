@@ -22,6 +22,38 @@ namespace csa {
 
 constexpr u32 NO_RANK = 0xFFFFFFFFu; // ranks are below 2^31
 
+// The tiles of a rank step are scanned in RERANK_SLABS slabs (rerank_scan_kernel): a tile's prefix is its prefix inside
+// its slab combined with the totals (max, max, sum, sum, -) of the slabs before. One slab per lane: a wave fetches the
+// totals in one round trip and reduces them, instead of walking them one after the other (up to 63 dependent loads
+// at the head of every workgroup of kernels that live on latency). Call with all 64 lanes; the same values return in each.
+constexpr u32 RERANK_SLABS = 64;
+static_assert(RERANK_SLABS == WAVE, "one slab total per lane");
+
+struct SlabPrefix {
+    u32 max0, max1, sum2, sum3;
+};
+
+__device__ __forceinline__ SlabPrefix slabs_before(const u32* __restrict__ slab_total, u32 slabs_before_mine)
+{
+    const u32 lane = threadIdx.x & 63u;
+    SlabPrefix p = {0u, 0u, 0u, 0u};
+    if (lane < slabs_before_mine) {
+        p.max0 = slab_total[lane * 5 + 0];
+        p.max1 = slab_total[lane * 5 + 1];
+        p.sum2 = slab_total[lane * 5 + 2];
+        p.sum3 = slab_total[lane * 5 + 3];
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const u32 o0 = __shfl_xor(p.max0, o), o1 = __shfl_xor(p.max1, o);
+        p.max0 = p.max0 > o0 ? p.max0 : o0;
+        p.max1 = p.max1 > o1 ? p.max1 : o1;
+        p.sum2 += __shfl_xor(p.sum2, o);
+        p.sum3 += __shfl_xor(p.sum3, o);
+    }
+    return p;
+}
+
 struct RerankArgs {
     const u64* keys;
     const u32* sufs;
@@ -235,12 +267,10 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
     // prefix of the tile = totals of the slabs before its slab, combined with its prefix inside the slab
     u32 pre_a = a.tile_prefix[(u64)tile * 4 + 0];
     u32 tile_rc = a.tile_prefix[(u64)tile * 4 + 2], tile_rh = a.tile_prefix[(u64)tile * 4 + 3];
-    for (u32 sl = 0; sl < tile / a.slab; ++sl) {
-        const u32 sa_ = a.slab_total[sl * 5 + 0];
-        pre_a = pre_a > sa_ ? pre_a : sa_;
-        tile_rc += a.slab_total[sl * 5 + 2];
-        tile_rh += a.slab_total[sl * 5 + 3];
-    }
+    const SlabPrefix sp = slabs_before(a.slab_total, tile / a.slab);
+    pre_a = pre_a > sp.max0 ? pre_a : sp.max0;
+    tile_rc += sp.sum2;
+    tile_rh += sp.sum3;
     if (t == 0 && tile_base + TILE >= m) // the last tile knows the totals
         a.gstart_out[tile_rh + tile_total_heads] = tile_rc + tile_total_surv; // gstart[groups] = survivors
     u32 ra = xa > pre_a ? xa : pre_a;
@@ -308,7 +338,6 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
 // Exclusive combination of the tile aggregates (max, max, sum, sum) over the tiles of one slab: workgroup s handles
 // tiles [s * slab, (s + 1) * slab) and writes each tile's prefix relative to the slab start plus the slab's total.
 // The applying pass adds the totals of the slabs before its own (at most RERANK_SLABS of them).
-constexpr u32 RERANK_SLABS = 64;
 
 __global__ __launch_bounds__(1024) void rerank_scan_kernel(const u32* __restrict__ tile_agg, u32* __restrict__ tile_prefix,
                                                            u32 tiles, u32 slab, u32* __restrict__ slab_total,
@@ -825,10 +854,9 @@ __global__ __launch_bounds__(BLOCK) void apply_small_kernel(ApplySmallArgs a)
         tot_h += s_w[ww][1];
     }
     u32 tile_rc = a.tile_prefix[(u64)tile * 4 + 2], tile_rh = a.tile_prefix[(u64)tile * 4 + 3];
-    for (u32 sl = 0; sl < tile / a.slab; ++sl) {
-        tile_rc += a.slab_total[sl * 5 + 2];
-        tile_rh += a.slab_total[sl * 5 + 3];
-    }
+    const SlabPrefix sp = slabs_before(a.slab_total, tile / a.slab);
+    tile_rc += sp.sum2;
+    tile_rh += sp.sum3;
     if (t == 0 && tile_base + TILE >= m)
         a.gstart_out[tile_rh + tot_h] = tile_rc + tot_s; // gstart[groups] = survivors
 #pragma unroll
@@ -947,11 +975,9 @@ __global__ __launch_bounds__(BLOCK) void place_big_kernel(PlaceArgs a)
     }
     // prefix of the tile = totals of the slabs before its slab, combined with its prefix inside the slab
     u32 pre_g = a.tile_prefix[(u64)tile * 4 + 0], pre_k = a.tile_prefix[(u64)tile * 4 + 1];
-    for (u32 sl = 0; sl < tile / a.slab; ++sl) {
-        const u32 sg = a.slab_total[sl * 5 + 0], sk = a.slab_total[sl * 5 + 1];
-        pre_g = pre_g > sg ? pre_g : sg;
-        pre_k = pre_k > sk ? pre_k : sk;
-    }
+    const SlabPrefix sp = slabs_before(a.slab_total, tile / a.slab);
+    pre_g = pre_g > sp.max0 ? pre_g : sp.max0;
+    pre_k = pre_k > sp.max1 ? pre_k : sp.max1;
     u32 ghead = xg > pre_g ? xg : pre_g;
     u32 khead = xk > pre_k ? xk : pre_k;
 #pragma unroll

@@ -178,16 +178,11 @@ __global__ __launch_bounds__(STEP_BLOCK) void step_rank_kernel(StepRankArgs a)
     }
     u32 pre_a = a.tile_prefix[(u64)tile * 4 + 0], pre_b = a.tile_prefix[(u64)tile * 4 + 1];
     u32 pre_c = a.tile_prefix[(u64)tile * 4 + 2];
-    u32 total_active = 0;
-    for (u32 sl = 0; sl < a.slabs; ++sl) {
-        if (sl < tile / a.slab) {
-            const u32 sa_ = a.slab_total[sl * 5 + 0], sb_ = a.slab_total[sl * 5 + 1];
-            pre_a = pre_a > sa_ ? pre_a : sa_;
-            pre_b = pre_b > sb_ ? pre_b : sb_;
-            pre_c += a.slab_total[sl * 5 + 2];
-        }
-        total_active += a.slab_total[sl * 5 + 2];
-    }
+    const SlabPrefix sp = slabs_before(a.slab_total, tile / a.slab);
+    pre_a = pre_a > sp.max0 ? pre_a : sp.max0;
+    pre_b = pre_b > sp.max1 ? pre_b : sp.max1;
+    pre_c += sp.sum2;
+    const u32 total_active = slabs_before(a.slab_total, a.slabs).sum2;
     if (tile == 0 && t == 0)
         *a.active_out = total_active;
     u32 ra = xa > pre_a ? xa : pre_a, rb = xb > pre_b ? xb : pre_b;
