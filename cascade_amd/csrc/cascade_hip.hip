@@ -89,11 +89,14 @@ constexpr int RANK_TILE = RANK_BLOCK * RANK_ITEMS;
 #ifndef CSA_SMALL_AVG_LIMIT
 #define CSA_SMALL_AVG_LIMIT 16
 #endif
+// tile of the small-group kernel and of the counting / applying kernels behind it (measured per sort of the 1B-token
+// workload with 16-byte loads in the applying kernel: 256 x 8 109.4 ms, 256 x 4 106.5, 512 x 4 106.2, 1024 x 4 106.7,
+// 512 x 2 106.3, 512 x 8 108.8, 128 x 8 110.4)
 #ifndef CSA_SMALL_BLOCK
-#define CSA_SMALL_BLOCK 256
+#define CSA_SMALL_BLOCK 512
 #endif
 #ifndef CSA_SMALL_ITEMS
-#define CSA_SMALL_ITEMS 8
+#define CSA_SMALL_ITEMS 4
 #endif
 constexpr int SMALL_BLOCK = CSA_SMALL_BLOCK;
 constexpr int SMALL_ITEMS = CSA_SMALL_ITEMS;
