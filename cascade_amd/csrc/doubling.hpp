@@ -706,30 +706,39 @@ __global__ __launch_bounds__(BLOCK) void count_ranks_kernel(const u32* __restric
 {
     constexpr int TILE = BLOCK * ITEMS;
     constexpr int WAVES = BLOCK / WAVE;
-    __shared__ u32 s_nr[TILE + 2];
     __shared__ u32 s_w[WAVES];
     const u32 t = threadIdx.x;
-    const u64 tile_base = (u64)blockIdx.x * TILE;
+    // blocked: thread t owns places base .. base + ITEMS - 1 and reads them, with the two places next to them, straight
+    // from the list (whole 16-byte loads where they all exist)
+    const u64 base = (u64)blockIdx.x * TILE + (u64)t * ITEMS;
+    u32 nrw[ITEMS + 2]; // places base - 1 .. base + ITEMS
+    if (ITEMS % 4 == 0 && base + ITEMS <= m) {
+        const uint4* n4 = reinterpret_cast<const uint4*>(nr + base); // base is a multiple of ITEMS
 #pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-        const u32 q = j * BLOCK + t;
-        const u64 c = tile_base + q;
-        s_nr[q + 1] = c < m ? nr[c] : 0u;
+        for (int k = 0; k < ITEMS; k += 4) {
+            const uint4 v = n4[k / 4];
+            nrw[k + 1] = v.x;
+            nrw[k + 2] = v.y;
+            nrw[k + 3] = v.z;
+            nrw[k + 4] = v.w;
+        }
+        nrw[0] = base >= 1 ? nr[base - 1] : 0u;
+        nrw[ITEMS + 1] = base + ITEMS < m ? nr[base + ITEMS] : 0u;
+    } else {
+#pragma unroll
+        for (int k = 0; k < ITEMS + 2; ++k) {
+            const u64 c = base + k; // place c - 1
+            nrw[k] = (c >= 1 && c - 1 < m) ? nr[c - 1] : 0u;
+        }
     }
-    if (t == 0)
-        s_nr[0] = tile_base >= 1 ? nr[tile_base - 1] : 0u;
-    if (t == 1)
-        s_nr[TILE + 1] = tile_base + TILE < m ? nr[tile_base + TILE] : 0u;
-    __syncthreads();
     u32 c_surv = 0, c_head = 0, c_chg = 0;
 #pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-        const u32 q = j * BLOCK + t + 1; // striped: neighbouring lanes, neighbouring LDS words
-        const u64 c = tile_base + q - 1;
+    for (int k = 0; k < ITEMS; ++k) {
+        const u64 c = base + k;
         if (c < m) {
-            const u32 word = s_nr[q], me = word & 0x7FFFFFFFu;
-            const bool head = c == 0 || (s_nr[q - 1] & 0x7FFFFFFFu) != me;
-            const bool last = c + 1 == m || (s_nr[q + 1] & 0x7FFFFFFFu) != me;
+            const u32 word = nrw[k + 1], me = word & 0x7FFFFFFFu;
+            const bool head = c == 0 || (nrw[k] & 0x7FFFFFFFu) != me;
+            const bool last = c + 1 == m || (nrw[k + 2] & 0x7FFFFFFFu) != me;
             const bool surv = !(head && last);
             c_surv += surv ? 1u : 0u;
             c_head += (head && surv) ? 1u : 0u;
