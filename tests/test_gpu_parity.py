@@ -20,18 +20,24 @@ def torch_mod():
     return torch
 
 
-@pytest.fixture(scope="module")
-def sorter(torch_mod):
+# Every test that sorts through these handles runs twice: with the default tile order of the radix passes (tiles numbered
+# by arrival) and with the XCD-chunked order a caller gets after csa_set_device_exclusive (the order the headline
+# benchmark figure is measured with). Both must give the oracle's bytes.
+TILE_ORDERS = pytest.mark.parametrize("exclusive", [False, True], ids=["tiles_by_arrival", "tiles_xcd_chunked"])
+
+
+@pytest.fixture(scope="module", params=[False, True], ids=["tiles_by_arrival", "tiles_xcd_chunked"])
+def sorter(torch_mod, request):
     from cascade_amd import PartitionSorter
-    s = PartitionSorter(1 << 22, key_words=1)
+    s = PartitionSorter(1 << 22, key_words=1, device_exclusive=request.param)
     yield s
     s.close()
 
 
-@pytest.fixture(scope="module")
-def sorter2(torch_mod):
+@pytest.fixture(scope="module", params=[False, True], ids=["tiles_by_arrival", "tiles_xcd_chunked"])
+def sorter2(torch_mod, request):
     from cascade_amd import PartitionSorter
-    s = PartitionSorter(1 << 21, key_words=2)
+    s = PartitionSorter(1 << 21, key_words=2, device_exclusive=request.param)
     yield s
     s.close()
 
@@ -230,16 +236,17 @@ def test_many_small_partitions_of_low_entropy(torch_mod):
             assert np.array_equal(got, oracle_lib.u64_to_sa40(sa)), (n, sigma)
 
 
+@TILE_ORDERS
 @pytest.mark.parametrize("config", [2, 3, 4, 5])
-def test_sixteen_million_symbols_pass_the_oracle_verifier(torch_mod, config):
+def test_sixteen_million_symbols_pass_the_oracle_verifier(torch_mod, config, exclusive):
     """Large enough for the bucketed rank update and many radix tiles; checked with the O(n) verifier of the
     oracle (pass = byte-equal to the reference's suffix array, which is unique) and with the device verifier."""
     from cascade_amd import PartitionSorter, workloads
     n = 1 << 24
     T = workloads.generate(config, n)
     d = to_dev(torch_mod, T)
-    with PartitionSorter(n, key_words=1) as s:
-        print(f"  sort config={config} n={n}", flush=True)
+    with PartitionSorter(n, key_words=1, device_exclusive=exclusive) as s:
+        print(f"  sort config={config} n={n} exclusive={exclusive}", flush=True)
         out = s.sort(d)
         torch_mod.cuda.synchronize()
         assert s.verify(d, out)
