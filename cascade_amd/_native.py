@@ -21,7 +21,7 @@ EXPORTS = (
     "csa_partition_id_bits", "csa_partition_ids_u16_dev", "csa_scatter_to_rank_order_dev", "csa_output_cut",
     "csa_stage_slab_u16_dev", "csa_count_messages_dev", "csa_message_offsets_dev", "csa_emit_messages_dev",
     "csa_join_messages_dev", "csa_join_messages_sorted_dev", "csa_sort_init_dev", "csa_sort_rerank_dev",
-    "csa_set_device_exclusive",
+    "csa_set_device_exclusive", "csa_radix_sort_pairs_static_dev",
 )
 
 
@@ -82,6 +82,8 @@ def load():
     lib.csa_pack_keys_u16_dev.argtypes = [vp, u64, i32, vp, vp]
     lib.csa_radix_sort_pairs_dev.restype = i32
     lib.csa_radix_sort_pairs_dev.argtypes = [vp, vp, vp, u64, i32, i32, vp]
+    lib.csa_radix_sort_pairs_static_dev.restype = i32
+    lib.csa_radix_sort_pairs_static_dev.argtypes = [vp, vp, u64, i32, i32, vp]
     lib.csa_verify_sa40_dev.restype = i32
     lib.csa_verify_sa40_dev.argtypes = [vp, vp, u64, u64, vp, vp, C.POINTER(i32)]
     lib.csa_last_error.restype = C.c_char_p

@@ -13,6 +13,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <vector>
 
 using namespace csa;
@@ -162,6 +163,32 @@ int bit_length(u64 v)
 
 } // namespace
 
+// ---- scratch of csa_radix_sort_pairs_static_dev, the one entry point that allocates nothing ----
+// One array per device, part of the code object: it exists from the moment the library is loaded until the process
+// ends. Host code never uses the name `scratch` as an address (on the host it is a stand-in, not device memory): the
+// address on the current device comes from hipGetSymbolAddress, once per device (static_scratch below), and everything
+// that needs the memory takes that pointer.
+namespace {
+constexpr u64 STATIC_SORT_MAX = CSA_STATIC_SORT_MAX_PAIRS;
+constexpr u64 STATIC_TILES = (STATIC_SORT_MAX + SORT_TILE - 1) / SORT_TILE;
+constexpr u64 STATIC_LB_TILE_WORDS = STATIC_TILES * RADIX_BINS;                                  // per pass
+constexpr u64 STATIC_LB_WORDS = STATIC_LB_TILE_WORDS + (STATIC_TILES / LB_GROUP + 1) * RADIX_BINS; // per pass, groups included
+constexpr u64 align256(u64 v) { return (v + 255u) & ~(u64)255u; }
+// layout: the ping-pong partners of the caller's arrays, then the control words, which every call clears
+constexpr u64 STATIC_OFF_KEYS = 0;
+constexpr u64 STATIC_OFF_VALS = align256(STATIC_OFF_KEYS + STATIC_SORT_MAX * sizeof(u64));
+constexpr u64 STATIC_OFF_CONTROL = align256(STATIC_OFF_VALS + STATIC_SORT_MAX * sizeof(u32));
+constexpr u64 STATIC_OFF_LOOKBACK = STATIC_OFF_CONTROL;
+constexpr u64 STATIC_OFF_GHIST = align256(STATIC_OFF_LOOKBACK + MAX_PASSES * STATIC_LB_WORDS * sizeof(u64));
+constexpr u64 STATIC_OFF_TICKETS = align256(STATIC_OFF_GHIST + MAX_PASSES * RADIX_BINS * sizeof(u32));
+constexpr u64 STATIC_OFF_ERR = align256(STATIC_OFF_TICKETS + MAX_PASSES * sizeof(u32));
+constexpr u64 STATIC_OFF_DIGIT_BASE = align256(STATIC_OFF_ERR + sizeof(u32)); // written before it is read: not cleared
+constexpr u64 STATIC_CONTROL_END = STATIC_OFF_DIGIT_BASE;
+constexpr u64 STATIC_SCRATCH_BYTES = align256(STATIC_OFF_DIGIT_BASE + MAX_PASSES * RADIX_BINS * sizeof(u32));
+} // namespace
+
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
 struct csa_handle {
     int device = 0;
     u64 cap = 0;
@@ -236,15 +263,23 @@ u32 hist_blocks(u64 items_per_block, u64 n)
     return (u32)(blocks ? blocks : 1);
 }
 
+// How the radix passes of a call number their tiles (radix_sort.hpp).
+struct TileOrder {
+    u32 order;     // TILES_BY_ARRIVAL or TILES_STATIC_CHUNKS
+    u32 xcd_chunk; // tiles of SORT_TILE pairs that one XCD takes in a row under TILES_STATIC_CHUNKS
+};
+
 // tile order of a pass over a.n pairs in tiles of `tile` pairs
-void set_tile_order(const csa_handle* h, OnesweepArgs& a, u32 tile)
+void set_tile_order(const TileOrder& o, OnesweepArgs& a, u32 tile)
 {
     a.tiles = (u32)(((u64)a.n + tile - 1) / tile);
-    a.order = h->tile_order;
+    a.order = o.order;
     // the chunk length is meant in tiles of SORT_TILE pairs: larger tiles, proportionally fewer per chunk
-    const u32 chunk = (u32)((u64)h->xcd_chunk * SORT_TILE / tile);
+    const u32 chunk = (u32)((u64)o.xcd_chunk * SORT_TILE / tile);
     a.xcd_chunk = chunk ? chunk : 1u;
 }
+
+TileOrder tile_order_of(const csa_handle* h) { return TileOrder{h->tile_order, h->xcd_chunk}; }
 
 bool wide_workgroups(const OnesweepArgs& a)
 {
@@ -252,9 +287,9 @@ bool wide_workgroups(const OnesweepArgs& a)
 }
 
 template <int SRC, int BLOCK, bool VALS>
-void launch_onesweep_shape(const csa_handle* h, OnesweepArgs& a, hipStream_t s)
+void launch_onesweep_shape(const TileOrder& o, OnesweepArgs& a, hipStream_t s)
 {
-    set_tile_order(h, a, BLOCK * SORT_ITEMS);
+    set_tile_order(o, a, BLOCK * SORT_ITEMS);
     if (a.shift >= 32)
         hipLaunchKernelGGL((onesweep_kernel<u64, BLOCK, SORT_ITEMS, SRC, 1, VALS>), dim3(a.tiles), dim3(BLOCK), 0, s, a);
     else
@@ -265,13 +300,14 @@ template <int SRC, bool VALS = true>
 void launch_onesweep(const csa_handle* h, OnesweepArgs& a, hipStream_t s)
 {
     if (wide_workgroups(a))
-        launch_onesweep_shape<SRC, SORT_WIDE_BLOCK, VALS>(h, a, s);
+        launch_onesweep_shape<SRC, SORT_WIDE_BLOCK, VALS>(tile_order_of(h), a, s);
     else
-        launch_onesweep_shape<SRC, SORT_BLOCK, VALS>(h, a, s);
+        launch_onesweep_shape<SRC, SORT_BLOCK, VALS>(tile_order_of(h), a, s);
 }
 
-void launch_onesweep32(const csa_handle* h, OnesweepArgs& a, hipStream_t s)
+void launch_onesweep32(const csa_handle* hh, OnesweepArgs& a, hipStream_t s)
 {
+    const TileOrder h = tile_order_of(hh);
     if (wide_workgroups(a)) {
         set_tile_order(h, a, SORT_WIDE_BLOCK * SORT32_ITEMS);
         hipLaunchKernelGGL((onesweep_kernel<u32, SORT_WIDE_BLOCK, SORT32_ITEMS, SRC_PAIRS, 0>), dim3(a.tiles), dim3(SORT_WIDE_BLOCK), 0, s, a);
@@ -1712,6 +1748,107 @@ int csa_radix_sort_pairs_dev(csa_handle* h, uint64_t* d_keys, uint32_t* d_vals, 
         HIP_TRY(hipMemcpyAsync(d_vals, h->idx[0], n * 4, hipMemcpyDeviceToDevice, L.stream));
     }
     return read_counts(L, nullptr);
+}
+
+extern "C++" {
+namespace {
+constexpr int STATIC_MAX_DEVICES = 64;
+std::mutex g_static_mutex;
+unsigned char* g_static_ptr[STATIC_MAX_DEVICES] = {}; // address of `scratch` on each device, asked for once per device
+
+// The current device's copy of `scratch`.
+int static_scratch(unsigned char** out)
+{
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= STATIC_MAX_DEVICES)
+        return fail(CSA_ERR_ARG, "csa_radix_sort_pairs_static_dev: device %d is beyond the %d devices this entry point keeps a scratch address for",
+                    dev, STATIC_MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (!g_static_ptr[dev]) {
+        void* p = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p)
+            return fail(CSA_ERR_HIP, "csa_radix_sort_pairs_static_dev: no address for the scratch array on device %d", dev);
+        g_static_ptr[dev] = static_cast<unsigned char*>(p);
+    }
+    *out = g_static_ptr[dev];
+    return CSA_OK;
+}
+} // namespace
+} // extern "C++"
+
+int csa_radix_sort_pairs_static_dev(uint64_t* d_keys, uint32_t* d_vals, uint64_t n, int begin_bit, int end_bit, void* stream)
+{
+    if (begin_bit < 0 || end_bit > 64 || begin_bit > end_bit)
+        return fail(CSA_ERR_ARG, "csa_radix_sort_pairs_static_dev: bad bit range [%d, %d)", begin_bit, end_bit);
+    if (n > STATIC_SORT_MAX)
+        return fail(CSA_ERR_TOO_LARGE, "csa_radix_sort_pairs_static_dev: %llu pairs exceed the %llu this entry point's fixed scratch holds "
+                    "(use csa_radix_sort_pairs_dev with a handle)", (unsigned long long)n, (unsigned long long)STATIC_SORT_MAX);
+    unsigned char* base = nullptr; // the device address of the scratch array: never the array's name from here on
+    int rc = static_scratch(&base);
+    if (rc)
+        return rc;
+    if (n == 0 || begin_bit == end_bit)
+        return CSA_OK;
+    if (!d_keys || !d_vals)
+        return fail(CSA_ERR_ARG, "csa_radix_sort_pairs_static_dev: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    u64* tmp_keys = reinterpret_cast<u64*>(base + STATIC_OFF_KEYS);
+    u32* tmp_vals = reinterpret_cast<u32*>(base + STATIC_OFF_VALS);
+    u64* lookback = reinterpret_cast<u64*>(base + STATIC_OFF_LOOKBACK);
+    u32* ghist = reinterpret_cast<u32*>(base + STATIC_OFF_GHIST);
+    u32* tickets = reinterpret_cast<u32*>(base + STATIC_OFF_TICKETS);
+    u32* err = reinterpret_cast<u32*>(base + STATIC_OFF_ERR);
+    u32* digit_base = reinterpret_cast<u32*>(base + STATIC_OFF_DIGIT_BASE);
+    // The array keeps what the last call left: look-back words, digit counts, tile tickets and the error word start at
+    // zero in every call (a fill kernel, not a memset node: the call may be recorded into a graph). With the words
+    // cleared the launch epoch can stay the same in every call and replay.
+    const u64 control_words = (STATIC_CONTROL_END - STATIC_OFF_CONTROL) / sizeof(u32);
+    hipLaunchKernelGGL(fill_u32_kernel, dim3((u32)((control_words + 255) / 256)), dim3(256), 0, s,
+                       reinterpret_cast<u32*>(base + STATIC_OFF_CONTROL), control_words, 0u);
+    const PassPlan plan = make_plan(begin_bit, end_bit);
+    HistArgs ha;
+    ha.keys = d_keys;
+    ha.vals = d_vals;
+    ha.text = nullptr;
+    ha.n = (u32)n;
+    ha.text_n = 0;
+    ha.word = 0;
+    ha.plan = plan;
+    ha.ghist = ghist;
+    hipLaunchKernelGGL(radix_hist_kernel, dim3(hist_blocks(256 * 16, n)), dim3(256), 0, s, ha);
+    hipLaunchKernelGGL(radix_scan_hist_kernel, dim3(1), dim3(256), 0, s, ghist, digit_base, plan.num_passes);
+    // every pass runs (skipping the passes whose digit is constant would need the counts on the host: a round trip)
+    const TileOrder by_arrival = {TILES_BY_ARRIVAL, XCD_CHUNK};
+    int where = 0; // 0: the pairs are in the caller's arrays, 1: in the scratch
+    for (int p = 0; p < plan.num_passes; ++p) {
+        OnesweepArgs a;
+        a.keys_in = where == 0 ? d_keys : tmp_keys;
+        a.vals_in = where == 0 ? d_vals : tmp_vals;
+        a.keys_out = where == 0 ? tmp_keys : d_keys;
+        a.vals_out = where == 0 ? tmp_vals : d_vals;
+        a.text = nullptr;
+        a.n = (u32)n;
+        a.text_n = 0;
+        a.tail = 0;
+        a.word = 0;
+        a.shift = plan.shift[p];
+        a.bits = plan.bits[p];
+        a.digit_base = digit_base + p * RADIX_BINS;
+        a.lookback = lookback + (u64)p * STATIC_LB_WORDS;
+        a.lookback_groups = a.lookback + STATIC_LB_TILE_WORDS;
+        a.ticket = tickets + p;
+        a.epoch = 1;
+        a.err = err;
+        launch_onesweep_shape<SRC_PAIRS, SORT_BLOCK, true>(by_arrival, a, s);
+        where ^= 1;
+    }
+    if (where)
+        hipLaunchKernelGGL(copy_pairs_kernel, dim3((u32)((n + 255) / 256)), dim3(256), 0, s, (const u64*)tmp_keys, (const u32*)tmp_vals,
+                           (u64)n, d_keys, d_vals);
+    HIP_TRY(hipGetLastError());
+    return CSA_OK;
 }
 
 int csa_verify_sa40_dev(csa_handle* h, const uint16_t* d_text, uint64_t n, uint64_t index_base,

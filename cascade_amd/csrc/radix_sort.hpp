@@ -441,4 +441,16 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
 #undef CSA_OPAQUE
 }
 
+// Sorted pairs that ended in the ping-pong partner go back to the caller's arrays (a kernel rather than a copy call,
+// so that a sort recorded into a graph consists of kernel launches only).
+__global__ __launch_bounds__(256) void copy_pairs_kernel(const u64* __restrict__ keys_in, const u32* __restrict__ vals_in, u64 n,
+                                                        u64* __restrict__ keys_out, u32* __restrict__ vals_out)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) {
+        keys_out[i] = keys_in[i];
+        vals_out[i] = vals_in[i];
+    }
+}
+
 } // namespace csa

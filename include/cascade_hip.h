@@ -121,6 +121,23 @@ int csa_pack_keys_u16_dev(const uint16_t* d_text, uint64_t n, int key_words, uin
 int csa_radix_sort_pairs_dev(csa_handle* h, uint64_t* d_keys, uint32_t* d_vals, uint64_t n, int begin_bit,
                              int end_bit, void* stream);
 
+/* The same sort for callers that cannot allocate (code recorded into a HIP graph, serving loops and harnesses that
+ * forbid hipMalloc): no handle, no hipMalloc / hipFree / allocating library routine, no host round trip. The call only
+ * enqueues kernels on the stream (no memset or copy nodes) and returns; the sorted pairs are in d_keys / d_vals when the
+ * stream has finished. Its scratch (the ping-pong partners of the two arrays, look-back words, digit counts) is a
+ * fixed array inside the library's code object, which every device that loads the library holds until the process
+ * ends: 8 * CSA_STATIC_SORT_MAX_PAIRS + 4 * CSA_STATIC_SORT_MAX_PAIRS bytes of pairs + 2.3 MB of control words, 14.3 MB
+ * in all. n > CSA_STATIC_SORT_MAX_PAIRS fails with CSA_ERR_TOO_LARGE. All calls on one device share that one array:
+ * calls that overlap on a device (two streams, two threads) race; serialise them. Every pass of the bit range runs
+ * (passes over a constant digit are not skipped: that needs the counts on the host). The stream's device must be the
+ * current one. The first call on a device looks the array's address up (hipGetSymbolAddress); make that call, with
+ * n = 0 if need be, before any stream capture begins.
+ * No counterpart in the reference (its sorts go through cub's workspace, allocated once by allocate_device_space). */
+#ifndef CSA_STATIC_SORT_MAX_PAIRS
+#define CSA_STATIC_SORT_MAX_PAIRS (1u << 20)
+#endif
+int csa_radix_sort_pairs_static_dev(uint64_t* d_keys, uint32_t* d_vals, uint64_t n, int begin_bit, int end_bit, void* stream);
+
 /* O(n) suffix-array check on the device: d_sa40 is a permutation of [index_base, index_base + n) and every
  * adjacent pair is in order (first symbols, then ranks of the successors; a successor past the end sorts
  * first). *ok = 1 if correct. Same rule as the reference's validator (test/end-to-end.cpp:13-80). */

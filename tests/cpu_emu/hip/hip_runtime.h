@@ -28,6 +28,7 @@
 #define __launch_bounds__(...)
 #define __restrict__
 #define __shared__ static
+#define __align__(n) __attribute__((aligned(n)))
 
 struct alignas(16) uint4 {
     unsigned x, y, z, w;
@@ -222,6 +223,10 @@ constexpr unsigned hipHostMallocDefault = 0;
 inline const char* hipGetErrorString(hipError_t e) { return e == hipSuccess ? "success" : "emulated failure"; }
 inline hipError_t hipGetLastError() { return hipSuccess; }
 inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
+// a __device__ array is an ordinary array here, so its name already is its address
+#define HIP_SYMBOL(x) (x)
+template <typename T>
+inline hipError_t hipGetSymbolAddress(void** p, T& symbol) { *p = &symbol; return hipSuccess; }
 enum hipDeviceAttribute_t { hipDeviceAttributeMultiprocessorCount = 63 };
 inline hipError_t hipDeviceGetAttribute(int* v, hipDeviceAttribute_t, int) { *v = 1; return hipSuccess; } // one "CU"
 inline hipError_t hipMalloc(void** p, size_t bytes)

@@ -131,6 +131,30 @@ def test_emulated_radix_sort_matches_stable_sort(emu):
     assert np.array_equal(k, wk) and np.array_equal(v, wv)
 
 
+def test_emulated_radix_sort_without_allocation_matches_the_one_with_a_handle(emu):
+    """csa_radix_sort_pairs_static_dev (fixed scratch inside the library, which keeps the last call's contents): two
+    calls in a row, the second smaller and over another bit range, each equal to csa_radix_sort_pairs_dev and to the
+    oracle's stable sort; sizes beyond the fixed scratch are refused."""
+    emu.csa_radix_sort_pairs_static_dev.restype = C.c_int
+    emu.csa_radix_sort_pairs_static_dev.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_int, C.c_int, C.c_void_p]
+    rng = np.random.default_rng(4)
+    h = C.c_void_p()
+    assert emu.csa_create(20000, 1, C.byref(h)) == 0
+    for n, b, e in ((17000, 0, 64), (3001, 5, 29), (1, 0, 64), (1024, 8, 24)):
+        keys = rng.integers(0, 1 << 63, n).astype(np.uint64) >> np.uint64(rng.integers(0, 40))
+        vals = rng.permutation(n).astype(np.uint32)
+        k0, v0 = keys.copy(), vals.copy()
+        assert emu.csa_radix_sort_pairs_dev(h, k0.ctypes.data, v0.ctypes.data, n, b, e, None) == 0
+        k1, v1 = keys.copy(), vals.copy()
+        assert emu.csa_radix_sort_pairs_static_dev(k1.ctypes.data, v1.ctypes.data, n, b, e, None) == 0
+        wk, wv = oracle_lib.stable_sort_pairs(keys, vals, b, e)
+        assert np.array_equal(k1, k0) and np.array_equal(v1, v0), (n, b, e)
+        assert np.array_equal(k1, wk) and np.array_equal(v1, wv), (n, b, e)
+    emu.csa_destroy(h)
+    big = np.zeros(20001, dtype=np.uint64)
+    assert emu.csa_radix_sort_pairs_static_dev(big.ctypes.data, big.ctypes.data, 20001, 0, 64, None) == -2
+
+
 @pytest.mark.parametrize("words,p", [(1, 1), (1, 3), (2, 17), (3, 300), (4, 5)])
 def test_emulated_partition_ids_match_the_oracle(emu, words, p):
     rng = np.random.default_rng(words * 1000 + p)
