@@ -288,6 +288,40 @@ def bench_next_rows(args):
         res["roofline"]["bound"] = "pcie (not an HBM figure: 2 B up + 5 B down per suffix over the host link)"
         res["roofline"]["peak"] = None
         res["roofline"]["frac"] = None
+    elif args.row == "pipeline":
+        # The same job inside the library: csa_sort_partitions_u16 takes the list of pinned host texts and returns the suffix
+        # arrays in pinned host memory; one handle, two device buffer sets, an upload and a download thread beside the
+        # calling one (the reference's dispatcher overlap, src/GPU_SACA.cu:1539-1589, without Python in the loop).
+        from cascade_amd import sort_partitions
+        parts = min(p, 12)
+        n = args.n if args.n is not None else 1 << 26
+        T = workloads.generate(args.config, parts * n)
+        h_text = torch.from_numpy(T.view(np.int16)).reshape(parts, n).pin_memory()
+        h_out = torch.empty((parts, 5 * n), dtype=torch.uint8).pin_memory()
+        ins = [h_text[q].numpy().view(np.uint16) for q in range(parts)]
+        outs = [h_out[q].numpy() for q in range(parts)]
+
+        def run():
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            _, stats = sort_partitions(ins, key_words=1, out=outs)
+            return (time.perf_counter() - t0) * 1e3, sum(st["ms_total"] for st in stats)
+        for _ in range(args.warmup):
+            run()
+        ms, in_hbm = min(run() for _ in range(args.steps))
+        sorter = PartitionSorter(n)
+        ok = True
+        for q in (0, parts // 2, parts - 1):
+            ok = ok and sorter.verify(h_text[q].to(dev), h_out[q].to(dev))
+        sorter.close()
+        pcie_bytes = parts * n * 7
+        res = _row_result("suffixes sorted/sec at 1 GPU, host buffers in and out", workloads.NAMES[args.config], parts * n, ms,
+                          "whole job inside csa_sort_partitions_u16: handle set-up, upload, partition sorts, download on three streams", pcie_bytes,
+                          {"texts": parts, "n_each": n, "ms_in_hbm_sorts_only": round(in_hbm, 2),
+                           "pcie_GBps_both_ways": round(pcie_bytes / ms / 1e6, 1)}, args.steps, args.warmup, ok)
+        res["roofline"]["bound"] = "pcie (not an HBM figure: 2 B up + 5 B down per suffix over the host link)"
+        res["roofline"]["peak"] = None
+        res["roofline"]["frac"] = None
     elif args.row in ("step_init", "step_rerank"):
         # one partition step under the exchange scheme: everything the reference does between the upload of a partition's
         # slabs and their download (src/GPU_SACA.cu:1112-1331 / 1715-1995). The synthetic partition: n suffixes of the
@@ -381,7 +415,7 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=1 << 26, help="symbols of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--generations", action="store_true", help="print the per-generation table to stderr")
-    ap.add_argument("--row", default="sort", choices=["sort", "partition_ids", "stage_slab", "messages", "join", "scatter", "step_init", "step_rerank", "overlap"],
+    ap.add_argument("--row", default="sort", choices=["sort", "partition_ids", "stage_slab", "messages", "join", "scatter", "step_init", "step_rerank", "overlap", "pipeline"],
                     help="which step to measure: the partition sort (the headline, default) or one of the steps around it")
     ap.add_argument("--shared-device", action="store_true",
                     help="measure the headline with the default tile order (safe next to other launches) only")

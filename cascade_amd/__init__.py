@@ -4,6 +4,6 @@ The compute lives in libcascade_hip.so (hand-written HIP, include/cascade_hip.h)
 host-side mirror of the reference's builder interface for that one path.
 """
 from . import _native, workloads
-from .gpu_saca import GPU_SACA, PartitionSorter, output_cut, pack_keys, partition_ids, sort_partition, stage_slab
+from .gpu_saca import GPU_SACA, PartitionSorter, output_cut, pack_keys, partition_ids, sort_partition, sort_partitions, stage_slab
 
-__all__ = ["GPU_SACA", "PartitionSorter", "output_cut", "pack_keys", "partition_ids", "sort_partition", "stage_slab", "workloads", "_native"]
+__all__ = ["GPU_SACA", "PartitionSorter", "output_cut", "pack_keys", "partition_ids", "sort_partition", "sort_partitions", "stage_slab", "workloads", "_native"]

@@ -21,8 +21,18 @@ EXPORTS = (
     "csa_partition_id_bits", "csa_partition_ids_u16_dev", "csa_scatter_to_rank_order_dev", "csa_output_cut",
     "csa_stage_slab_u16_dev", "csa_count_messages_dev", "csa_message_offsets_dev", "csa_emit_messages_dev",
     "csa_join_messages_dev", "csa_join_messages_sorted_dev", "csa_sort_init_dev", "csa_sort_rerank_dev",
-    "csa_set_device_exclusive", "csa_radix_sort_pairs_static_dev",
+    "csa_set_device_exclusive", "csa_radix_sort_pairs_static_dev", "csa_enable_profile_ranges",
+    "csa_slab_bytes_per_suffix", "csa_sort_init_slabs", "csa_sort_rerank_slabs", "csa_scatter_slabs", "csa_sort_partitions_u16",
 )
+
+
+class CsaSlab(C.Structure):
+    """csa_slab of include/cascade_hip.h: one pinned host slab of a partition."""
+    _fields_ = [
+        ("key", C.c_void_p), ("suf", C.c_void_p), ("beta", C.c_void_p), ("msg_target", C.c_void_p), ("msg_rank", C.c_void_p),
+        ("off", C.c_uint64), ("size", C.c_uint64), ("inbox_off", C.c_uint32), ("inbox_sz", C.c_uint32),
+        ("outbox_off", C.c_uint32), ("outbox_sz", C.c_uint32),
+    ]
 
 
 class CsaStats(C.Structure):
@@ -78,6 +88,8 @@ def load():
     lib.csa_sort_partition_u16_dev.argtypes = [vp, vp, u64, u64, vp, vp, u32, C.POINTER(CsaStats)]
     lib.csa_sort_partition_u16.restype = i32
     lib.csa_sort_partition_u16.argtypes = [vp, u64, i32, vp, C.POINTER(CsaStats)]
+    lib.csa_sort_partitions_u16.restype = i32
+    lib.csa_sort_partitions_u16.argtypes = [u32, vp, vp, vp, i32, vp, C.POINTER(CsaStats)]
     lib.csa_pack_keys_u16_dev.restype = i32
     lib.csa_pack_keys_u16_dev.argtypes = [vp, u64, i32, vp, vp]
     lib.csa_radix_sort_pairs_dev.restype = i32
@@ -110,6 +122,16 @@ def load():
     lib.csa_sort_init_dev.argtypes = [vp, vp, i32, vp, vp, u64, u32, vp, vp, vp, vp, vp, vp, vp]
     lib.csa_sort_rerank_dev.restype = i32
     lib.csa_sort_rerank_dev.argtypes = [vp, vp, vp, vp, u64, vp, vp, u32, u64, u32, vp, vp, vp, vp, vp, vp, vp]
+    lib.csa_enable_profile_ranges.restype = i32
+    lib.csa_enable_profile_ranges.argtypes = [i32]
+    lib.csa_slab_bytes_per_suffix.restype = u64
+    lib.csa_slab_bytes_per_suffix.argtypes = [i32]
+    lib.csa_sort_init_slabs.restype = i32
+    lib.csa_sort_init_slabs.argtypes = [vp, C.POINTER(CsaSlab), u32, u64, i32, u32, u64, vp, vp, vp]
+    lib.csa_sort_rerank_slabs.restype = i32
+    lib.csa_sort_rerank_slabs.argtypes = [vp, C.POINTER(CsaSlab), u32, u64, u64, u64, u32, u64, vp, vp, vp]
+    lib.csa_scatter_slabs.restype = i32
+    lib.csa_scatter_slabs.argtypes = [vp, C.POINTER(CsaSlab), u32, u64, u64, u64, vp]
     lib.csa_output_cut.restype = None
     lib.csa_output_cut.argtypes = [u64, u64, u64, u64, u64, C.POINTER(u64 * 6)]
     _lib = lib

@@ -20,8 +20,8 @@ HIPCC_FLAGS = [
     "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared", "-Wall",
     # packed FP32 instructions stay off (nothing here is floating point, the flag is policy for this target)
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    # the radix pass runs its tile body inside a loop of rounds: values the machine-level loop-invariant code motion
-    # hoists out of that loop stay live through the whole body and cost the kernel half of its occupancy
+    # machine-level loop-invariant code motion hoists values out of the kernels' unrolled item loops that then stay
+    # live through the whole body; without it the radix pass needs fewer vector registers
     "-mllvm", "-disable-machine-licm",
 ]
 

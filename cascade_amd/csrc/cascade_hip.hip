@@ -13,6 +13,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <dlfcn.h>
 #include <mutex>
 #include <vector>
 
@@ -37,6 +38,72 @@ int fail(int code, const char* fmt, ...)
         if (e_ != hipSuccess)                                                                          \
             return fail(CSA_ERR_HIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), __FILE__, __LINE__); \
     } while (0)
+
+// Named ranges for a profiler's timeline, one per partition step and per generation: the counterpart of the NVTX ranges
+// the reference opens under -DPROFILE (include/profile.hpp:19-80; PROFILE_SCOPE_FMT at src/GPU_SACA.cu:1114,1717,2004,2111).
+// The roctx library is looked up at run time when csa_enable_profile_ranges(1) asks for it, so the library neither
+// links against a profiler nor pays for ranges nobody reads.
+#ifndef HIPEMU
+struct ProfileRanges {
+    std::mutex mu;
+    bool tried = false;
+    int (*push)(const char*) = nullptr;
+    int (*pop)() = nullptr;
+    bool enabled = false;
+} g_ranges;
+
+int enable_ranges(bool on)
+{
+    std::lock_guard<std::mutex> lock(g_ranges.mu);
+    if (on && !g_ranges.tried) {
+        g_ranges.tried = true;
+        for (const char* name : {"librocprofiler-sdk-roctx.so", "librocprofiler-sdk-roctx.so.1", "libroctx64.so", "libroctx64.so.4"}) {
+            if (void* lib = dlopen(name, RTLD_NOW | RTLD_GLOBAL)) {
+                g_ranges.push = reinterpret_cast<int (*)(const char*)>(dlsym(lib, "roctxRangePushA"));
+                g_ranges.pop = reinterpret_cast<int (*)()>(dlsym(lib, "roctxRangePop"));
+                if (g_ranges.push && g_ranges.pop)
+                    break;
+                g_ranges.push = nullptr;
+                g_ranges.pop = nullptr;
+            }
+        }
+    }
+    g_ranges.enabled = on && g_ranges.push && g_ranges.pop;
+    return on && !g_ranges.enabled ? 1 : 0;
+}
+#else
+struct ProfileRanges {
+    int (*push)(const char*) = nullptr;
+    int (*pop)() = nullptr;
+    bool enabled = false;
+} g_ranges;
+int enable_ranges(bool) { return 1; }
+#endif
+
+struct RangeScope {
+    bool open = false;
+    explicit RangeScope(const char* fmt, ...)
+    {
+        if (!g_ranges.enabled)
+            return;
+        char name[128];
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(name, sizeof(name), fmt, ap);
+        va_end(ap);
+        g_ranges.push(name);
+        open = true;
+    }
+    void close()
+    {
+        if (open)
+            g_ranges.pop();
+        open = false;
+    }
+    ~RangeScope() { close(); }
+    RangeScope(const RangeScope&) = delete;
+    RangeScope& operator=(const RangeScope&) = delete;
+};
 
 // tile shape of the radix pass; overridable at build time for tuning runs
 #ifndef CSA_SORT_BLOCK
@@ -189,6 +256,11 @@ constexpr u64 STATIC_SCRATCH_BYTES = align256(STATIC_OFF_DIGIT_BASE + MAX_PASSES
 
 static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
 
+namespace {
+struct SlabArena; // device image of a partition's host slabs (slab_entries.hpp)
+void free_slab_arena(csa_handle* h);
+}
+
 struct csa_handle {
     int device = 0;
     u64 cap = 0;
@@ -217,6 +289,7 @@ struct csa_handle {
     u32 xcd_chunk = XCD_CHUNK;                   // tiles of a radix pass that one XCD takes in a row under TILES_STATIC_CHUNKS
     u32 defer_min = DEFER_MIN; // lists at least this long use the bucketed rank update (env CASCADE_DEFER_MIN overrides)
     u64* step64[2] = {nullptr, nullptr}; // two more 8-byte arrays of the capacity, for the per-generation partition steps
+    SlabArena* slab_arena = nullptr;     // allocated by the first call of a slab-shaped entry
     u32 window_min_changed = WINDOW_MIN_CHANGED; // env CASCADE_WINDOW_MIN_CHANGED overrides (0xFFFFFFFF: never)
     std::vector<hipEvent_t> events;
     hipEvent_t ev_gen[CSA_MAX_GENERATIONS + 2] = {};
@@ -710,10 +783,12 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
         ++folded;
     const u32 tail = n < ell ? n : ell;
 
+    RangeScope range_sort("sort_partition n=%u", n);
     HIP_TRY(hipMemsetAsync(h->counts, 0, 4 * sizeof(u32), s));
     HIP_TRY(hipEventRecord(h->ev_gen[0], s));
 
     // ---- generation 0: sort every suffix by its K-gram key, ties of tail suffixes broken by length ----
+    RangeScope range_gen0("generation 0 m=%u", n);
     int passes = 0, p1 = 0, in_out = 0;
     const PassPlan full = make_plan(0, 64);
     u64* K[2] = {h->key[0], h->key[1]};
@@ -758,6 +833,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
                                     reinterpret_cast<u32*>(bkey[1]) + h->cap};
     u32 m = 0, groups = 0, big = 0;
     rc = rerank_step(L, ra, defer_buf, &m, &groups, &st->rank_update[0]);
+    range_gen0.close();
     if (rc)
         return rc;
     st->passes[0] = passes;
@@ -778,6 +854,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
         st->active[gen] = m;
         st->groups[gen] = groups;
         const u32 m_in = m;
+        RangeScope range_g("generation %d m=%u groups=%u", gen, m, groups);
         const RankTables r = rank_tables(h, m_in, SMALL_TILE);
         u32* nr_list = reinterpret_cast<u32*>(key_out); // refined rank at every place of the sorted list
         // 1. gather rank[x + h]; small groups are sorted and ranked inside their tile, members of large groups set aside
@@ -1604,6 +1681,7 @@ void csa_destroy(csa_handle* h)
 {
     if (!h)
         return;
+    free_slab_arena(h);
     for (int i = 0; i < 3; ++i)
         (void)hipFree(h->key[i]);
     for (int i = 0; i < 5; ++i)
@@ -1664,39 +1742,6 @@ int csa_sort_partition_u16_dev(csa_handle* h, const uint16_t* d_text, uint64_t n
     L.flags = flags;
     L.stats = st;
     return sort_partition(L, d_text, n, index_base, d_sa40);
-}
-
-int csa_sort_partition_u16(const uint16_t* h_text, uint64_t n, int key_words, uint8_t* h_sa40, csa_stats* stats)
-{
-    if (n > CSA_MAX_PART_SZ)
-        return fail(CSA_ERR_TOO_LARGE, "csa_sort_partition_u16: %llu suffixes exceed the partition limit %llu",
-                    (unsigned long long)n, (unsigned long long)CSA_MAX_PART_SZ);
-    if (n > 0 && (!h_text || !h_sa40))
-        return fail(CSA_ERR_ARG, "csa_sort_partition_u16: null text or output pointer");
-    csa_handle* h = nullptr;
-    int rc = csa_create(n, key_words, &h);
-    if (rc)
-        return rc;
-    uint16_t* d_text = nullptr;
-    uint8_t* d_sa = nullptr;
-    hipError_t e = hipMalloc((void**)&d_text, n ? n * 2 : 4);
-    if (e == hipSuccess)
-        e = hipMalloc((void**)&d_sa, n ? n * 5 : 4);
-    if (e == hipSuccess && n)
-        e = hipMemcpy(d_text, h_text, n * 2, hipMemcpyHostToDevice);
-    if (e != hipSuccess)
-        rc = fail(CSA_ERR_HIP, "csa_sort_partition_u16: %s", hipGetErrorString(e));
-    if (!rc)
-        rc = csa_sort_partition_u16_dev(h, d_text, n, 0, d_sa, nullptr, 0, stats);
-    if (!rc && n) {
-        e = hipMemcpy(h_sa40, d_sa, n * 5, hipMemcpyDeviceToHost);
-        if (e != hipSuccess)
-            rc = fail(CSA_ERR_HIP, "csa_sort_partition_u16: %s", hipGetErrorString(e));
-    }
-    (void)hipFree(d_text);
-    (void)hipFree(d_sa);
-    csa_destroy(h);
-    return rc;
 }
 
 int csa_pack_keys_u16_dev(const uint16_t* d_text, uint64_t n, int key_words, uint64_t* d_keys, void* stream)
@@ -1881,4 +1926,14 @@ int csa_verify_sa40_dev(csa_handle* h, const uint16_t* d_text, uint64_t n, uint6
     return CSA_OK;
 }
 
+int csa_enable_profile_ranges(int enable)
+{
+    if (enable_ranges(enable != 0))
+        return fail(CSA_ERR_ARG, "csa_enable_profile_ranges: no roctx library (librocprofiler-sdk-roctx.so, libroctx64.so) could be loaded");
+    return CSA_OK;
+}
+
 } // extern "C"
+
+#include "slab_entries.hpp"
+#include "host_pipeline.hpp"

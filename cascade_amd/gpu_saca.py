@@ -205,6 +205,26 @@ def sort_partition(text, key_words=1):
     return sa40, stats_to_dict(st)
 
 
+def sort_partitions(texts, key_words=1, index_base=None, out=None):
+    """Independent partitions in host memory, pipelined through the device (csa_sort_partitions_u16): the upload of one, the
+    sort of another and the download of a third overlap. texts: uint16 numpy arrays (views of pinned memory transfer at the
+    link's rate); out: optional uint8 numpy arrays of 5 * n bytes to fill. Returns (list of sa40 arrays, list of statistics)."""
+    lib = _native.load()
+    texts = [np.ascontiguousarray(t, dtype=np.uint16) for t in texts]
+    count = len(texts)
+    if out is None:
+        out = [np.zeros(SA_WIDTH * t.size, dtype=np.uint8) for t in texts]
+    assert len(out) == count and all(o.dtype == np.uint8 and o.size >= SA_WIDTH * t.size and o.flags["C_CONTIGUOUS"]
+                                     for o, t in zip(out, texts))
+    ptrs_in = (C.c_void_p * max(count, 1))(*[t.ctypes.data if t.size else None for t in texts])
+    ptrs_out = (C.c_void_p * max(count, 1))(*[o.ctypes.data if t.size else None for o, t in zip(out, texts)])
+    sizes = (C.c_uint64 * max(count, 1))(*[t.size for t in texts])
+    bases = (C.c_uint64 * max(count, 1))(*[int(b) for b in index_base]) if index_base is not None else None
+    stats = (_native.CsaStats * max(count, 1))()
+    _native.check(lib.csa_sort_partitions_u16(count, ptrs_in, sizes, bases, int(key_words), ptrs_out, stats))
+    return [o[:SA_WIDTH * t.size] for o, t in zip(out, texts)], [stats_to_dict(stats[k]) for k in range(count)]
+
+
 class GPU_SACA:
     """`GPU_SACA(ip_path, op_path).build_SA()`: file of uint16 symbols in, file of 5-byte suffix indices out."""
 

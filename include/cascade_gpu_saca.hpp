@@ -9,8 +9,10 @@
 //   sort_and_init_rank_and_filter(p_id, ., buf_id) include/GPU_SACA.hpp:272
 //   sort_and_re_rank_and_filter(p_id, ., buf_id)   include/GPU_SACA.hpp:279
 //   scatter_to_rank_order(p_id, ., buf_id)         include/GPU_SACA.hpp:288
-// Where the reference passes a Partition_Assembly (pinned host slabs that its pipeline uploads and downloads around the
-// call, include/Staging_Slab.hpp:20-119), the members here take a Device_Partition: the same columns, already in HBM.
+// The three per-partition members take what the reference's take: a Partition_Assembly, the chain of pinned host slabs
+// (include/Staging_Slab.hpp:20-119) that holds the partition before and after; upload, device step and download happen
+// inside, as in src/GPU_SACA.cu:1125-1133,1305-1331. Overloads that take a Device_Partition (the same columns, already in
+// HBM) serve callers that keep partitions on the device.
 // A failure prints the library's message and ends the process, as CUDA_CHECK does (include/utility.cuh:19-29); code
 // that wants the status instead calls the C ABI directly.
 #ifndef CASCADE_GPU_SACA_HPP
@@ -32,6 +34,35 @@ using idx_t = std::uint64_t;  // text positions, sizes (reference: include/types
 using p_id_t = std::uint16_t; // partition ids
 using p_sz_t = std::uint32_t; // partition-local ranks
 using beta_t = std::uint32_t; // pair of routing tags
+
+// A slab of a partition in pinned host memory: the reference's Staging_Slab (include/Staging_Slab.hpp:20-119) with the
+// same accessors, laid out as the C ABI's csa_slab. The buffers belong to the caller (the reference's slab pool).
+struct Staging_Slab : csa_slab {
+    Staging_Slab() : csa_slab{} {}
+    auto key() const { return csa_slab::key; }
+    auto suf() const { return csa_slab::suf; }
+    auto beta() const { return csa_slab::beta; }
+    auto msg_target() const { return csa_slab::msg_target; }
+    auto msg_rank() const { return csa_slab::msg_rank; }
+    auto off() const { return csa_slab::off; }
+    auto size() const { return csa_slab::size; }
+    auto inbox_off() const { return csa_slab::inbox_off; }
+    auto inbox_sz() const { return csa_slab::inbox_sz; }
+    auto outbox_off() const { return csa_slab::outbox_off; }
+    auto outbox_sz() const { return csa_slab::outbox_sz; }
+    void set_outbox_off_and_size(idx_t off, idx_t sz) { csa_slab::outbox_off = static_cast<std::uint32_t>(off), csa_slab::outbox_sz = static_cast<std::uint32_t>(sz); }
+    // Tags the slab with the chunk it carries (src/Staging_Slab.cpp:38-41).
+    void assign(idx_t off, idx_t sz, p_sz_t msg_off, p_sz_t inbox_sz)
+    {
+        csa_slab::off = off, csa_slab::size = sz, csa_slab::inbox_off = msg_off, csa_slab::inbox_sz = inbox_sz;
+        csa_slab::outbox_off = csa_slab::outbox_sz = 0;
+    }
+};
+
+// The chain of slabs that makes up a partition (include/Staging_Slab.hpp:122-126).
+struct Partition_Assembly {
+    std::vector<Staging_Slab*> slab;
+};
 
 // One partition's columns on the device, before and after a step (the device-side image of a Partition_Assembly).
 struct Device_Partition {
@@ -64,8 +95,13 @@ public:
     {
     }
 
-    // For a pipeline that drives partitions itself: p partitions of at most max_part_sz suffixes.
-    GPU_SACA(idx_t max_part_sz, p_id_t p, int key_words = 1) : key_words_(key_words), p_(p), max_part_sz_(max_part_sz) {}
+    // For a pipeline that drives partitions itself: p partitions of at most max_part_sz suffixes, staged through slabs
+    // of chunk_cap suffixes (a multiple of 4096, as the reference's slab_capacity gives).
+    GPU_SACA(idx_t max_part_sz, p_id_t p, int key_words = 1, idx_t chunk_cap = idx_t(1) << 21)
+        : key_words_(key_words), p_(p), max_part_sz_(max_part_sz), chunk_cap_(chunk_cap), msg_off_(p, std::vector<p_sz_t>(p, 0)),
+          active_sz_(p, 0)
+    {
+    }
 
     GPU_SACA(const GPU_SACA&) = delete;
     GPU_SACA& operator=(const GPU_SACA&) = delete;
@@ -104,6 +140,43 @@ public:
     {
         ctx_ = ctx;
         gen_ = gen;
+    }
+
+    // What the reference's backend holds per partition and the members fill: the exclusive END offset of every
+    // destination's group in the partition's outbox (backend_->msg_off(p_id)) and the new active-set size
+    // (backend_->active_slot(p_id)).
+    p_sz_t* msg_off(p_id_t p_id) { return msg_off_[p_id].data(); }
+    idx_t* active_slot(p_id_t p_id) { return &active_sz_[p_id]; }
+    idx_t chunk_cap() const { return chunk_cap_; }
+
+    // The partition's slabs in, its ranks, lanes and outbox back in the slabs (src/GPU_SACA.cu:1112-1331).
+    void sort_and_init_rank_and_filter(p_id_t p_id, Partition_Assembly& p_assembly, idx_t buf_id)
+    {
+        std::vector<csa_slab> slabs = gather(p_assembly);
+        check(csa_sort_init_slabs(csa_[buf_id], slabs.data(), static_cast<std::uint32_t>(slabs.size()), total(slabs), key_words_, p_,
+                                  chunk_cap_, msg_off(p_id), active_slot(p_id), stream_[buf_id]));
+        spread(slabs, p_assembly);
+    }
+
+    // The same for a later generation; every slab also carries its chunk of the partition's inbox (src/GPU_SACA.cu:1715-1995).
+    void sort_and_re_rank_and_filter(p_id_t p_id, Partition_Assembly& p_assembly, idx_t buf_id)
+    {
+        std::vector<csa_slab> slabs = gather(p_assembly);
+        idx_t inbox_sz = 0;
+        for (const auto& s : slabs)
+            inbox_sz += s.inbox_sz;
+        check(csa_sort_rerank_slabs(csa_[buf_id], slabs.data(), static_cast<std::uint32_t>(slabs.size()), total(slabs), inbox_sz, ctx_,
+                                    p_, chunk_cap_, msg_off(p_id), active_slot(p_id), stream_[buf_id]));
+        spread(slabs, p_assembly);
+    }
+
+    // Lanes and final ranks in the slabs -> the partition's stretch of the output, cut for the output file whose
+    // byte range for this partition starts at out_lo = 5 * P_off[p_id] (src/GPU_SACA.cu:2107-2164).
+    void scatter_to_rank_order(p_id_t /*p_id*/, Partition_Assembly& p_assembly, idx_t buf_id, idx_t out_lo)
+    {
+        std::vector<csa_slab> slabs = gather(p_assembly);
+        check(csa_scatter_slabs(csa_[buf_id], slabs.data(), static_cast<std::uint32_t>(slabs.size()), total(slabs), out_lo, chunk_cap_,
+                                stream_[buf_id]));
     }
 
     void sort_and_init_rank_and_filter(p_id_t /*p_id*/, Device_Partition& part, idx_t buf_id)
@@ -165,6 +238,27 @@ public:
     const csa_stats& stats() const { return stats_; } // generations and their sizes of the last build_SA()
 
 private:
+    static std::vector<csa_slab> gather(const Partition_Assembly& a)
+    {
+        std::vector<csa_slab> slabs;
+        slabs.reserve(a.slab.size());
+        for (const auto* s : a.slab)
+            slabs.push_back(*s);
+        return slabs;
+    }
+    static void spread(const std::vector<csa_slab>& slabs, Partition_Assembly& a)
+    {
+        for (std::size_t c = 0; c < slabs.size(); ++c)
+            a.slab[c]->set_outbox_off_and_size(slabs[c].outbox_off, slabs[c].outbox_sz);
+    }
+    static idx_t total(const std::vector<csa_slab>& slabs)
+    {
+        idx_t sz = 0;
+        for (const auto& s : slabs)
+            sz += s.size;
+        return sz;
+    }
+
     [[noreturn]] static void fail(const std::string& what)
     {
         std::cerr << what << ". Aborting.\n";
@@ -180,6 +274,9 @@ private:
     int key_words_ = 1;
     p_id_t p_ = 1;
     idx_t max_part_sz_ = 0;
+    idx_t chunk_cap_ = idx_t(1) << 21; // the reference's CHUNK_CAP (include/GPU_SACA.hpp:99)
+    std::vector<std::vector<p_sz_t>> msg_off_;
+    std::vector<idx_t> active_sz_;
     idx_t ctx_ = 0, gen_ = 0;
     csa_handle* csa_[STREAM_C] = {};
     void* stream_[STREAM_C] = {};

@@ -108,6 +108,16 @@ int csa_sort_partition_u16_dev(csa_handle* h, const uint16_t* d_text, uint64_t n
  * (src/main.cu:12-46 -> GPU_SACA::build_SA, src/GPU_SACA.cu:125-216). */
 int csa_sort_partition_u16(const uint16_t* h_text, uint64_t n, int key_words, uint8_t* h_sa40, csa_stats* stats);
 
+/* The same for `count` independent partitions in host memory, pipelined: one handle sized for the largest of them, two
+ * sets of device buffers, three streams. While partition k is sorted, the text of partition k + 1 is uploaded and the
+ * suffix array of partition k - 1 is downloaded (an upload thread and a download thread beside the calling one), which is
+ * how the reference's three dispatcher threads overlap transfers and device work (src/GPU_SACA.cu:1539-1589).
+ * h_texts[k]: n[k] symbols; h_sa40[k]: room for 5 * n[k] bytes; index_base (may be NULL = all zero): the suffix index of
+ * each partition's first symbol; stats (may be NULL): `count` records. Pinned host buffers (hipHostMalloc) transfer at the
+ * link's rate and overlap fully; pageable ones work, staged by the runtime. The call returns when everything is back. */
+int csa_sort_partitions_u16(uint32_t count, const uint16_t* const* h_texts, const uint64_t* n, const uint64_t* index_base,
+                            int key_words, uint8_t* const* h_sa40, csa_stats* stats);
+
 /* ---- the stages, exposed one by one so each can be checked against its CPU restatement ---- */
 
 /* K-gram key packing: d_keys[j * key_words + w] = symbols [j + 4w, j + 4w + 4) of the zero-padded text,
@@ -254,6 +264,61 @@ int csa_sort_rerank_dev(csa_handle* h, const uint32_t* d_rank, const uint8_t* d_
                         uint32_t p, uint32_t* d_rank_out, uint8_t* d_suf40_out, uint8_t* d_msg_target, uint32_t* d_msg_rank,
                         uint32_t* d_msg_off, void* stream, csa_step_result* res);
 
+/* ---- the same three steps in the form the reference's pipeline calls them: a partition as a chain of pinned host slabs ---- */
+
+/* One slab of a partition: the pointers and offsets of the reference's Staging_Slab (include/Staging_Slab.hpp:20-119).
+ * The buffers are host memory, pinned for transfers that overlap other work (hipHostMalloc; pageable memory works, more
+ * slowly). Capacities as the reference allocates them (src/Staging_Slab.cpp:27-35) for a slab of chunk_cap suffixes:
+ * key 8 * key_words * chunk_cap bytes, suf 5 * chunk_cap, beta 4 * chunk_cap, msg_target 5 * 2 * chunk_cap (and at least
+ * two disk blocks of 4096 bytes for the scatter's edges), msg_rank 4 * 2 * chunk_cap. */
+typedef struct csa_slab {
+    void* key;            /* key(): generation 0 in: key_words 64-bit words per suffix; later generations and scatter in:
+                             uint32 partition-local ranks; out (sort steps): uint32 ranks */
+    uint8_t* suf;         /* suf(): 5-byte lanes in; out: lanes (sort steps), the chunk's block-aligned piece (scatter) */
+    uint32_t* beta;       /* beta(): routing-tag pairs in (unused by the scatter) */
+    uint8_t* msg_target;  /* msg_target(): the slab's chunk of the inbox in (later generations), of the outbox out;
+                             scatter out: the unaligned head of the output at [0, ...), its tail at [4096, ...) */
+    uint32_t* msg_rank;   /* msg_rank(): likewise */
+    uint64_t off;         /* off(): where the slab's content starts in the partition */
+    uint64_t size;        /* size(): suffixes in the slab, at most chunk_cap */
+    uint32_t inbox_off;   /* inbox_off(), inbox_sz(): the slab's chunk of the partition's inbox (later generations) */
+    uint32_t inbox_sz;
+    uint32_t outbox_off;  /* written by the sort steps (set_outbox_off_and_size): the slab's chunk of the outbox, */
+    uint32_t outbox_sz;   /* messages [2 * c * chunk_cap, ...) for the c-th slab of the list */
+} csa_slab;
+
+/* Device bytes the slab-shaped entries add to a handle per suffix of its capacity (the device image of the slabs going
+ * in and coming out), on top of csa_bytes_per_suffix and the 16 bytes of the step entries. Allocated by the first such
+ * call, kept until csa_destroy. */
+uint64_t csa_slab_bytes_per_suffix(int key_words);
+
+/* GPU_SACA::sort_and_init_rank_and_filter(p_id, p_assembly, buf_id) (include/GPU_SACA.hpp:272, src/GPU_SACA.cu:1112-1331)
+ * as the dispatcher calls it: uploads key(), suf(), beta() of every slab to the slab's off() (:1125-1133), runs
+ * csa_sort_init_dev, then downloads into every slab its share of the ranks (over key()) and lanes, active suffixes
+ * first, and its chunk of the outbox, split at 2 * chunk_cap messages per slab (:1305-1331).
+ * h_msg_off receives the p exclusive END offsets of the destinations' groups (backend_->msg_off(p_id)), *h_active_slot
+ * the new active-set size (backend_->active_slot(p_id)); either may be NULL. part_sz = the slabs' sizes summed <= the
+ * handle's capacity. The call returns after the stream has finished (the reference's caller synchronises right after,
+ * src/GPU_SACA.cu:1582). */
+int csa_sort_init_slabs(csa_handle* h, csa_slab* slabs, uint32_t slab_c, uint64_t part_sz, int key_words, uint32_t p,
+                        uint64_t chunk_cap, uint32_t* h_msg_off, uint64_t* h_active_slot, void* stream);
+
+/* GPU_SACA::sort_and_re_rank_and_filter (include/GPU_SACA.hpp:279, src/GPU_SACA.cu:1715-1995) likewise: key() carries the
+ * uint32 ranks kept from the step before (:1739-1741), msg_target() / msg_rank() the slab's chunk of the partition's inbox at
+ * inbox_off() (:1814-1819); inbox_sz = the whole inbox <= the handle's capacity (:1807-1812); ctx = the context this
+ * generation resolves to (set_context, src/GPU_SACA.cu:1043-1049). Outputs as csa_sort_init_slabs (:1969-1995). */
+int csa_sort_rerank_slabs(csa_handle* h, csa_slab* slabs, uint32_t slab_c, uint64_t part_sz, uint64_t inbox_sz, uint64_t ctx,
+                          uint32_t p, uint64_t chunk_cap, uint32_t* h_msg_off, uint64_t* h_active_slot, void* stream);
+
+/* GPU_SACA::scatter_to_rank_order (include/GPU_SACA.hpp:288, src/GPU_SACA.cu:2107-2164): uploads suf() and the ranks in
+ * key() of every slab, scatters the lanes to rank order, and downloads the partition's stretch of the output as
+ * Output_File::cut shares it out over the slabs (csa_output_cut with chunk_bytes = 5 * chunk_cap): slab c's whole disk
+ * blocks into suf(), the unaligned head into the first slab's msg_target(), the unaligned tail into the last slab's
+ * msg_target() + 4096. out_lo = byte offset of the partition in the output file (5 * P_off[p_id]). chunk_cap must be
+ * a multiple of 4096 and slab_c * chunk_cap must reach part_sz. Returns after the stream has finished. */
+int csa_scatter_slabs(csa_handle* h, csa_slab* slabs, uint32_t slab_c, uint64_t part_sz, uint64_t out_lo, uint64_t chunk_cap,
+                      void* stream);
+
 /* ---- the step after the partition sort, for partitions that come back as (suffix, local rank) pairs ---- */
 
 /* d_sa40 entry rank[i] = d_suf entry i for i in [0, part_sz): 5-byte little-endian lanes in, lanes in rank order out.
@@ -271,6 +336,13 @@ int csa_scatter_to_rank_order_dev(csa_handle* h, const uint8_t* d_suf, const uin
  * out[4..5] = its unaligned tail (last chunk only); absent parts are empty intervals.
  * Pure host arithmetic: Output_File::cut (src/Output_File.cpp:18-35; struct at include/Output_File.hpp:29-37). */
 void csa_output_cut(uint64_t lo, uint64_t hi, uint64_t chunk_bytes, uint64_t c, uint64_t chunk_c, uint64_t out[6]);
+
+/* Named ranges on a profiler's timeline (roctx; shown by rocprofv3 --marker-trace): one per partition sort, per
+ * generation inside it, and per slab-shaped partition step. Off by default; enable != 0 loads the roctx library at run time
+ * and fails with CSA_ERR_ARG where there is none. Process-wide.
+ * Replaces the NVTX ranges of the reference's -DPROFILE build (include/profile.hpp:19-80; PROFILE_SCOPE_FMT at
+ * src/GPU_SACA.cu:1114,1717,2004,2111). */
+int csa_enable_profile_ranges(int enable);
 
 /* Message of the calling thread's last failed call ("" if none). */
 const char* csa_last_error(void);

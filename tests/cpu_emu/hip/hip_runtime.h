@@ -245,6 +245,10 @@ inline hipError_t hipMemsetAsync(void* p, int v, size_t bytes, hipStream_t) { re
 inline hipError_t hipMemcpy(void* d, const void* s, size_t bytes, hipMemcpyKind) { std::memmove(d, s, bytes); return hipSuccess; }
 inline hipError_t hipMemcpyAsync(void* d, const void* s, size_t bytes, hipMemcpyKind k, hipStream_t) { return hipMemcpy(d, s, bytes, k); }
 inline hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
+constexpr unsigned hipStreamNonBlocking = 1;
+inline hipError_t hipStreamCreateWithFlags(hipStream_t* s, unsigned) { *s = nullptr; return hipSuccess; }
+inline hipError_t hipStreamDestroy(hipStream_t) { return hipSuccess; }
+inline hipError_t hipSetDevice(int) { return hipSuccess; }
 inline hipError_t hipDeviceSynchronize() { return hipSuccess; }
 inline hipError_t hipEventCreate(hipEvent_t* e) { *e = new hipEmuEvent(); return hipSuccess; }
 inline hipError_t hipEventDestroy(hipEvent_t e) { delete e; return hipSuccess; }

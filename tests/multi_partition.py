@@ -73,13 +73,68 @@ def validate_coherent_targets(suf, rank, pid, n, stride, ell):
     assert (tag[1:][tied] == tag[:-1][tied]).all(), "target coherence invariant broken"
 
 
+class SlabPool:
+    """Host slabs with the reference's capacities for chunk_cap suffixes (src/Staging_Slab.cpp:27-35), handed out as csa_slab
+    records. host_buf(nbytes) returns a uint8 numpy array (pinned memory on the GPU, plain memory under the emulation)."""
+
+    def __init__(self, host_buf, chunk_cap, key_words):
+        self.host_buf, self.cap, self.kw, self.bufs = host_buf, chunk_cap, key_words, []
+
+    def _slab(self, c):
+        while len(self.bufs) <= c:
+            cap = self.cap
+            self.bufs.append({"key": self.host_buf(8 * self.kw * cap), "suf": self.host_buf(5 * cap), "beta": self.host_buf(4 * cap),
+                              "msg_target": self.host_buf(max(10 * cap, 2 * 4096)), "msg_rank": self.host_buf(8 * cap)})
+        return self.bufs[c]
+
+    def assemble(self, pieces, inbox_pieces=()):
+        """pieces: [(off, size)] of the partition's content per slab; inbox_pieces: [(off, size)] of its inbox per slab.
+        Returns the ctypes array of csa_slab and the buffers of each."""
+        from cascade_amd._native import CsaSlab
+        slab_c = max(len(pieces), len(inbox_pieces))
+        arr = (CsaSlab * max(slab_c, 1))()
+        bufs = []
+        for c in range(slab_c):
+            b = self._slab(c)
+            off, size = pieces[c] if c < len(pieces) else (0, 0)
+            ioff, isz = inbox_pieces[c] if c < len(inbox_pieces) else (0, 0)
+            arr[c].key, arr[c].suf, arr[c].beta = b["key"].ctypes.data, b["suf"].ctypes.data, b["beta"].ctypes.data
+            arr[c].msg_target, arr[c].msg_rank = b["msg_target"].ctypes.data, b["msg_rank"].ctypes.data
+            arr[c].off, arr[c].size, arr[c].inbox_off, arr[c].inbox_sz = off, size, ioff, isz
+            arr[c].outbox_off, arr[c].outbox_sz = 0xFFFFFFFF, 0xFFFFFFFF  # the call must set them
+            bufs.append(b)
+        return arr, slab_c, bufs
+
+
+def ragged_pieces(total, chunk_cap, rng):
+    """[0, total) cut into consecutive pieces of 0 to chunk_cap elements: full ones, short ones and the odd empty one."""
+    pieces, off = [], 0
+    while off < total:
+        kind = rng.integers(4)
+        if kind == 0:
+            size = chunk_cap
+        elif kind == 1 and rng.integers(3) == 0:
+            size = 0
+        elif kind == 2:  # a short one, so that small partitions span several slabs too
+            size = int(rng.integers(1, min(chunk_cap, total // 4 + 1) + 1))
+        else:
+            size = int(rng.integers(1, chunk_cap + 1))
+        size = min(size, total - off)
+        pieces.append((off, size))
+        off += size
+    return pieces
+
+
 def build_sa(lib, to_dev, to_host, T, p, key_words=1, pivot_words=2, seed=0, max_generations=64, log=None, join_handle=None,
-             step_handle=None):
+             step_handle=None, slab_handle=None, host_buf=None, chunk_cap=4096):
     """Returns (sa uint64[n], generations run). `to_dev(np array)` gives an object with .ptr; `to_host(obj)` the array back.
     log (a list) receives (generation, partition, cohort, survivors, messages, pills) per step. join_handle: a handle
     whose scratch the join may use to sort the inbox first (csa_join_messages_sorted_dev). step_handle: a handle of at
     least the largest partition's capacity; with it, each partition step is ONE call of csa_sort_init_dev /
-    csa_sort_rerank_dev (sorts, ranking, split and messages inside the library) instead of numpy glue between stages."""
+    csa_sort_rerank_dev (sorts, ranking, split and messages inside the library) instead of numpy glue between stages.
+    slab_handle (with host_buf and chunk_cap): each partition step is ONE call of csa_sort_init_slabs / csa_sort_rerank_slabs on
+    host slabs of ragged sizes, as the reference's dispatcher calls its members with a Partition_Assembly, and the final
+    permutation goes through csa_scatter_slabs with the output cut into disk blocks."""
     T = np.ascontiguousarray(T, dtype=np.uint16)
     n, ell = T.size, 4 * key_words
     rng = np.random.default_rng(seed)
@@ -105,6 +160,7 @@ def build_sa(lib, to_dev, to_host, T, p, key_words=1, pivot_words=2, seed=0, max
         part.append({"suf": suf, "rank": np.zeros(suf.size, dtype=np.uint32), "active": suf.size})
     inbox = [(np.zeros(0, dtype=np.uint64), np.zeros(0, dtype=np.uint32)) for _ in range(p)]
 
+    pool = SlabPool(host_buf, chunk_cap, key_words) if slab_handle is not None else None
     gen, ctx = 0, ell
     while any(pt["active"] > 0 for pt in part):
         assert gen < max_generations
@@ -128,6 +184,62 @@ def build_sa(lib, to_dev, to_host, T, p, key_words=1, pivot_words=2, seed=0, max
             assert lib.csa_stage_slab_u16_dev(d_T.ptr, n, d_lanes.ptr, a, key_words, d_map.ptr, p, ctx,
                                               1 if gen == 0 else 0, d_keys.ptr if gen == 0 else None, d_beta.ptr, None) == 0
             beta = to_host(d_beta)
+            if slab_handle is not None:
+                # ---- the whole step, host slabs in and out (src/GPU_SACA.cu:1112-1331 / 1715-1995 as the dispatcher calls them) ----
+                import ctypes as C
+                lanes = oracle_lib.u64_to_sa40(suf)
+                tgt, rk = inbox[q] if gen > 0 else (np.zeros(0, dtype=np.uint64), np.zeros(0, dtype=np.uint32))
+                tgt_lanes = oracle_lib.u64_to_sa40(tgt)
+                pieces = ragged_pieces(a, chunk_cap, rng)
+                inbox_pieces = ragged_pieces(tgt.size, chunk_cap, rng)
+                arr, slab_c, bufs = pool.assemble(pieces, inbox_pieces)
+                keys_h = to_host(d_keys).reshape(a, key_words) if gen == 0 else None
+                for c, b in enumerate(bufs):
+                    off, size = arr[c].off, arr[c].size
+                    if gen == 0:
+                        b["key"].view(np.uint64)[:size * key_words] = keys_h[off:off + size].reshape(-1)
+                    else:
+                        b["key"].view(np.uint32)[:size] = prim[off:off + size]
+                    b["suf"][:5 * size] = lanes[5 * off:5 * (off + size)]
+                    b["beta"].view(np.uint32)[:size] = beta[off:off + size]
+                    ioff, isz = arr[c].inbox_off, arr[c].inbox_sz
+                    b["msg_target"][:5 * isz] = tgt_lanes[5 * ioff:5 * (ioff + isz)]
+                    b["msg_rank"].view(np.uint32)[:isz] = rk[ioff:ioff + isz]
+                end = np.zeros(p, dtype=np.uint32)
+                active_slot = C.c_uint64(0xFFFFFFFFFFFFFFFF)
+                if gen == 0:
+                    rc = lib.csa_sort_init_slabs(slab_handle, arr, slab_c, a, key_words, p, chunk_cap, end.ctypes.data,
+                                                 C.byref(active_slot), None)
+                else:
+                    rc = lib.csa_sort_rerank_slabs(slab_handle, arr, slab_c, a, tgt.size, ctx, p, chunk_cap, end.ctypes.data,
+                                                   C.byref(active_slot), None)
+                assert rc == 0, lib.csa_last_error()
+                a_new, total = int(active_slot.value), int(end[p - 1])
+                new_suf, new_rank = np.zeros(a, dtype=np.uint64), np.zeros(a, dtype=np.uint32)
+                m_tgt, m_rank = np.zeros(total, dtype=np.uint64), np.zeros(total, dtype=np.uint32)
+                for c, b in enumerate(bufs):
+                    off, size = arr[c].off, arr[c].size
+                    new_suf[off:off + size] = oracle_lib.sa40_to_u64(b["suf"][:5 * size])
+                    new_rank[off:off + size] = b["key"].view(np.uint32)[:size]
+                    # the outbox is shared out in chunks of 2 * chunk_cap messages per slab (src/GPU_SACA.cu:1318-1320)
+                    ooff, osz = arr[c].outbox_off, arr[c].outbox_sz
+                    assert ooff == 2 * c * chunk_cap and osz == max(0, min(2 * chunk_cap, total - ooff)), (c, ooff, osz, total)
+                    m_tgt[ooff:ooff + osz] = oracle_lib.sa40_to_u64(b["msg_target"][:5 * osz])
+                    m_rank[ooff:ooff + osz] = b["msg_rank"].view(np.uint32)[:osz]
+                full_end = np.concatenate([end, [total]]).astype(np.uint32)
+                validate_messages(m_tgt, m_rank, full_end, q, pid, psz, n, ctx)
+                start = 0
+                for dest in range(p):
+                    e = int(end[dest])
+                    outboxes[dest][0].append(m_tgt[start:e])
+                    outboxes[dest][1].append(m_rank[start:e])
+                    start = e
+                pt["suf"][:a], pt["rank"][:a] = new_suf, new_rank
+                pt["active"] = a_new
+                retired_now.append(pt["suf"][a_new:a].copy())
+                if log is not None:
+                    log.append((gen, q, a, a_new, total, int((m_rank >> np.uint32(31)).sum())))
+                continue
             if step_handle is not None:
                 # ---- the whole step inside the library (src/GPU_SACA.cu:1112-1331 / 1715-1995) ----
                 import ctypes as C
@@ -244,6 +356,32 @@ def build_sa(lib, to_dev, to_host, T, p, key_words=1, pivot_words=2, seed=0, max
 
     # ---- every partition to rank order, partitions concatenated (src/GPU_SACA.cu:2107-2164) ----
     sa = np.zeros(n, dtype=np.uint64)
+    if slab_handle is not None:
+        # the partitions' stretches of the output file, as Output_File::cut shares them out over the slabs
+        # (src/GPU_SACA.cu:2146-2163): whole disk blocks in suf(), the unaligned edges in the first and last slab's msg_target()
+        file_bytes = np.full(5 * n, 0xEE, dtype=np.uint8)
+        for q in range(p):
+            m = part[q]["suf"].size
+            if m == 0:
+                continue
+            lanes = oracle_lib.u64_to_sa40(part[q]["suf"])
+            pieces = ragged_pieces(m, chunk_cap, rng)
+            while len(pieces) * chunk_cap < m + chunk_cap:  # room for every chunk window of the output
+                pieces.append((m, 0))
+            arr, slab_c, bufs = pool.assemble(pieces)
+            for c, b in enumerate(bufs):
+                off, size = arr[c].off, arr[c].size
+                b["suf"][:5 * size] = lanes[5 * off:5 * (off + size)]
+                b["key"].view(np.uint32)[:size] = part[q]["rank"][off:off + size]
+            lo = 5 * int(P_off[q])
+            rc = lib.csa_scatter_slabs(slab_handle, arr, slab_c, m, lo, chunk_cap, None)
+            assert rc == 0, lib.csa_last_error()
+            for c, b in enumerate(bufs):
+                cut = oracle_lib.output_cut(lo, lo + 5 * m, 5 * chunk_cap, c, slab_c)
+                file_bytes[cut[0]:cut[1]] = b["suf"][:cut[1] - cut[0]]
+                file_bytes[cut[2]:cut[3]] = b["msg_target"][:cut[3] - cut[2]]
+                file_bytes[cut[4]:cut[5]] = b["msg_target"][4096:4096 + cut[5] - cut[4]]
+        return oracle_lib.sa40_to_u64(file_bytes), gen
     h = lib_handle(lib)
     try:
         for q in range(p):

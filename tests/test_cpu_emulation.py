@@ -37,6 +37,9 @@ def emu():
     lib.csa_join_messages_sorted_dev.argtypes = [vp, vp, vp, u32, vp, vp, vp, u64, vp]
     lib.csa_sort_init_dev.argtypes = [vp, vp, i32, vp, vp, u64, u32, vp, vp, vp, vp, vp, vp, vp]
     lib.csa_sort_rerank_dev.argtypes = [vp, vp, vp, vp, u64, vp, vp, u32, u64, u32, vp, vp, vp, vp, vp, vp, vp]
+    lib.csa_sort_init_slabs.argtypes = [vp, C.POINTER(_native.CsaSlab), u32, u64, i32, u32, u64, vp, vp, vp]
+    lib.csa_sort_rerank_slabs.argtypes = [vp, C.POINTER(_native.CsaSlab), u32, u64, u64, u64, u32, u64, vp, vp, vp]
+    lib.csa_scatter_slabs.argtypes = [vp, C.POINTER(_native.CsaSlab), u32, u64, u64, u64, vp]
     return lib
 
 
@@ -286,6 +289,27 @@ def test_multi_partition_pipeline_with_the_emulated_step_entries(emu, p, key_wor
     # the same run with numpy glue between the stages: the same cohorts, survivors and message counts at every step
     multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, p, key_words=key_words, log=glue_log)
     assert log == glue_log
+
+
+@pytest.mark.parametrize("p,key_words,sigma,n,chunk_cap", [(3, 1, 3, 2000, 4096), (4, 2, 2, 1500, 4096)])
+def test_multi_partition_pipeline_through_the_emulated_slab_entries(emu, p, key_words, sigma, n, chunk_cap):
+    """csa_sort_init_slabs / csa_sort_rerank_slabs / csa_scatter_slabs: every partition step takes and returns host slabs of
+    ragged sizes (several per partition, some empty, the inbox shared out over them), the final permutation comes back cut
+    into disk blocks and edges; the suffix array assembled from those pieces is the oracle's."""
+    import multi_partition
+    T = texts.random_text(n, sigma, 31 * p + n, sep_every=0)
+    T[n // 3:n // 3 + 700] = T[:700]
+    T[-5:] = 0
+    h = C.c_void_p()
+    assert emu.csa_create(n, 1, C.byref(h)) == 0
+    try:
+        # slabs far smaller than the reference's: a partition of a few thousand suffixes still spans several
+        sa, gens = multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, p, key_words=key_words,
+                                            slab_handle=h, host_buf=lambda nbytes: np.zeros(nbytes, dtype=np.uint8), chunk_cap=chunk_cap)
+    finally:
+        emu.csa_destroy(h)
+    want, _ = oracle_lib.prefix_doubling(T, key_words)
+    assert np.array_equal(sa, want) and gens >= 5
 
 
 def test_step_entries_on_a_text_of_one_symbol(emu):

@@ -58,6 +58,86 @@ def test_partitions_that_only_exchange_messages_build_the_oracles_suffix_array(g
     assert gens >= 10 and sum(step[5] for step in log if step[0] >= 1) > 0
 
 
+def pinned_host_buf(nbytes):
+    """uint8 numpy view of freshly pinned host memory (the view keeps the tensor alive)."""
+    import torch
+    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, pin_memory=True).numpy()
+
+
+@pytest.mark.parametrize("p,key_words,chunk_cap", [(3, 1, 4096), (16, 2, 8192), (40, 1, 4096), (9, 4, 4096), (1, 1, 32768)])
+def test_slab_shaped_entries_from_pinned_host_slabs_build_the_oracles_suffix_array(gpu, p, key_words, chunk_cap):
+    """The three members as the reference's dispatcher calls them (src/GPU_SACA.cu:1579-1580, 2356): every partition step takes
+    the partition as pinned host slabs of ragged sizes (upload, device step, download inside csa_sort_init_slabs /
+    csa_sort_rerank_slabs), and csa_scatter_slabs returns each partition's stretch of the output cut into disk blocks and
+    edges. The file assembled from those pieces is the oracle's suffix array."""
+    lib, to_dev, to_host = gpu
+    n = 120000
+    T = texts.random_text(n, 4, 11 * p, sep_every=0)
+    T[30000:70000] = T[:40000]
+    T[-9:] = 0
+    log = []
+    h = C.c_void_p()
+    assert lib.csa_create(n, 1, C.byref(h)) == 0
+    try:
+        print(f"  slab entries n={n} p={p} key_words={key_words} chunk_cap={chunk_cap}", flush=True)
+        sa, gens = multi_partition.build_sa(lib, to_dev, to_host, T, p, key_words=key_words, log=log, slab_handle=h,
+                                            host_buf=pinned_host_buf, chunk_cap=chunk_cap)
+    finally:
+        lib.csa_destroy(h)
+    want, _ = oracle_lib.prefix_doubling(T, key_words)
+    assert np.array_equal(sa, want)
+    assert gens >= 10 and (p == 1 or sum(step[5] for step in log if step[0] >= 1) > 0)
+
+
+def test_slab_shaped_entries_report_what_the_device_entries_report(gpu):
+    """The same pipeline through csa_sort_*_dev and through csa_sort_*_slabs: cohort, survivors, messages and pills agree in
+    every generation of every partition."""
+    lib, to_dev, to_host = gpu
+    from cascade_amd import workloads
+    T = workloads.generate(3, 200000)
+    n, p = T.size, 12
+    logs = []
+    for mode in ("dev", "slabs"):
+        log = []
+        h = C.c_void_p()
+        assert lib.csa_create(n, 1, C.byref(h)) == 0
+        try:
+            print(f"  {mode} entries n={n} p={p}", flush=True)
+            kw = {"step_handle": h} if mode == "dev" else {"slab_handle": h, "host_buf": pinned_host_buf, "chunk_cap": 8192}
+            sa, _ = multi_partition.build_sa(lib, to_dev, to_host, T, p, log=log, seed=5, **kw)
+        finally:
+            lib.csa_destroy(h)
+        assert np.array_equal(sa, oracle_lib.prefix_doubling(T, 1)[0])
+        logs.append(log)
+    assert logs[0] == logs[1]
+
+
+def test_slab_entries_refuse_slabs_that_do_not_make_up_the_partition(gpu):
+    lib, _, _ = gpu
+    from cascade_amd import _native
+    h = C.c_void_p()
+    assert lib.csa_create(10000, 1, C.byref(h)) == 0
+    try:
+        pool = multi_partition.SlabPool(pinned_host_buf, 4096, 1)
+        arr, slab_c, _ = pool.assemble([(0, 4096), (4096, 1000)])
+        end, act = np.zeros(3, dtype=np.uint32), C.c_uint64(0)
+        # sizes that do not add up to the partition, a slab beyond chunk_cap, a partition beyond the handle
+        assert lib.csa_sort_init_slabs(h, arr, slab_c, 6000, 1, 3, 4096, end.ctypes.data, C.byref(act), None) == _native.CSA_ERR_ARG
+        assert b"slabs hold" in lib.csa_last_error()
+        assert lib.csa_sort_init_slabs(h, arr, slab_c, 5096, 1, 3, 4000, end.ctypes.data, C.byref(act), None) == _native.CSA_ERR_ARG
+        assert lib.csa_sort_init_slabs(h, arr, slab_c, 20000, 1, 3, 4096, end.ctypes.data, C.byref(act), None) == _native.CSA_ERR_ARG
+        # an inbox that the slabs do not carry in full
+        assert lib.csa_sort_rerank_slabs(h, arr, slab_c, 5096, 77, 8, 3, 4096, end.ctypes.data, C.byref(act), None) == _native.CSA_ERR_ARG
+        assert b"inbox" in lib.csa_last_error()
+        # a scatter whose chunks cannot carry the output: chunk_cap not a multiple of 4096 suffixes
+        arr2, c2, bufs = pool.assemble([(0, 3000), (3000, 2096)])
+        for b in bufs:
+            b["key"].view(np.uint32)[:4096] = 0
+        assert lib.csa_scatter_slabs(h, arr2, c2, 5096, 0, 3000, None) == _native.CSA_ERR_ARG
+    finally:
+        lib.csa_destroy(h)
+
+
 def _shape(name):
     from cascade_amd import workloads
     if name == "one_symbol":       # one group until the very end; every pivot equal, so all but one partition are empty

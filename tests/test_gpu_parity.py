@@ -193,6 +193,29 @@ def test_host_buffer_entry_point_and_file_interface(torch_mod, tmp_path):
     assert np.array_equal(np.fromfile(op, dtype=np.uint8), sa40)
 
 
+def test_pipelined_host_buffer_entry_sorts_every_partition_of_a_list(torch_mod):
+    """csa_sort_partitions_u16: partitions of different sizes (an empty one among them) from pinned and from pageable host
+    memory, with index bases, each byte-equal to the oracle's sort; the upload and download threads must hand every
+    buffer over at the right time."""
+    from cascade_amd import sort_partitions, workloads
+    rng = np.random.default_rng(8)
+    sizes = [70000, 1, 0, 300000, 5000, 123457, 2, 99999, 150000]
+    texts_k = [workloads.generate(3 if k % 2 else 5, n) if n >= 64 else rng.integers(0, 3, n).astype(np.uint16) for k, n in enumerate(sizes)]
+    bases = [int(rng.integers(0, 1 << 39)) for _ in sizes]
+    for pinned in (False, True):
+        ins, outs = texts_k, None
+        if pinned:
+            keep = [torch_mod.from_numpy(t.view(np.int16).copy()).pin_memory() for t in texts_k]
+            ins = [k.numpy().view(np.uint16) for k in keep]
+            outs = [torch_mod.empty(max(5 * t.size, 1), dtype=torch_mod.uint8, pin_memory=True).numpy() for t in texts_k]
+        print(f"  pipelined host entry, {len(sizes)} partitions, pinned={pinned}", flush=True)
+        got, stats = sort_partitions(ins, key_words=1, index_base=bases, out=outs)
+        for k, T in enumerate(texts_k):
+            want = oracle_lib.sa40_to_u64(oracle_lib.build_sa40(T)) + np.uint64(bases[k])
+            assert np.array_equal(oracle_lib.sa40_to_u64(got[k]), want), (k, T.size, pinned)
+            assert stats[k]["n"] == T.size
+
+
 def test_text_pointer_at_every_alignment(torch_mod, sorter, sorter2):
     # the text may start anywhere inside an aligned 8-byte word (a window of a larger buffer), and end anywhere too
     torch = torch_mod
