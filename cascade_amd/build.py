@@ -20,8 +20,9 @@ HIPCC_FLAGS = [
     "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared", "-Wall",
     # packed FP32 instructions stay off (nothing here is floating point, the flag is policy for this target)
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    # machine-level loop-invariant code motion hoists values out of the kernels' unrolled item loops that then stay
-    # live through the whole body; without it the radix pass needs fewer vector registers
+    # machine-level loop-invariant code motion hoists values out of loops that then stay live through the whole body:
+    # without it partition_ids_kernel fits 5 waves per SIMD instead of 4 (8.7 -> 7.7 ms per 1e9 suffixes); the other
+    # kernels are unchanged by it
     "-mllvm", "-disable-machine-licm",
 ]
 
