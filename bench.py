@@ -31,20 +31,36 @@ def algorithmic_bytes(n, active):
     return per_gen, 14 * n
 
 
-def measured_traffic_per_pair():
-    """HBM bytes one radix pass moves per pair, from the FETCH_SIZE / WRITE_SIZE counter runs of this same command
-    that are summarised in profiles/ (lines 'fetch_bytes_per_pair = X' and 'write_bytes_per_pair = Y', already
-    scaled by what the counters read for the plain copy below). None where no summary is committed."""
-    path = os.path.join(ROOT, "profiles", "onesweep_c3_1b_pmc_traffic.txt")
-    got = {}
+PROFILE_TAG = {2: "c2_256m", 3: "c3_1b", 4: "c4_2b", 5: "c5_512m"}
+
+
+def measured_traffic(config):
+    """HBM bytes moved, from the FETCH_SIZE / WRITE_SIZE counter runs of this same command on the same workload that are
+    summarised in profiles/partition_sort_<workload>_pmc_traffic.txt (already scaled by what the counters read for the
+    plain copy below; a sort of a given text moves the same bytes in every run). Lines read:
+      fetch_bytes_per_pair = X / write_bytes_per_pair = Y     one radix pass, per (key, index) pair
+      generation_traffic g=<g> read_GB=<r> write_GB=<w>       every generation
+      sort_traffic read_GB=<r> write_GB=<w>                   the whole sort, output included
+    Returns (source file, bytes per pair or None, {g: bytes}, job bytes or None); all None where no summary is committed."""
+    name = f"partition_sort_{PROFILE_TAG.get(config, 'none')}_pmc_traffic.txt"
+    path = os.path.join(ROOT, "profiles", name)
+    per_pair, gens, job = {}, {}, None
     try:
         for line in open(path):
+            f = line.split()
             for key in ("fetch_bytes_per_pair", "write_bytes_per_pair"):
                 if line.startswith(key) and "=" in line:
-                    got[key] = float(line.split("=")[1].split()[0])
+                    per_pair[key] = float(line.split("=")[1].split()[0])
+            if f and f[0] == "generation_traffic":
+                kv = dict(x.split("=") for x in f[1:])
+                gens[int(kv["g"])] = (float(kv["read_GB"]) + float(kv["write_GB"])) * 1e9
+            if f and f[0] == "sort_traffic":
+                kv = dict(x.split("=") for x in f[1:])
+                job = (float(kv["read_GB"]) + float(kv["write_GB"])) * 1e9
     except OSError:
-        return None
-    return got["fetch_bytes_per_pair"] + got["write_bytes_per_pair"] if len(got) == 2 else None
+        return None, None, {}, None
+    pp = per_pair["fetch_bytes_per_pair"] + per_pair["write_bytes_per_pair"] if len(per_pair) == 2 else None
+    return "profiles/" + name, pp, gens, job
 
 
 def cpu_baseline(config, sample_n):
@@ -412,8 +428,13 @@ def main():
     ap.add_argument("--config", type=int, default=3, help="workload 1..5 (3 = the 1B-token headline)")
     ap.add_argument("--n", type=int, default=None, help="override the partition size (scaled construction)")
     ap.add_argument("--key-words", type=int, default=1)
-    ap.add_argument("--cpu-sample", type=int, default=1 << 26, help="symbols of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--cpu-sample", type=int, default=None,
+                    help="symbols of the CPU baseline sample (0 = skip); default: what the reference's comparison sort finishes "
+                         "in 10 to 30 s on the workload (2^26 on the token corpora, less where long repeats make every comparison deep)")
     ap.add_argument("--no-verify", action="store_true")
+    ap.add_argument("--no-oracle-verify", action="store_true",
+                    help="check the headline output with the device verifier only (the default also runs the CPU oracle's O(n) "
+                         "verifier on it, about 23 bytes of host memory per suffix)")
     ap.add_argument("--generations", action="store_true", help="print the per-generation table to stderr")
     ap.add_argument("--row", default="sort", choices=["sort", "partition_ids", "stage_slab", "messages", "join", "scatter", "step_init", "step_rerank", "overlap", "pipeline"],
                     help="which step to measure: the partition sort (the headline, default) or one of the steps around it")
@@ -424,6 +445,8 @@ def main():
     ap.add_argument("--partitions", type=int, default=256, help="partitions of --row partition_ids")
     args = ap.parse_args()
 
+    if args.cpu_sample is None:
+        args.cpu_sample = {1: 1 << 20, 2: 1 << 26, 3: 1 << 26, 4: 1 << 23, 5: 1 << 18}.get(args.config, 1 << 20)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU: a partition is sorted inside one device's HBM and nothing here "
               "shards it; run with --gpus 1", file=sys.stderr)
@@ -445,7 +468,9 @@ def main():
     T = workloads.generate(args.config, n)
     t_gen = time.perf_counter() - t0
     d_text = torch.from_numpy(T.view(np.int16)).to(dev)
-    del T
+    oracle_check = not (args.no_verify or args.no_oracle_verify)
+    if not oracle_check:
+        del T
     out = torch.empty(5 * n + 128, dtype=torch.uint8, device=dev)
     # bench.py is the only user of the GPU while it runs, which is what csa_set_device_exclusive asks the caller to
     # declare; the time of the default tile order (safe next to other launches) is measured beside it
@@ -480,9 +505,23 @@ def main():
     ms_per_step = 1e3 * elapsed / args.steps
     st = sorter.last_stats
     verified = None
-    if not args.no_verify:
-        verified = sorter.verify(d_text, out)
+    verified_by = []
+    if oracle_check:
+        # the CPU oracle's O(n) verifier (the reference's rule, test/end-to-end.cpp:46-80) on the headline output:
+        # outside the timed region, and the only use of the oracle besides the CPU baseline below
+        import oracle_lib
+        t1 = time.perf_counter()
+        verified = bool(oracle_lib.is_correct_sa40(out[:5 * n].cpu().numpy(), T))
+        print(f"[bench] oracle verifier: {verified} in {time.perf_counter() - t1:.1f} s", file=sys.stderr, flush=True)
+        verified_by.append("oracle orc_is_correct_sa40_u16 (host, O(n): permutation + every adjacent pair in order)")
+        del T
         if not verified:
+            print("[bench] the oracle's verifier REJECTED the suffix array", file=sys.stderr)
+    if not args.no_verify:
+        ok_dev = sorter.verify(d_text, out)
+        verified = ok_dev if verified is None else (verified and ok_dev)
+        verified_by.append("csa_verify_sa40_dev (device, same rule)")
+        if not ok_dev:
             print("[bench] the device verifier REJECTED the suffix array", file=sys.stderr)
 
     ms_by_arrival = ms_per_step
@@ -502,11 +541,23 @@ def main():
 
     per_gen, a_out = algorithmic_bytes(n, st["active"])
     a_total = sum(per_gen) + a_out
+    full_workload = args.n is None and args.key_words == 1
+    traffic_source, per_pair, moved_gen, moved_job = measured_traffic(args.config) if full_workload else (None, None, {}, None)
     gen_table = []
     for g in range(st["generations"]):
         gbs = per_gen[g] / (st["ms"][g] * 1e-3) / 1e9 if st["ms"][g] > 0 else 0.0
-        gen_table.append({"g": g, "active": st["active"][g], "groups": st["groups"][g], "big": st["big"][g], "passes": st["passes"][g], "rank_update": st["rank_update"][g], "small_only": st["small_only"][g],
-                          "ms": round(st["ms"][g], 3), "alg_GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4)})
+        # alg_over_peak: the yardstick's bytes (8 radix passes over every active suffix in every generation) over the time,
+        # as a share of the HBM peak. It is NOT a roofline fraction: generations whose groups are sorted inside LDS move far
+        # fewer bytes than the yardstick charges and come out above 1. frac_moved is the roofline fraction: bytes the
+        # counters saw this generation move (from the committed profile of this workload) over this run's time.
+        row = {"g": g, "active": st["active"][g], "groups": st["groups"][g], "big": st["big"][g], "passes": st["passes"][g],
+               "rank_update": st["rank_update"][g], "small_only": st["small_only"][g], "dense": st["dense"][g], "ms": round(st["ms"][g], 3),
+               "alg_GBps": round(gbs, 1), "alg_over_peak": round(gbs / HBM_PEAK_GBS, 4)}
+        if g in moved_gen and st["ms"][g] > 0:
+            mv = moved_gen[g] / (st["ms"][g] * 1e-3) / 1e9
+            row["moved_GBps"] = round(mv, 1)
+            row["frac_moved"] = round(mv / HBM_PEAK_GBS, 4)
+        gen_table.append(row)
     if args.generations:
         for row in gen_table:
             print("[gen]", json.dumps(row), file=sys.stderr)
@@ -516,12 +567,13 @@ def main():
     avg_launch_ms = radix_ms / radix_launches if radix_launches else 0.0
     achieved = (RADIX_PASS_BYTES_PER_PAIR * radix_pairs / (radix_ms * 1e-3) / 1e9) if radix_ms > 0 else 0.0
     pairs_per_launch = radix_pairs / radix_launches if radix_launches else 0
-    per_pair = measured_traffic_per_pair() if (args.config == 3 and args.n is None and args.key_words == 1) else None
     roofline = {
         "bound": "hbm", "kernel": "onesweep_kernel (one radix pass over (key, index) pairs)",
         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
         "traffic": round(per_pair * pairs_per_launch) if per_pair is not None else None,
+        "traffic_source": traffic_source,
+        "frac_moved": round(per_pair * radix_pairs / (radix_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4) if per_pair is not None and radix_ms > 0 else None,
         "algorithmic_bytes_per_launch": round(RADIX_PASS_BYTES_PER_PAIR * pairs_per_launch),
         "launches_per_step": radix_launches / args.steps, "avg_launch_ms": round(avg_launch_ms, 4),
         "pairs_per_launch": pairs_per_launch,
@@ -537,12 +589,14 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u64 keys / u32 ranks", "data": "synthetic",
         "config": {"workload": workloads.NAMES[args.config], "n": n, "key_words": args.key_words,
-                   "generations": st["generations"], "bit_exact_verified": verified,
+                   "generations": st["generations"], "bit_exact_verified": verified, "verified_by": verified_by,
                    "tile_order": "by arrival" if args.shared_device else "XCD-chunked (device declared exclusive)",
                    "ms_per_step_tiles_by_arrival": round(ms_by_arrival, 3)},
         "roofline": roofline,
-        "job_hbm_frac": round(a_total / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        "job_alg_over_peak": round(a_total / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         "job_algorithmic_bytes_per_suffix": round(a_total / n, 1),
+        "job_frac_moved": round(moved_job / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4) if moved_job else None,
+        "job_moved_bytes_per_suffix": round(moved_job / n, 1) if moved_job else None,
         "generations": gen_table,
     }
     if args.cpu_sample > 0:

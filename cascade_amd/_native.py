@@ -46,6 +46,7 @@ class CsaStats(C.Structure):
         ("passes", C.c_int32 * CSA_MAX_GENERATIONS),
         ("rank_update", C.c_int32 * CSA_MAX_GENERATIONS),
         ("small_only", C.c_int32 * CSA_MAX_GENERATIONS),
+        ("dense", C.c_int32 * CSA_MAX_GENERATIONS),
         ("ms", C.c_float * CSA_MAX_GENERATIONS),
         ("ms_output", C.c_float),
         ("ms_total", C.c_float),

@@ -181,6 +181,12 @@ constexpr int EVENT_POOL = 2 * CSA_MAX_GENERATIONS * MAX_PASSES * 2;
 #ifndef CSA_DEFER_MIN
 #define CSA_DEFER_MIN (1u << 23)
 #endif
+// Lists of at least this many suffixes may take the dense form of a later generation (the whole partition sorted again
+// by keys read in text order); below it the generation is over before the choice matters. Smaller in test builds.
+#ifndef CSA_DENSE_MIN
+#define CSA_DENSE_MIN (1u << 16)
+#endif
+constexpr u32 DENSE_MIN = CSA_DENSE_MIN;
 constexpr u32 XCD_CHUNK = 16;
 // Windows of rank[] that the last step of generation 0's bucketed update assembles in LDS (1 << 14 positions; twice
 // that on the largest partitions, whose two passes cover 16 position bits at most). Smaller in test builds, so that
@@ -394,8 +400,10 @@ void launch_onesweep32(const csa_handle* hh, OnesweepArgs& a, hipStream_t s)
 // (pairs kin/vin, or the text); passes alternate between the (kin, vin) and (kout, vout) sets, the
 // very first one writing to (kout, vout). *result_in_out = 1 if the sorted pairs ended in (kout, vout).
 // Passes whose digit is the same for every pair are skipped (they would be the identity).
+// src = SRC_RANKS: pair i is ((rank_src[i], rank_src[i + hop]), i), i < n, built by the first pass that runs.
 int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 word, u64* kin, u32* vin, u64* kout,
-               u32* vout, u32 n, const PassPlan& plan, int* result_in_out, int* passes_run)
+               u32* vout, u32 n, const PassPlan& plan, int* result_in_out, int* passes_run, const u32* rank_src = nullptr,
+               u32 hop = 0)
 {
     csa_handle* h = L.h;
     hipStream_t s = L.stream;
@@ -405,7 +413,7 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
         return CSA_OK;
     // ghist[MAX_PASSES][256] followed by the two byte histograms of the text
     HIP_TRY(hipMemsetAsync(h->ghist, 0, (MAX_PASSES + 2) * RADIX_BINS * sizeof(u32), s));
-    if (src == SRC_PAIRS) {
+    if (src == SRC_PAIRS || src == SRC_RANKS) {
         HistArgs ha;
         ha.keys = kin;
         ha.vals = vin;
@@ -415,6 +423,10 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
         ha.word = word;
         ha.plan = plan;
         ha.ghist = h->ghist;
+        if (src == SRC_RANKS) {
+            ha.rank = rank_src;
+            ha.hop = hop;
+        }
         hipLaunchKernelGGL(radix_hist_kernel, dim3(hist_blocks(256 * 16, n)), dim3(256), 0, s, ha);
     } else {
         // every suffix of the text takes part and the plan is the eight bytes of one key word: the digit
@@ -465,6 +477,8 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
         a.lookback_groups = h->lookback + h->lookback_tile_words;
         a.epoch = next_epoch(h);
         a.err = h->counts + 2;
+        a.rank = rank_src;
+        a.hop = hop;
         int rc = next_ticket(L, &a.ticket);
         if (rc)
             return rc;
@@ -474,6 +488,8 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
         const int use_src = first ? src : SRC_PAIRS;
         if (use_src == SRC_PAIRS)
             launch_onesweep<SRC_PAIRS>(h, a, s);
+        else if (use_src == SRC_RANKS)
+            launch_onesweep<SRC_RANKS>(h, a, s);
         else
             launch_onesweep<SRC_TEXT>(h, a, s);
         if (timed) {
@@ -829,10 +845,12 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     // scratch of the bucketed rank update: all free while (and after) a list is being ranked
     // (the records of generation 0 start in the third key array and swap with the sort's other output array; the sorted
     // keys themselves are still being read when the first records are written)
-    const DeferBuffers defer_buf = {{bkey[0], key_out}, bx[0], bx[1], reinterpret_cast<u32*>(bkey[0]), reinterpret_cast<u32*>(bkey[1]),
-                                    reinterpret_cast<u32*>(bkey[1]) + h->cap};
+    auto defer_buffers = [&]() { // (by the roles the arrays have when it is asked for: a dense generation swaps two of them)
+        return DeferBuffers{{bkey[0], key_out}, bx[0], bx[1], reinterpret_cast<u32*>(bkey[0]), reinterpret_cast<u32*>(bkey[1]),
+                            reinterpret_cast<u32*>(bkey[1]) + h->cap};
+    };
     u32 m = 0, groups = 0, big = 0;
-    rc = rerank_step(L, ra, defer_buf, &m, &groups, &st->rank_update[0]);
+    rc = rerank_step(L, ra, defer_buffers(), &m, &groups, &st->rank_update[0]);
     range_gen0.close();
     if (rc)
         return rc;
@@ -855,6 +873,62 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
         st->groups[gen] = groups;
         const u32 m_in = m;
         RangeScope range_g("generation %d m=%u groups=%u", gen, m, groups);
+        const u64 hop = ctx < wide_ell ? (ctx < wide_ell - ctx ? ctx : wide_ell - ctx) : ctx;
+        // A dense generation: most of the partition is still active and its groups are long (a small alphabet, a
+        // periodic text), so nearly every member would go through the radix sort anyway. Then the whole partition is sorted
+        // again, as in generation 0, by keys that are read in text order: (rank[x], rank[x + hop]) for x = 0, 1, ...,
+        // two coalesced streams instead of one random gather per member; the ranks come out of the same run ranking as
+        // in generation 0 and go back to rank[] through the bucketed update instead of scattered writes. Suffixes that had
+        // retired are alone with their rank: they sort to the place they hold already and keep their rank.
+        const bool dense = (u64)m_in * 5 >= (u64)n * 3 && (u64)m_in > (u64)groups * SMALL_MAXG_HI && (u64)m_in >= DENSE_MIN;
+        if (dense) {
+            PassPlan plan; // the digits of the two ranks of a key: bits [0, sec_bits) and [32, 32 + sec_bits)
+            plan.num_passes = 0;
+            for (int half = 0; half < 2; ++half)
+                for (int b = 0; b < sec_bits; b += RADIX_BITS) {
+                    plan.shift[plan.num_passes] = 32 * half + b;
+                    plan.bits[plan.num_passes] = sec_bits - b < RADIX_BITS ? sec_bits - b : RADIX_BITS;
+                    plan.num_passes++;
+                }
+            passes = 0;
+            rc = radix_sort(L, SRC_RANKS, nullptr, n, 0, 0, bkey[0], bx[0], bkey[1], bx[1], n, plan, &in_out, &passes, h->rank, (u32)hop);
+            if (rc)
+                return rc;
+            RerankArgs rd;
+            memset(&rd, 0, sizeof(rd));
+            rd.keys = bkey[in_out];
+            rd.sufs = bx[in_out];
+            rd.m = n;
+            rd.key_words = 1;
+            rd.n = n;
+            rd.ell = 0; // no suffix is set apart for running off the text: the tied ones never do, the others are alone anyway
+            rd.text = d_text;
+            rd.rank = h->rank;
+            rd.sufs_out = ax;
+            rd.gids_out = agid;
+            rd.gprim_out = h->gprim[gp ^ 1];
+            rd.gstart_out = h->gstart[gp ^ 1];
+            DeferBuffers db = defer_buffers();
+            db.recs[0] = bkey[in_out ^ 1]; // the records of the rank update: the two 8-byte arrays that do not hold the sorted keys
+            db.recs[1] = key_out;
+            rc = rerank_step(L, rd, db, &m, &groups, &st->rank_update[gen]);
+            if (rc)
+                return rc;
+            // the freshly sorted index array is the suffix array under construction from here on; the old one is scratch
+            u32* const old_sa32 = sa32;
+            sa32 = bx[in_out];
+            bx[in_out] = old_sa32;
+            big = m_in;
+            st->big[gen] = m_in;
+            st->passes[gen] = passes;
+            st->dense[gen] = 1;
+            all_small = false;
+            gp ^= 1;
+            HIP_TRY(hipEventRecord(h->ev_gen[gen + 1], s));
+            gen++;
+            ctx += hop;
+            continue;
+        }
         const RankTables r = rank_tables(h, m_in, SMALL_TILE);
         u32* nr_list = reinterpret_cast<u32*>(key_out); // refined rank at every place of the sorted list
         // 1. gather rank[x + h]; small groups are sorted and ranked inside their tile, members of large groups set aside
@@ -867,7 +941,6 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
         sa.rank = h->rank;
         sa.m = m_in;
         sa.n = n;
-        const u64 hop = ctx < wide_ell ? (ctx < wide_ell - ctx ? ctx : wide_ell - ctx) : ctx;
         sa.h = (u32)hop;
         sa.sec_bits = sec_bits;
         sa.groups = groups;
@@ -956,6 +1029,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
         aa.m = m_in;
         aa.n = n;
         aa.rank = h->rank;
+        const DeferBuffers defer_buf = defer_buffers();
         aa.rank_vals = st->rank_update[gen] == 2 ? defer_buf.vals : nullptr;
         aa.sa32 = sa32;
         aa.sufs_out = ax;
@@ -1017,11 +1091,12 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
             st->passes[g] = st->passes[g + merged];
             st->rank_update[g] = st->rank_update[g + merged];
             st->small_only[g] = st->small_only[g + merged];
+            st->dense[g] = st->dense[g + merged];
             st->ms[g] = st->ms[g + merged];
         }
         for (int g = gen - merged; g < gen; ++g) {
             st->active[g] = st->groups[g] = st->big[g] = 0;
-            st->passes[g] = st->rank_update[g] = st->small_only[g] = 0;
+            st->passes[g] = st->rank_update[g] = st->small_only[g] = st->dense[g] = 0;
             st->ms[g] = 0.0f;
         }
         st->generations = gen - merged;

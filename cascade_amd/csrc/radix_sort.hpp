@@ -26,8 +26,17 @@ struct PassPlan {
 // How a pass obtains its input pairs.
 enum : int {
     SRC_PAIRS = 0, // keys_in[i], vals_in[i]
-    SRC_TEXT = 1   // generation 0, first pass: the pair of virtual position i is built from the text
+    SRC_TEXT = 1,  // generation 0, first pass: the pair of virtual position i is built from the text
+    SRC_RANKS = 2  // a dense later generation, first pass: pair i = ((rank[i], rank[i + hop]), i), built from rank[]
 };
+
+// Key of text position i in a dense generation: its rank, then the rank of the suffix `hop` symbols on (0 past the
+// end of the text; no tied suffix reaches there).
+__device__ __forceinline__ u64 rank_pair_key(const u32* __restrict__ rank, u32 n, u32 hop, u32 i)
+{
+    const u64 j = (u64)i + hop;
+    return ((u64)rank[i] << 32) | (u64)(j < (u64)n ? rank[j] : 0u);
+}
 
 // Generation 0 feeds the suffixes in the order (n-1, n-2, ..., n-tail, 0, 1, ..., n-tail-1): the last
 // `tail` suffixes run off the text inside their key, must each stay a group of one and sort
@@ -48,6 +57,8 @@ struct HistArgs {
     u32 word;   // key word to build from the text
     PassPlan plan;
     u32* ghist; // [MAX_PASSES][256], zeroed by the caller
+    const u32* rank = nullptr; // non-null: the keys are rank_pair_key(rank, n, hop, i) instead of keys[i]
+    u32 hop = 0;
 };
 
 // Digit counters live in LDS as hist[pass][bin][copy]: a lane adds to copy (lane % COPIES), so the lanes of
@@ -64,7 +75,7 @@ __global__ __launch_bounds__(256) void radix_hist_kernel(HistArgs a)
     const u32 copy = threadIdx.x & (HIST_COPIES - 1);
     const u64 stride = (u64)gridDim.x * 256;
     for (u64 i = (u64)blockIdx.x * 256 + threadIdx.x; i < a.n; i += stride) {
-        const u64 key = a.keys[i];
+        const u64 key = a.rank ? rank_pair_key(a.rank, a.n, a.hop, (u32)i) : a.keys[i];
         for (int p = 0; p < a.plan.num_passes; ++p) {
             const u32 d = (u32)(key >> a.plan.shift[p]) & ((1u << a.plan.bits[p]) - 1u);
             atomicAdd(&s_hist[(p * RADIX_BINS + d) * HIST_COPIES + copy], 1u);
@@ -184,6 +195,8 @@ struct OnesweepArgs {
     u32 tiles;             // tiles of the pass = workgroups of the launch
     u32 epoch;
     u32* err;
+    const u32* rank = nullptr; // SRC_RANKS: rank[] by text position ...
+    u32 hop = 0;               // ... and the distance to the second rank of a key
 };
 
 // How the workgroups of a radix pass come by their tiles (one each). Whatever the order, a tile waits for the tiles
@@ -238,11 +251,12 @@ __device__ __forceinline__ u32 onesweep_tile_number(const OnesweepArgs& a)
 template <typename KeyT, int BLOCK, int ITEMS, int SRC, int HI, bool VALS = true>
 __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(OnesweepArgs a)
 {
-    static_assert(VALS || SRC == SRC_PAIRS, "the text pass makes the suffix indices");
+    static_assert(VALS || SRC == SRC_PAIRS, "the passes that build their keys make the suffix indices");
     constexpr int TILE = BLOCK * ITEMS;
     constexpr int WAVES = BLOCK / WAVE;
     static_assert(BLOCK >= RADIX_BINS, "one thread per digit is assumed");
     static_assert(sizeof(KeyT) == 8 || (SRC == SRC_PAIRS && HI == 0), "narrow keys are plain pairs");
+    auto rank_key = [&](u32 i) -> u64 { return rank_pair_key(a.rank, a.n, a.hop, i); }; // SRC_RANKS: pair i is text position i
     const KeyT* __restrict__ keys_in = static_cast<const KeyT*>(a.keys_in);
     KeyT* __restrict__ keys_out = static_cast<KeyT*>(a.keys_out);
 
@@ -308,6 +322,8 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
             const u64 i = base + first_local + k * WAVE;
             if (SRC == SRC_PAIRS)
                 key[k] = keys_in[i];
+            else if (SRC == SRC_RANKS)
+                key[k] = (KeyT)rank_key((u32)i);
             else
                 key[k] = (KeyT)text_key((u32)i);
         }
@@ -320,6 +336,8 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
             if (local < valid) {
                 if (SRC == SRC_PAIRS)
                     key[k] = keys_in[i];
+                else if (SRC == SRC_RANKS)
+                    key[k] = (KeyT)rank_key((u32)i);
                 else
                     key[k] = (KeyT)text_key((u32)i);
             }
@@ -409,7 +427,9 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
         const u32 local = first_local + k * WAVE;
         val[k] = 0;
         if (VALS && local < valid)
-            val[k] = SRC == SRC_TEXT ? virtual_to_suffix((u32)(base + local), a.text_n, a.tail) : a.vals_in[base + local];
+            val[k] = SRC == SRC_TEXT    ? virtual_to_suffix((u32)(base + local), a.text_n, a.tail)
+                     : SRC == SRC_RANKS ? (u32)(base + local)
+                                        : a.vals_in[base + local];
     }
     // ---- write runs of equal digits to their global places ----
     u32 dst[ITEMS];

@@ -26,6 +26,7 @@ def stats_to_dict(st):
         "passes": [int(st.passes[i]) for i in range(g)],
         "rank_update": [int(st.rank_update[i]) for i in range(g)],
         "small_only": [int(st.small_only[i]) for i in range(g)],
+        "dense": [int(st.dense[i]) for i in range(g)],
         "ms": [float(st.ms[i]) for i in range(g)],
         "ms_output": float(st.ms_output),
         "ms_total": float(st.ms_total),

@@ -56,6 +56,8 @@ typedef struct csa_stats {
                                                  2 bucketed by one pass into cache-sized windows */
     int32_t small_only[CSA_MAX_GENERATIONS];  /* 1: generation g held small groups only and ran as two fused kernels
                                                  (in-tile sort + ranking + counting, then apply) without a radix sort */
+    int32_t dense[CSA_MAX_GENERATIONS];       /* 1: generation g > 0 sorted the whole partition again by (rank[x], rank[x + h])
+                                                 read in text order (most suffixes still active, in long groups) */
     float ms[CSA_MAX_GENERATIONS];        /* device time of generation g */
     float ms_output;                      /* sa40 emission */
     float ms_total;                       /* first kernel to last kernel, on the stream */

@@ -27,8 +27,8 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_stats_struct_layout_matches_header():
-    # 8 + 4 + 4 + 3 * 64*8 + 4 * 64*4 + 4 + 4 + 8 + 8 + 8
-    assert C.sizeof(_native.CsaStats) == 8 + 4 + 4 + 512 + 512 + 512 + 256 + 256 + 256 + 256 + 4 + 4 + 8 + 8 + 8
+    # 8 + 4 + 4 + 3 * 64*8 + 5 * 64*4 + 4 + 4 + 8 + 8 + 8
+    assert C.sizeof(_native.CsaStats) == 8 + 4 + 4 + 512 + 512 + 512 + 256 + 256 + 256 + 256 + 256 + 4 + 4 + 8 + 8 + 8
 
 
 def test_argument_errors_need_no_gpu():

@@ -55,6 +55,7 @@ def emu_sort(lib, T, key_words):
     assert rc == 0, lib.csa_last_error()
     emu_sort.rank_update = [int(st.rank_update[i]) for i in range(st.generations)]
     emu_sort.small_only = [int(st.small_only[i]) for i in range(st.generations)]
+    emu_sort.dense = [int(st.dense[i]) for i in range(st.generations)]
     return out[:5 * n], [int(st.active[i]) for i in range(st.generations)], [int(st.big[i]) for i in range(st.generations)]
 
 
@@ -118,6 +119,19 @@ def test_small_and_large_groups_take_both_paths(emu):
     # once a generation had no large group, the following ones run as the fused small-group generation
     first_small = big.index(0, 1)
     assert emu_sort.small_only == [0] * (first_small + 1) + [1] * (len(big) - first_small - 1) and 1 in emu_sort.small_only
+
+
+@pytest.mark.parametrize("name,key_words", [("one_symbol", 1), ("period_3", 4)])
+def test_dense_generations_sort_the_whole_partition_again(emu, name, key_words):
+    """Texts whose suffixes nearly all stay tied, in a handful of long groups, for many generations: those generations take
+    the dense form (keys (rank[x], rank[x + h]) read in text order, every suffix sorted again, ranks back through the
+    bucketed update). Same suffix array and the same active counts as the oracle's doubling, for plain and folded wide keys."""
+    T = {"one_symbol": np.full(3100, 7, dtype=np.uint16), "period_3": np.tile(np.array([3, 1, 4], dtype=np.uint16), 1040)}[name]
+    got, active, _ = emu_sort(emu, T, key_words)
+    sa, counts = oracle_lib.prefix_doubling(T, key_words)
+    assert np.array_equal(got, oracle_lib.u64_to_sa40(sa)) and active == counts
+    assert emu_sort.dense[0] == 0 and sum(emu_sort.dense) >= 5 and emu_sort.dense[-1] == 0
+    assert all(u == 1 for u, d in zip(emu_sort.rank_update, emu_sort.dense) if d)
 
 
 def test_emulated_radix_sort_matches_stable_sort(emu):

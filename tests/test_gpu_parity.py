@@ -276,13 +276,20 @@ def test_sixteen_million_symbols_pass_the_oracle_verifier(torch_mod, config, exc
         got = out.cpu().numpy()
         how = s.last_stats["rank_update"]
         fused = s.last_stats["small_only"]
+        dense = s.last_stats["dense"]
     assert oracle_lib.is_correct_sa40(got, T)
     assert how[0] == 1  # generation 0 went through the two-pass bucketed rank update
     assert fused[0] == 0
     if config in (3, 4):  # their late generations hold small groups only (the long runs of config 5 never do)
         assert fused[-1] == 1
-    if config == 4:     # four letters: nearly every rank changes in generation 1, which takes the one-pass kind
+    if config == 4:
+        # four letters: after generation 0 every suffix is still active, in 256 and then 65536 long groups: those two
+        # generations sort the whole partition again from rank[] (and write their ranks through the bucketed update);
+        # the next one, whose groups are short, changes most of its ranks and takes the one-pass kind of update
+        assert dense[:4] == [0, 1, 1, 0] and how[1] == 1 and how[2] == 1
         assert 2 in how[1:] and 0 in how[1:]
+    else:
+        assert not any(dense)
 
 
 def test_random_small_texts_against_the_oracle(torch_mod):
