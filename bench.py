@@ -352,7 +352,8 @@ def bench_next_rows(args):
         _, packed, _ = partition_ids(d_text, torch.from_numpy(pivots.view(np.int64)).to(dev).reshape(-1, 2), p, want_ids=False)
         suf = torch.randperm(n, device=dev)
         lanes = torch.stack([(suf >> (8 * b)) & 0xFF for b in range(5)], dim=1).to(torch.uint8).reshape(-1).contiguous()
-        keys, beta = stage_slab(d_text, lanes, 1, packed, p, 4, True)
+        kw = args.key_words
+        keys, beta = stage_slab(d_text, lanes, kw, packed, p, 4 * kw, True)
         sorter = PartitionSorter(n)
         rank_out = torch.empty(n, dtype=torch.int32, device=dev)
         suf_out = torch.empty(5 * n, dtype=torch.uint8, device=dev)
@@ -360,23 +361,23 @@ def bench_next_rows(args):
         off = torch.zeros(p + 1, dtype=torch.int32, device=dev)
         res = StepResult()
         st = torch.cuda.current_stream(dev).cuda_stream
-        init = lambda: _native.check(lib.csa_sort_init_dev(sorter._h, keys.data_ptr(), 1, lanes.data_ptr(), beta.data_ptr(), n, p,
+        init = lambda: _native.check(lib.csa_sort_init_dev(sorter._h, keys.data_ptr(), kw, lanes.data_ptr(), beta.data_ptr(), n, p,
                                                             rank_out.data_ptr(), suf_out.data_ptr(), mt.data_ptr(), mr.data_ptr(),
                                                             off.data_ptr(), st, C.byref(res)))
         if args.row == "step_init":
             ms, _ = _timed(torch, init, args.steps, args.warmup)
             # the whole text as one partition: its step-0 ranks are those of the resident sort's generation 0, so as many
             # suffixes survive as the partition sort reports active after generation 0
-            check = PartitionSorter(n)
+            check = PartitionSorter(n, key_words=kw)
             check.sort(d_text)
             resident = check.last_stats["active"][1] if check.last_stats["generations"] > 1 else 0
             # with several partitions the forward tag (the partition of the suffix one context further) refines the order
             ok = int(res.active) == resident if p == 1 else int(res.active) <= resident
             check.close()
-            alg = n * (8 + 5 + 4 + 2 * 2 * 24 + 8 * 2 * 24 + 41 + 41 + 9)  # unpack, two tag passes, eight key passes, rank, split, narrow (src/GPU_SACA.cu:1157-1331)
+            alg = n * (8 * kw + 5 + 4 + 2 * 2 * 24 + 8 * kw * 2 * 24 + 41 + 41 + 9)  # unpack, two tag passes, eight passes per key word, rank, split, narrow (src/GPU_SACA.cu:1157-1331)
             res_row = _row_result("suffixes through a generation-0 partition step/sec at 1 GPU", workloads.NAMES[args.config], n, ms,
-                                  "csa_sort_init_dev (10 radix passes + glue)", alg,
-                                  {"partitions": p, "active_after": int(res.active), "messages": int(res.messages)}, args.steps, args.warmup, ok)
+                                  "csa_sort_init_dev (the reference: %d radix passes + glue)" % (2 + 8 * kw), alg,
+                                  {"partitions": p, "key_words": kw, "active_after": int(res.active), "messages": int(res.messages)}, args.steps, args.warmup, ok)
         else:
             init()
             a = int(res.active)

@@ -1470,26 +1470,86 @@ int csa_sort_init_dev(csa_handle* h, const uint64_t* d_keys, int key_words, cons
     hipStream_t s = L.stream;
     const u32 blocks = (u32)((m + 255) / 256);
     HIP_TRY(hipMemsetAsync(h->counts, 0, 4 * sizeof(u32), s));
-    // stable LSD sort by (key words, forward tag): the tag first, then the words from the least significant one
-    // (src/GPU_SACA.cu:1165-1227), always on (64-bit key, permutation) pairs
     u64* K[2] = {h->key[0], h->key[1]};
     u32* P[2] = {h->idx[0], h->idx[1]};
     int kc = 0, pc = 0; // the arrays that hold the current keys / permutation
-    hipLaunchKernelGGL(iota_kernel, dim3(blocks), dim3(256), 0, s, P[pc], m);
-    hipLaunchKernelGGL(tag_keys_kernel, dim3(blocks), dim3(256), 0, s, d_beta, m, K[kc]);
     int in_out = 0, passes = 0;
-    rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, K[kc], P[pc], K[kc ^ 1], P[pc ^ 1], (u32)m, make_plan(0, 16), &in_out, &passes);
-    if (rc)
-        return rc;
-    pc ^= in_out;
-    for (int w = key_words - 1; w >= 0; --w) {
-        hipLaunchKernelGGL(gather_u64_kernel, dim3(blocks), dim3(256), 0, s, (const u64*)d_keys, (const u32*)P[pc], m, (u32)key_words,
-                           (u32)w, K[0]);
+    hipLaunchKernelGGL(iota_kernel, dim3(blocks), dim3(256), 0, s, P[pc], m);
+    if (key_words == 1) {
+        // stable LSD sort by (key word, forward tag): the tag first, then the word (src/GPU_SACA.cu:1165-1227), on
+        // (64-bit key, permutation) pairs
+        hipLaunchKernelGGL(tag_keys_kernel, dim3(blocks), dim3(256), 0, s, d_beta, m, K[kc]);
+        rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, K[kc], P[pc], K[kc ^ 1], P[pc ^ 1], (u32)m, make_plan(0, 16), &in_out, &passes);
+        if (rc)
+            return rc;
+        pc ^= in_out;
+        hipLaunchKernelGGL(gather_u64_kernel, dim3(blocks), dim3(256), 0, s, (const u64*)d_keys, (const u32*)P[pc], m, 1u, 0u, K[0]);
         rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, K[0], P[pc], K[1], P[pc ^ 1], (u32)m, make_plan(0, 64), &in_out, &passes);
         if (rc)
             return rc;
         kc = in_out;
         pc ^= in_out;
+    } else {
+        // Wider keys: the same order, (key words, forward tag), reached from the most significant word. All suffixes are
+        // sorted by word 0 alone. Only those that tie with a neighbour on it can still change places, and only inside their
+        // run: they are taken out in order, sorted among themselves by (word 0, ..., word W - 1, tag) with the stable LSD
+        // passes of the reference (tag, then the words from the last, src/GPU_SACA.cu:1165-1227) and put back, in that
+        // order, at the places the tied entries held. Sorting every suffix on every word costs 2 + 8 W passes over the
+        // partition; this costs 8, plus 2 + 8 W over the tied ones.
+        hipLaunchKernelGGL(gather_u64_kernel, dim3(blocks), dim3(256), 0, s, (const u64*)d_keys, (const u32*)P[pc], m, (u32)key_words, 0u,
+                           K[0]);
+        rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, K[0], P[pc], K[1], P[pc ^ 1], (u32)m, make_plan(0, 64), &in_out, &passes);
+        if (rc)
+            return rc;
+        kc = in_out;
+        pc ^= in_out;
+        const RankTables r = rank_tables(h, (u32)m, STEP_TILE);
+        TieArgs ta;
+        ta.keys = K[kc];
+        ta.perm = P[pc];
+        ta.m = m;
+        ta.pos_out = h->idx[4];
+        ta.perm_out = h->idx[2];
+        ta.tile_agg = r.tile_agg;
+        ta.tile_splits = r.tile_splits;
+        ta.tile_prefix = r.tile_prefix;
+        ta.slab_total = r.slab_total;
+        ta.slab = r.slab;
+        ta.slabs = r.slabs;
+        ta.total_out = reinterpret_cast<unsigned long long*>(h->counts + 6);
+        hipLaunchKernelGGL((tie_kernel<false>), dim3(r.tiles), dim3(STEP_BLOCK), 0, s, ta);
+        hipLaunchKernelGGL(rerank_scan_kernel, dim3(r.slabs), dim3(1024), 0, s, r.tile_agg, r.tile_prefix, r.tiles, r.slab, r.slab_total,
+                           r.tile_splits);
+        hipLaunchKernelGGL((tie_kernel<true>), dim3(r.tiles), dim3(STEP_BLOCK), 0, s, ta);
+        HIP_TRY(hipGetLastError());
+        rc = read_counts(L, nullptr);
+        if (rc)
+            return rc;
+        const u64 tied = h->h_pinned[6];
+        if (tied > m)
+            return fail(CSA_ERR_INTERNAL, "csa_sort_init_dev: %llu of %llu suffixes counted as tied", (unsigned long long)tied, (unsigned long long)m);
+        if (tied > 0) {
+            const u32 tblocks = (u32)((tied + 255) / 256);
+            u64* SK[2] = {K[kc ^ 1], h->key[2]}; // the sorted word 0 stays in K[kc]
+            u32* SV[2] = {h->idx[2], h->idx[3]};
+            int sv = 0;
+            hipLaunchKernelGGL(gather_tag_keys_kernel, dim3(tblocks), dim3(256), 0, s, d_beta, (const u32*)SV[sv], tied, SK[0]);
+            rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, SK[0], SV[sv], SK[1], SV[sv ^ 1], (u32)tied, make_plan(0, 16), &in_out, &passes);
+            if (rc)
+                return rc;
+            sv ^= in_out;
+            for (int w = key_words - 1; w >= 0; --w) {
+                hipLaunchKernelGGL(gather_u64_kernel, dim3(tblocks), dim3(256), 0, s, (const u64*)d_keys, (const u32*)SV[sv], tied,
+                                   (u32)key_words, (u32)w, SK[0]);
+                rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, SK[0], SV[sv], SK[1], SV[sv ^ 1], (u32)tied, make_plan(0, 64), &in_out, &passes);
+                if (rc)
+                    return rc;
+                sv ^= in_out;
+            }
+            hipLaunchKernelGGL(scatter_u32_kernel, dim3(tblocks), dim3(256), 0, s, (const u32*)SV[sv], (const u32*)h->idx[4], tied, m, P[pc],
+                               h->counts + 2);
+            HIP_TRY(hipGetLastError());
+        }
     }
     // sorted: key word 0 in K[kc], the permutation in P[pc]
     u64* sorted_key1 = nullptr;

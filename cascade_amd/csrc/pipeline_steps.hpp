@@ -50,6 +50,109 @@ __global__ __launch_bounds__(256) void gather_u32_kernel(const u32* __restrict__
         dst[i] = src[perm[i]];
 }
 
+// keys[i] = forward tag of suffix perm[i]
+__global__ __launch_bounds__(256) void gather_tag_keys_kernel(const u32* __restrict__ beta, const u32* __restrict__ perm, u64 count,
+                                                              u64* __restrict__ keys)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i < count)
+        keys[i] = beta[perm[i]] >> 16;
+}
+
+// dst[pos[i]] = src[i] (pos strictly increasing: the places of the tied entries in the sorted list)
+__global__ __launch_bounds__(256) void scatter_u32_kernel(const u32* __restrict__ src, const u32* __restrict__ pos, u64 count, u64 m,
+                                                          u32* __restrict__ dst, u32* err)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= count)
+        return;
+    const u32 at = pos[i];
+    if (at < m)
+        dst[at] = src[i];
+    else
+        atomicExch(err, DEV_ERR_RERANK_RANGE);
+}
+
+// Entries of a list sorted by its first key word that tie with a neighbour on that word, compacted in order: their
+// places in the list and the suffixes (permutation entries) at those places. Only they can change places when the later
+// key words and the forward tag are taken into account, and they stay inside their run. Two launches around
+// rerank_scan_kernel (count, apply), like the rank step.
+struct TieArgs {
+    const u64* keys; // sorted
+    const u32* perm;
+    u64 m;
+    u32* pos_out;
+    u32* perm_out;
+    u32* tile_agg;    // [tiles][4]: slot 2 carries the count
+    u32* tile_splits; // [tiles]
+    const u32* tile_prefix;
+    const u32* slab_total;
+    u32 slab;
+    u32 slabs;
+    unsigned long long* total_out;
+};
+
+template <bool APPLY>
+__global__ __launch_bounds__(STEP_BLOCK) void tie_kernel(TieArgs a)
+{
+    constexpr int WAVES = STEP_BLOCK / WAVE;
+    __shared__ u32 s_w[WAVES];
+    const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
+    const u32 tile = blockIdx.x;
+    const u64 base = (u64)tile * STEP_TILE + (u64)t * STEP_ITEMS;
+    u64 key[STEP_ITEMS + 2]; // entries base - 1 .. base + STEP_ITEMS
+#pragma unroll
+    for (int k = 0; k < STEP_ITEMS + 2; ++k) {
+        const u64 c = base + k;
+        key[k] = (c >= 1 && c - 1 < a.m) ? a.keys[c - 1] : 0;
+    }
+    u32 tied = 0, cnt = 0;
+#pragma unroll
+    for (int k = 0; k < STEP_ITEMS; ++k) {
+        const u64 i = base + k;
+        if (i < a.m) {
+            const bool left = i >= 1 && key[k] == key[k + 1], right = i + 1 < a.m && key[k + 2] == key[k + 1];
+            if (left || right) {
+                tied |= 1u << k;
+                cnt++;
+            }
+        }
+    }
+    const u32 ic = wave_incl_sum(cnt);
+    if (lane == 63u)
+        s_w[w] = ic;
+    __syncthreads();
+    u32 before = ic - cnt, total = 0;
+    for (u32 ww = 0; ww < WAVES; ++ww) {
+        if (ww < w)
+            before += s_w[ww];
+        total += s_w[ww];
+    }
+    if (!APPLY) {
+        if (t == 0) {
+            a.tile_agg[(u64)tile * 4 + 0] = 0;
+            a.tile_agg[(u64)tile * 4 + 1] = 0;
+            a.tile_agg[(u64)tile * 4 + 2] = total;
+            a.tile_agg[(u64)tile * 4 + 3] = 0;
+            a.tile_splits[tile] = 0;
+        }
+        return;
+    }
+    u32 at = a.tile_prefix[(u64)tile * 4 + 2] + slabs_before(a.slab_total, tile / a.slab).sum2 + before;
+    const u32 all = slabs_before(a.slab_total, a.slabs).sum2;
+    if (tile == 0 && t == 0)
+        *a.total_out = all;
+#pragma unroll
+    for (int k = 0; k < STEP_ITEMS; ++k) {
+        if (tied & (1u << k)) {
+            const u64 i = base + k;
+            a.pos_out[at] = (u32)i;
+            a.perm_out[at] = a.perm[i];
+            at++;
+        }
+    }
+}
+
 // words[i] = suffix of lane perm[i] (or i), with the forward tag of its routing tags in the top 16 bits when with_tag
 // (reference: unpack_tagged_lanes_kernel / unpack_lanes_kernel, include/GPU_SACA.cuh:94-119); beta_out[i] = beta[perm[i]].
 __global__ __launch_bounds__(256) void unpack_words_kernel(const u8* __restrict__ lanes, const u32* __restrict__ beta,
