@@ -1433,12 +1433,13 @@ int check_step_args(csa_handle* h, const char* who, u64 m, u32 p, const void* a,
                     (unsigned long long)h->cap);
     if (m && (!a || !b || !c || !d))
         return fail(CSA_ERR_ARG, "%s: null buffer", who);
-    for (int i = 0; i < 2; ++i)
-        if (!h->step64[i]) {
-            const hipError_t e = hipMalloc((void**)&h->step64[i], (h->cap ? h->cap : 1) * sizeof(u64));
-            if (e != hipSuccess)
-                return fail(CSA_ERR_HIP, "%s: %s while allocating the step scratch", who, hipGetErrorString(e));
-        }
+    if (!h->step64[0]) { // one block: generation 0 also uses it as one array of 16-byte records
+        const u64 cap = h->cap ? h->cap : 1;
+        const hipError_t e = hipMalloc((void**)&h->step64[0], 2 * cap * sizeof(u64));
+        if (e != hipSuccess)
+            return fail(CSA_ERR_HIP, "%s: %s while allocating the step scratch", who, hipGetErrorString(e));
+        h->step64[1] = h->step64[0] + cap;
+    }
     return CSA_OK;
 }
 
@@ -1560,7 +1561,11 @@ int csa_sort_init_dev(csa_handle* h, const uint64_t* d_keys, int key_words, cons
     }
     u64* sorted_words = h->key[2];
     u32* sorted_beta = h->idx[2];
-    hipLaunchKernelGGL(unpack_words_kernel, dim3(blocks), dim3(256), 0, s, d_suf40, d_beta, (const u32*)P[pc], m, 1, sorted_words,
+    // the carried columns follow the permutation: lane and routing tags of a suffix are first put side by side in one
+    // 16-byte record (a streaming pass), so that the gather costs one random line per suffix instead of two
+    uint4* carried = reinterpret_cast<uint4*>(h->step64[0]);
+    hipLaunchKernelGGL(pack_carried_kernel, dim3(blocks), dim3(256), 0, s, d_suf40, d_beta, m, carried);
+    hipLaunchKernelGGL(gather_carried_kernel, dim3(blocks), dim3(256), 0, s, (const uint4*)carried, (const u32*)P[pc], m, sorted_words,
                        sorted_beta);
     HIP_TRY(hipGetLastError());
     return finish_partition_step<true>(L, K[kc], sorted_key1, d_keys, P[pc], key_words, sorted_words, sorted_beta, m, 4ull * (u64)key_words, p, h->step64[0],
@@ -1832,8 +1837,7 @@ void csa_destroy(csa_handle* h)
     (void)hipFree(h->ghist);
     (void)hipFree(h->digit_base);
     (void)hipFree(h->tickets);
-    (void)hipFree(h->step64[0]);
-    (void)hipFree(h->step64[1]);
+    (void)hipFree(h->step64[0]); // (both halves)
     (void)hipFree(h->counts);
     if (h->h_pinned)
         (void)hipHostFree(h->h_pinned);

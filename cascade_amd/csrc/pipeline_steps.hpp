@@ -173,6 +173,35 @@ __global__ __launch_bounds__(256) void unpack_words_kernel(const u8* __restrict_
         beta_out[i] = bt;
 }
 
+// carried[i] = (suffix of lane i with the forward tag in the top 16 bits, routing tags of suffix i): what generation 0
+// moves along with a suffix, in one 16-byte record
+__global__ __launch_bounds__(256) void pack_carried_kernel(const u8* __restrict__ lanes, const u32* __restrict__ beta, u64 count,
+                                                           uint4* __restrict__ carried)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= count)
+        return;
+    u64 v = 0;
+#pragma unroll
+    for (int b = 0; b < 5; ++b)
+        v |= (u64)lanes[5 * i + b] << (8 * b);
+    const u32 bt = beta[i];
+    v |= (u64)(bt >> 16) << 48;
+    carried[i] = make_uint4((u32)v, (u32)(v >> 32), bt, 0u);
+}
+
+// words[i], beta_out[i] = the record of suffix perm[i]
+__global__ __launch_bounds__(256) void gather_carried_kernel(const uint4* __restrict__ carried, const u32* __restrict__ perm, u64 count,
+                                                             u64* __restrict__ words, u32* __restrict__ beta_out)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= count)
+        return;
+    const uint4 r = carried[perm[i]];
+    words[i] = (u64)r.x | ((u64)r.y << 32);
+    beta_out[i] = r.z;
+}
+
 // Run ranking with the active / retired split, in the three launches of the rank step (count, rerank_scan_kernel, apply).
 // Generation 0: the list is sorted by (key words, forward tag); rank = offset of the head of the run of equal
 // (key, tag), stored as a plain rank (include/GPU_SACA.cuh:191-208). Generation t: the list is sorted by the composite
