@@ -94,10 +94,10 @@ def test_text_at_every_alignment_inside_an_eight_byte_word(emu, key_words):
     # the first pass stages the text with aligned 8-byte loads: the text may start anywhere inside such a word, and
     # its end (here a run of zeros, which ties with the key padding) anywhere too
     rng = np.random.default_rng(7)
-    backing = np.zeros(2600, dtype=np.uint16)
+    backing = np.zeros(1400, dtype=np.uint16)
     base_off = (-backing.ctypes.data // 2) % 4  # symbols to the next 8-byte boundary
     for off in range(4):
-        for n in (1301 + off, 1304):
+        for n in ((641 + off, 644) if key_words == 1 else (643 - off,)):
             T = backing[base_off + off:base_off + off + n]
             T[:] = rng.integers(0, 3, n)
             T[-5:] = 0
@@ -126,7 +126,7 @@ def test_dense_generations_sort_the_whole_partition_again(emu, name, key_words):
     """Texts whose suffixes nearly all stay tied, in a handful of long groups, for many generations: those generations take
     the dense form (keys (rank[x], rank[x + h]) read in text order, every suffix sorted again, ranks back through the
     bucketed update). Same suffix array and the same active counts as the oracle's doubling, for plain and folded wide keys."""
-    T = {"one_symbol": np.full(3100, 7, dtype=np.uint16), "period_3": np.tile(np.array([3, 1, 4], dtype=np.uint16), 1040)}[name]
+    T = {"one_symbol": np.full(1700, 7, dtype=np.uint16), "period_3": np.tile(np.array([3, 1, 4], dtype=np.uint16), 560)}[name]
     got, active, _ = emu_sort(emu, T, key_words)
     sa, counts = oracle_lib.prefix_doubling(T, key_words)
     assert np.array_equal(got, oracle_lib.u64_to_sa40(sa)) and active == counts
@@ -282,15 +282,15 @@ def test_multi_partition_pipeline_through_the_emulated_stage_kernels(emu, p, key
         assert gens >= 6 and sum(step[5] for step in log if step[0] >= 1) > 0  # pills travelled in later generations
 
 
-@pytest.mark.parametrize("p,key_words,sigma,n", [(5, 4, 2, 900), (4, 1, 2, 1300)])
+@pytest.mark.parametrize("p,key_words,sigma,n", [(5, 4, 2, 700), (4, 1, 2, 900)])
 def test_multi_partition_pipeline_with_the_emulated_step_entries(emu, p, key_words, sigma, n):
     """The same pipeline with each partition step as one call of csa_sort_init_dev / csa_sort_rerank_dev."""
     import multi_partition
     T = texts.random_text(n, sigma, 13 * p + n, sep_every=0)
     T[-7:] = 0
     if key_words == 1:  # long repeats: many generations, pills forwarded
-        T[500:900] = T[:400]
-        T[1000:1250] = T[100:350]
+        T[300:600] = T[:300]
+        T[650:850] = T[100:300]
     h = C.c_void_p()
     assert emu.csa_create(n, 1, C.byref(h)) == 0
     log, glue_log = [], []
@@ -305,14 +305,14 @@ def test_multi_partition_pipeline_with_the_emulated_step_entries(emu, p, key_wor
     assert log == glue_log
 
 
-@pytest.mark.parametrize("p,key_words,sigma,n,chunk_cap", [(3, 1, 3, 2000, 4096), (4, 2, 2, 1500, 4096)])
+@pytest.mark.parametrize("p,key_words,sigma,n,chunk_cap", [(3, 1, 3, 1400, 4096), (4, 2, 2, 1100, 4096)])
 def test_multi_partition_pipeline_through_the_emulated_slab_entries(emu, p, key_words, sigma, n, chunk_cap):
     """csa_sort_init_slabs / csa_sort_rerank_slabs / csa_scatter_slabs: every partition step takes and returns host slabs of
     ragged sizes (several per partition, some empty, the inbox shared out over them), the final permutation comes back cut
     into disk blocks and edges; the suffix array assembled from those pieces is the oracle's."""
     import multi_partition
     T = texts.random_text(n, sigma, 31 * p + n, sep_every=0)
-    T[n // 3:n // 3 + 700] = T[:700]
+    T[n // 3:n // 3 + 400] = T[:400]
     T[-5:] = 0
     h = C.c_void_p()
     assert emu.csa_create(n, 1, C.byref(h)) == 0
