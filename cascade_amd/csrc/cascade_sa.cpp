@@ -6,6 +6,9 @@
 
 #include <chrono>
 
+// every member of the builder class is compiled with the program, the per-partition members that it does not call included
+template class cascade_hip::GPU_SACA<std::uint16_t>;
+
 int main(int argc, char** argv)
 {
     using T_sym_ = std::uint16_t;
