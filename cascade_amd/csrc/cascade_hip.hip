@@ -427,7 +427,34 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
             ha.rank = rank_src;
             ha.hop = hop;
         }
-        hipLaunchKernelGGL(radix_hist_kernel, dim3(hist_blocks(256 * 16, n)), dim3(256), 0, s, ha);
+        // the two halves of a (rank[i], rank[i + hop]) key are the same array, one shifted by hop: when the plan takes
+        // the same digits from both halves, one histogram of rank[] and one of its first hop entries give them all
+        const int half = plan.num_passes / 2;
+        bool mirrored = src == SRC_RANKS && plan.num_passes == 2 * half && half >= 1 && half <= RANK_HIST_PASSES;
+        for (int p = 0; mirrored && p < half; ++p)
+            mirrored = plan.shift[p] + plan.bits[p] <= 32 && plan.shift[half + p] == 32 + plan.shift[p] && plan.bits[half + p] == plan.bits[p];
+        if (mirrored) {
+            RankHistArgs ra;
+            ra.rank = rank_src;
+            ra.num_passes = half;
+            for (int p = 0; p < half; ++p) {
+                ra.shift[p] = plan.shift[p];
+                ra.bits[p] = plan.bits[p];
+            }
+            const u32 cut = hop < n ? hop : n;
+            ra.begin = 0;
+            ra.end = n;
+            ra.out = h->ghist + half * RADIX_BINS;
+            hipLaunchKernelGGL(rank_hist_kernel, dim3(hist_blocks(256 * 16, n)), dim3(256), 0, s, ra);
+            if (cut > 0) {
+                ra.end = cut;
+                ra.out = h->ghist;
+                hipLaunchKernelGGL(rank_hist_kernel, dim3(hist_blocks(256 * 16, cut)), dim3(256), 0, s, ra);
+            }
+            hipLaunchKernelGGL(rank_hist_combine_kernel, dim3(1), dim3(256), 0, s, h->ghist, half, cut);
+        } else {
+            hipLaunchKernelGGL(radix_hist_kernel, dim3(hist_blocks(256 * 16, n)), dim3(256), 0, s, ha);
+        }
     } else {
         // every suffix of the text takes part and the plan is the eight bytes of one key word: the digit
         // histograms follow from the byte histogram of the text, whatever order the pairs are in

@@ -92,6 +92,59 @@ __global__ __launch_bounds__(256) void radix_hist_kernel(HistArgs a)
     }
 }
 
+// Digit histograms of rank[begin .. end): out[p][d] counts the entries whose digit (rank >> shift[p]) & mask[p] is d, for up
+// to four digits of a 32-bit rank. The keys (rank[i], rank[i + hop]) of a dense generation need no histogram of their own:
+// their high halves are rank[0 .. n), their low halves rank[hop .. n) and min(hop, n) zeros (rank_hist_combine_kernel).
+constexpr int RANK_HIST_PASSES = 4;
+constexpr int RANK_HIST_COPIES = 16;
+
+struct RankHistArgs {
+    const u32* rank;
+    u32 begin, end;
+    int num_passes; // <= RANK_HIST_PASSES
+    int shift[RANK_HIST_PASSES];
+    int bits[RANK_HIST_PASSES];
+    u32* out; // [num_passes][256], zeroed by the caller
+};
+
+__global__ __launch_bounds__(256) void rank_hist_kernel(RankHistArgs a)
+{
+    __shared__ u32 s_hist[RANK_HIST_PASSES * RADIX_BINS * RANK_HIST_COPIES];
+    for (int i = threadIdx.x; i < RANK_HIST_PASSES * RADIX_BINS * RANK_HIST_COPIES; i += 256)
+        s_hist[i] = 0;
+    __syncthreads();
+    const u32 copy = threadIdx.x & (RANK_HIST_COPIES - 1);
+    const u64 stride = (u64)gridDim.x * 256;
+    for (u64 i = (u64)a.begin + (u64)blockIdx.x * 256 + threadIdx.x; i < a.end; i += stride) {
+        const u32 r = a.rank[i];
+        for (int p = 0; p < a.num_passes; ++p) {
+            const u32 d = (r >> a.shift[p]) & ((1u << a.bits[p]) - 1u);
+            atomicAdd(&s_hist[(p * RADIX_BINS + d) * RANK_HIST_COPIES + copy], 1u);
+        }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < a.num_passes * RADIX_BINS; i += 256) {
+        u32 v = 0;
+#pragma unroll
+        for (int c = 0; c < RANK_HIST_COPIES; ++c)
+            v += s_hist[i * RANK_HIST_COPIES + c];
+        if (v)
+            atomicAdd(&a.out[i], v);
+    }
+}
+
+// ghist rows [half, 2 half) hold the histograms of rank[0 .. n) (the high halves of the keys), rows [0, half) those of
+// rank[0 .. cut), cut = min(hop, n). Rows [0, half) become the histograms of the low halves: all entries but the first
+// cut, plus cut zeros.
+__global__ __launch_bounds__(256) void rank_hist_combine_kernel(u32* ghist, int half, u32 cut)
+{
+    const u32 d = threadIdx.x;
+    for (int p = 0; p < half; ++p) {
+        const u32 all = ghist[(half + p) * RADIX_BINS + d], head = ghist[p * RADIX_BINS + d];
+        ghist[p * RADIX_BINS + d] = all - head + (d == 0 ? cut : 0u);
+    }
+}
+
 // Histogram of the low and of the high byte of every symbol of the text: bytehist[0][d], bytehist[1][d].
 // The eight digit histograms of a K-gram key word follow from these two (text_hist_expand_kernel).
 constexpr int TEXT_HIST_COPIES = 16;
