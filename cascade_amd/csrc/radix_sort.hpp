@@ -73,12 +73,31 @@ __global__ __launch_bounds__(256) void radix_hist_kernel(HistArgs a)
         s_hist[i] = 0;
     __syncthreads();
     const u32 copy = threadIdx.x & (HIST_COPIES - 1);
-    const u64 stride = (u64)gridDim.x * 256;
-    for (u64 i = (u64)blockIdx.x * 256 + threadIdx.x; i < a.n; i += stride) {
-        const u64 key = a.rank ? rank_pair_key(a.rank, a.n, a.hop, (u32)i) : a.keys[i];
+    // four keys per thread and round, as two 16-byte loads where they all exist: a thread with one 8-byte load in
+    // flight per round leaves the kernel waiting on latency (1.6 TB/s)
+    const bool aligned16 = (reinterpret_cast<uintptr_t>(a.keys) & 15u) == 0; // a caller's array need not be
+    const u64 stride = (u64)gridDim.x * 256 * 4;
+    for (u64 i = ((u64)blockIdx.x * 256 + threadIdx.x) * 4; i < a.n; i += stride) {
+        u64 key[4];
+        const int have = a.n - i < 4 ? (int)(a.n - i) : 4;
+        if (!a.rank && have == 4 && aligned16) {
+            const uint4 lo = *reinterpret_cast<const uint4*>(a.keys + i), hi = *reinterpret_cast<const uint4*>(a.keys + i + 2);
+            key[0] = (u64)lo.x | ((u64)lo.y << 32);
+            key[1] = (u64)lo.z | ((u64)lo.w << 32);
+            key[2] = (u64)hi.x | ((u64)hi.y << 32);
+            key[3] = (u64)hi.z | ((u64)hi.w << 32);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                key[k] = k < have ? (a.rank ? rank_pair_key(a.rank, a.n, a.hop, (u32)(i + k)) : a.keys[i + k]) : 0;
+        }
         for (int p = 0; p < a.plan.num_passes; ++p) {
-            const u32 d = (u32)(key >> a.plan.shift[p]) & ((1u << a.plan.bits[p]) - 1u);
-            atomicAdd(&s_hist[(p * RADIX_BINS + d) * HIST_COPIES + copy], 1u);
+            const int sh = a.plan.shift[p];
+            const u32 mask = (1u << a.plan.bits[p]) - 1u;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (k < have)
+                    atomicAdd(&s_hist[(p * RADIX_BINS + ((u32)(key[k] >> sh) & mask)) * HIST_COPIES + copy], 1u);
         }
     }
     __syncthreads();
@@ -114,12 +133,27 @@ __global__ __launch_bounds__(256) void rank_hist_kernel(RankHistArgs a)
         s_hist[i] = 0;
     __syncthreads();
     const u32 copy = threadIdx.x & (RANK_HIST_COPIES - 1);
-    const u64 stride = (u64)gridDim.x * 256;
-    for (u64 i = (u64)a.begin + (u64)blockIdx.x * 256 + threadIdx.x; i < a.end; i += stride) {
-        const u32 r = a.rank[i];
+    // eight ranks per thread and round (two 16-byte loads where they all exist and are aligned)
+    const bool aligned16 = (reinterpret_cast<uintptr_t>(a.rank + a.begin) & 15u) == 0;
+    const u64 stride = (u64)gridDim.x * 256 * 8;
+    for (u64 i = (u64)a.begin + ((u64)blockIdx.x * 256 + threadIdx.x) * 8; i < a.end; i += stride) {
+        u32 r[8];
+        const int have = a.end - i < 8 ? (int)(a.end - i) : 8;
+        if (have == 8 && aligned16) {
+            const uint4 lo = *reinterpret_cast<const uint4*>(a.rank + i), hi = *reinterpret_cast<const uint4*>(a.rank + i + 4);
+            r[0] = lo.x, r[1] = lo.y, r[2] = lo.z, r[3] = lo.w, r[4] = hi.x, r[5] = hi.y, r[6] = hi.z, r[7] = hi.w;
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                r[k] = k < have ? a.rank[i + k] : 0u;
+        }
         for (int p = 0; p < a.num_passes; ++p) {
-            const u32 d = (r >> a.shift[p]) & ((1u << a.bits[p]) - 1u);
-            atomicAdd(&s_hist[(p * RADIX_BINS + d) * RANK_HIST_COPIES + copy], 1u);
+            const int sh = a.shift[p];
+            const u32 mask = (1u << a.bits[p]) - 1u;
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                if (k < have)
+                    atomicAdd(&s_hist[(p * RADIX_BINS + ((r[k] >> sh) & mask)) * RANK_HIST_COPIES + copy], 1u);
         }
     }
     __syncthreads();
