@@ -452,9 +452,24 @@ __global__ __launch_bounds__(256) void position_hist_kernel(const u32* __restric
     __syncthreads();
     const u32 copy = threadIdx.x & 7u;
     const u32 mask = (1u << bits) - 1u;
-    const u64 stride = (u64)gridDim.x * 256;
-    for (u64 i = (u64)blockIdx.x * 256 + threadIdx.x; i < m; i += stride)
-        atomicAdd(&s_hist[((pos[i] >> shift) & mask) * 8 + copy], 1u);
+    // four positions per thread and round (one 16-byte load where they all exist: the lists are 16-byte aligned)
+    const u64 stride = (u64)gridDim.x * 256 * 4;
+    for (u64 i = ((u64)blockIdx.x * 256 + threadIdx.x) * 4; i < m; i += stride) {
+        u32 x[4];
+        const int have = m - i < 4 ? (int)(m - i) : 4;
+        if (have == 4 && (reinterpret_cast<uintptr_t>(pos) & 15u) == 0) {
+            const uint4 v = *reinterpret_cast<const uint4*>(pos + i);
+            x[0] = v.x, x[1] = v.y, x[2] = v.z, x[3] = v.w;
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                x[k] = k < have ? pos[i + k] : 0u;
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            if (k < have)
+                atomicAdd(&s_hist[((x[k] >> shift) & mask) * 8 + copy], 1u);
+    }
     __syncthreads();
     for (int i = threadIdx.x; i < POS_BINS; i += 256) {
         u32 v = 0;

@@ -190,18 +190,22 @@ __global__ __launch_bounds__(256) void text_byte_hist_kernel(const u16* __restri
         s_hist[i] = 0;
     __syncthreads();
     const u32 copy = threadIdx.x & (TEXT_HIST_COPIES - 1);
-    const u64 stride = (u64)gridDim.x * 256 * 8;
-    for (u64 i = ((u64)blockIdx.x * 256 + threadIdx.x) * 8; i < n; i += stride) {
-        u16 sym[8];
-        if (i + 8 <= n) {
-            __builtin_memcpy(sym, text + i, 16); // 16-byte aligned: hipMalloc base + 16 * k
+    const u64 stride = (u64)gridDim.x * 256 * 16;
+    const bool aligned16 = (reinterpret_cast<uintptr_t>(text) & 15u) == 0;
+    for (u64 i = ((u64)blockIdx.x * 256 + threadIdx.x) * 16; i < n; i += stride) {
+        u16 sym[16];
+        if (i + 16 <= n && aligned16) { // two 16-byte loads in flight per thread
+            const uint4* p4 = reinterpret_cast<const uint4*>(text + i);
+            const uint4 v0 = p4[0], v1 = p4[1];
+            __builtin_memcpy(sym, &v0, 16);
+            __builtin_memcpy(sym + 8, &v1, 16);
         } else {
 #pragma unroll
-            for (int k = 0; k < 8; ++k)
+            for (int k = 0; k < 16; ++k)
                 sym[k] = i + k < n ? text[i + k] : 0;
         }
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
+        for (int k = 0; k < 16; ++k) {
             if (i + k < n) {
                 atomicAdd(&s_hist[(0 * RADIX_BINS + (sym[k] & 0xFFu)) * TEXT_HIST_COPIES + copy], 1u);
                 atomicAdd(&s_hist[(1 * RADIX_BINS + (sym[k] >> 8)) * TEXT_HIST_COPIES + copy], 1u);
