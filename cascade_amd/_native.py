@@ -13,6 +13,7 @@ CSA_MAX_PART_SZ = 2147483647
 CSA_MAX_INDEX = 1 << 40
 CSA_OK, CSA_ERR_ARG, CSA_ERR_TOO_LARGE, CSA_ERR_HIP, CSA_ERR_INTERNAL = 0, -1, -2, -3, -4
 CSA_FLAG_KERNEL_TIMING = 1
+CSA_TUNE_DEFER_MIN, CSA_TUNE_WINDOW_MIN_CHANGED, CSA_TUNE_XCD_CHUNK = 0, 1, 2
 
 # every symbol include/cascade_hip.h declares
 EXPORTS = (
@@ -21,7 +22,7 @@ EXPORTS = (
     "csa_partition_id_bits", "csa_partition_ids_u16_dev", "csa_scatter_to_rank_order_dev", "csa_output_cut",
     "csa_stage_slab_u16_dev", "csa_count_messages_dev", "csa_message_offsets_dev", "csa_emit_messages_dev",
     "csa_join_messages_dev", "csa_join_messages_sorted_dev", "csa_sort_init_dev", "csa_sort_rerank_dev",
-    "csa_set_device_exclusive", "csa_radix_sort_pairs_static_dev", "csa_enable_profile_ranges",
+    "csa_set_device_exclusive", "csa_set_tuning", "csa_radix_sort_pairs_static_dev", "csa_enable_profile_ranges",
     "csa_slab_bytes_per_suffix", "csa_sort_init_slabs", "csa_sort_rerank_slabs", "csa_scatter_slabs", "csa_sort_partitions_u16",
 )
 
@@ -85,6 +86,8 @@ def load():
     lib.csa_destroy.argtypes = [vp]
     lib.csa_set_device_exclusive.restype = C.c_int
     lib.csa_set_device_exclusive.argtypes = [vp, C.c_int]
+    lib.csa_set_tuning.restype = C.c_int
+    lib.csa_set_tuning.argtypes = [vp, C.c_int, C.c_uint32]
     lib.csa_sort_partition_u16_dev.restype = i32
     lib.csa_sort_partition_u16_dev.argtypes = [vp, vp, u64, u64, vp, vp, u32, C.POINTER(CsaStats)]
     lib.csa_sort_partition_u16.restype = i32

@@ -293,10 +293,10 @@ struct csa_handle {
     u32 tile_order = TILES_BY_ARRIVAL;           // how the radix passes number their tiles (radix_sort.hpp), in use
     u32 tile_order_exclusive = TILES_BY_ARRIVAL; // the order after csa_set_device_exclusive
     u32 xcd_chunk = XCD_CHUNK;                   // tiles of a radix pass that one XCD takes in a row under TILES_STATIC_CHUNKS
-    u32 defer_min = DEFER_MIN; // lists at least this long use the bucketed rank update (env CASCADE_DEFER_MIN overrides)
+    u32 defer_min = DEFER_MIN; // lists at least this long use the bucketed rank update (csa_set_tuning)
     u64* step64[2] = {nullptr, nullptr}; // two more 8-byte arrays of the capacity, for the per-generation partition steps
     SlabArena* slab_arena = nullptr;     // allocated by the first call of a slab-shaped entry
-    u32 window_min_changed = WINDOW_MIN_CHANGED; // env CASCADE_WINDOW_MIN_CHANGED overrides (0xFFFFFFFF: never)
+    u32 window_min_changed = WINDOW_MIN_CHANGED; // csa_set_tuning (0xFFFFFFFF: never)
     std::vector<hipEvent_t> events;
     hipEvent_t ev_gen[CSA_MAX_GENERATIONS + 2] = {};
     bool ev_gen_ready = false;
@@ -1767,10 +1767,6 @@ int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
     csa_handle* h = new csa_handle();
     h->cap = max_part_sz ? max_part_sz : 1;
     h->key_words = key_words;
-    if (const char* e = getenv("CASCADE_DEFER_MIN"))
-        h->defer_min = (u32)strtoul(e, nullptr, 10);
-    if (const char* e = getenv("CASCADE_WINDOW_MIN_CHANGED"))
-        h->window_min_changed = (u32)strtoul(e, nullptr, 10);
     const u64 cap = h->cap;
     const u64 sort_tiles = (cap + SORT_TILE - 1) / SORT_TILE;
     const u64 rank_tiles = (cap + RANK_TILE - 1) / RANK_TILE;
@@ -1784,17 +1780,10 @@ int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
         e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, h->device);
     // Tile order of the radix passes: by arrival, unless the caller declares the device its own
     // (csa_set_device_exclusive); the XCD-chunked order then needs 8 * XCD_CHUNK workgroups of a pass resident at once
-    // and is offered only on a device with room for twice that many. CASCADE_XCD_CHUNK overrides the chunk length
-    // (0: never chunked), for experiments and for the CPU emulation's test of the failure path.
+    // and is offered only on a device with room for twice that many (csa_set_tuning changes the chunk length).
     h->tile_order = TILES_BY_ARRIVAL;
     h->tile_order_exclusive = cus >= 2 * 8 * (int)XCD_CHUNK ? TILES_STATIC_CHUNKS : TILES_BY_ARRIVAL;
     h->xcd_chunk = XCD_CHUNK;
-    if (const char* c = getenv("CASCADE_XCD_CHUNK")) {
-        const u32 v = (u32)strtoul(c, nullptr, 10);
-        h->tile_order_exclusive = v ? TILES_STATIC_CHUNKS : TILES_BY_ARRIVAL;
-        if (v)
-            h->xcd_chunk = v;
-    }
     auto alloc = [&](void** p, u64 bytes) {
         if (e == hipSuccess)
             e = hipMalloc(p, bytes ? bytes : 4);
@@ -1833,6 +1822,25 @@ int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
         return rc;
     }
     *out = h;
+    return CSA_OK;
+}
+
+int csa_set_tuning(csa_handle* h, int knob, uint32_t value)
+{
+    if (!h)
+        return fail(CSA_ERR_ARG, "csa_set_tuning: null handle");
+    switch (knob) {
+    case CSA_TUNE_DEFER_MIN: h->defer_min = value; break;
+    case CSA_TUNE_WINDOW_MIN_CHANGED: h->window_min_changed = value; break;
+    case CSA_TUNE_XCD_CHUNK:
+        h->tile_order_exclusive = value ? TILES_STATIC_CHUNKS : TILES_BY_ARRIVAL;
+        if (value)
+            h->xcd_chunk = value;
+        if (h->tile_order != TILES_BY_ARRIVAL) // the handle is in the exclusive order already: follow
+            h->tile_order = h->tile_order_exclusive;
+        break;
+    default: return fail(CSA_ERR_ARG, "csa_set_tuning: unknown knob %d", knob);
+    }
     return CSA_OK;
 }
 

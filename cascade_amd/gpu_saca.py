@@ -54,6 +54,11 @@ class PartitionSorter:
         radix passes may then use the XCD-chunked tile order, which is not safe next to other launches."""
         _native.check(self._lib.csa_set_device_exclusive(self._h, 1 if exclusive else 0))
 
+    def set_tuning(self, knob, value):
+        """One of the thresholds that choose between equivalent ways of doing a step (csa_set_tuning; knob = one of
+        _native.CSA_TUNE_*)."""
+        _native.check(self._lib.csa_set_tuning(self._h, int(knob), int(value)))
+
     def close(self):
         if self._h:
             self._lib.csa_destroy(self._h)

@@ -92,6 +92,19 @@ int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out);
  * No counterpart in the reference (CUB's passes always number tiles by arrival). */
 int csa_set_device_exclusive(csa_handle* h, int exclusive);
 
+/* Thresholds that choose between equivalent ways of doing a step (the results are the same either way); for tests
+ * that want a path taken at small sizes and for measurements. The defaults are the measured best on MI355X.
+ *   CSA_TUNE_DEFER_MIN           smallest list whose generation-0 ranks are written through the two-pass bucketed update
+ *                                (default 2^23 suffixes)
+ *   CSA_TUNE_WINDOW_MIN_CHANGED  fewest changed ranks for the windowed update of later generations (default 2^22;
+ *                                0xFFFFFFFF: never)
+ *   CSA_TUNE_XCD_CHUNK           tiles (of 8192 pairs) that one XCD takes in a row under csa_set_device_exclusive
+ *                                (default 16; 0: the exclusive order is the default order); call before
+ *                                csa_set_device_exclusive
+ * No counterpart in the reference. */
+enum { CSA_TUNE_DEFER_MIN = 0, CSA_TUNE_WINDOW_MIN_CHANGED = 1, CSA_TUNE_XCD_CHUNK = 2 };
+int csa_set_tuning(csa_handle* h, int knob, uint32_t value);
+
 /* Frees everything the handle owns (reference: the destructor, src/GPU_SACA.cu:103-120). */
 void csa_destroy(csa_handle* h);
 

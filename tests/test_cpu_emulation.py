@@ -340,13 +340,13 @@ def test_step_entries_on_a_text_of_one_symbol(emu):
     assert np.array_equal(sa, np.arange(T.size - 1, -1, -1, dtype=np.uint64)), gens
 
 
-def test_chunked_tile_order_without_resident_workgroups_ends_in_an_error_not_a_hang(emu, monkeypatch):
+def test_chunked_tile_order_without_resident_workgroups_ends_in_an_error_not_a_hang(emu):
     # The XCD-chunked tile order of the radix pass waits for tiles whose workgroups are dispatched later. The emulator
     # runs one workgroup at a time, the extreme case of a device shared with other launches: the wait must run into
     # its spin limit, every later workgroup and kernel of the step must leave at once, and the call must report
     # CSA_ERR_INTERNAL. By default (no csa_set_device_exclusive) tiles are numbered by arrival and the same text sorts.
     emu.csa_set_device_exclusive.argtypes = [C.c_void_p, C.c_int]
-    monkeypatch.setenv("CASCADE_XCD_CHUNK", "16")
+    emu.csa_set_tuning.argtypes = [C.c_void_p, C.c_int, C.c_uint32]
     T = texts.random_text(140000, 5, 3, sep_every=0)  # 137 tiles of 1024 keys: one whole group of 8 chunks of 16
     n = T.size
     h = C.c_void_p()
@@ -354,6 +354,8 @@ def test_chunked_tile_order_without_resident_workgroups_ends_in_an_error_not_a_h
     out = np.zeros(5 * n + 8, dtype=np.uint8)
     st = _native.CsaStats()
     try:
+        # (the emulated device has too few compute units for the chunked order to be offered by itself)
+        assert emu.csa_set_tuning(h, _native.CSA_TUNE_XCD_CHUNK, 16) == 0
         assert emu.csa_set_device_exclusive(h, 1) == 0
         rc = emu.csa_sort_partition_u16_dev(h, T.ctypes.data, n, 0, out.ctypes.data, None, 0, C.byref(st))
         assert rc == -4 and b"spin limit" in emu.csa_last_error(), (rc, emu.csa_last_error())

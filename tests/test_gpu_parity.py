@@ -340,15 +340,13 @@ def test_random_small_texts_against_the_oracle(torch_mod):
         assert np.array_equal(got, oracle_lib.build_sa40(T)), (case, n, sigma, kw)
 
 
-def test_bucketed_rank_updates_at_small_and_ragged_sizes(torch_mod, monkeypatch):
+def test_bucketed_rank_updates_at_small_and_ragged_sizes(torch_mod):
     """The bucketed rank updates normally serve lists of millions of suffixes: generation 0 sends (position, rank)
     records through value-less radix passes and a window placement, later generations (position, rank) pairs through one
-    pass and a windowed scatter. With their thresholds at 1 (read when a handle is made) every list takes them: sizes
+    pass and a windowed scatter. With their thresholds at 1 (csa_set_tuning) every list takes them: sizes
     around the tile, window and pass boundaries, checked against the oracle, and the library must report that it went
     that way."""
-    from cascade_amd import PartitionSorter, workloads
-    monkeypatch.setenv("CASCADE_DEFER_MIN", "1")
-    monkeypatch.setenv("CASCADE_WINDOW_MIN_CHANGED", "1")
+    from cascade_amd import PartitionSorter, workloads, _native
     rng = np.random.default_rng(77)
     sizes = [1, 2, 5, 255, 1024, 1025, 8191, 8193, (1 << 14) - 1, 1 << 14, (1 << 14) + 1, 16385 * 3, (1 << 16) + 7,
              (1 << 18) - 3, (1 << 20) + 11]
@@ -361,6 +359,8 @@ def test_bucketed_rank_updates_at_small_and_ragged_sizes(torch_mod, monkeypatch)
             T = workloads.generate(5, n) if n >= 64 else np.zeros(n, dtype=np.uint16)
         with PartitionSorter(n, key_words=1 + case % 2) as s:
             print(f"  bucketed case={case} n={n} key_words={s.key_words}", flush=True)
+            s.set_tuning(_native.CSA_TUNE_DEFER_MIN, 1)
+            s.set_tuning(_native.CSA_TUNE_WINDOW_MIN_CHANGED, 1)
             got = s.sort(to_dev(torch_mod, T)).cpu().numpy()
             how = s.last_stats["rank_update"]
         if n <= 1 << 16:
