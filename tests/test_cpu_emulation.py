@@ -157,7 +157,7 @@ def test_emulated_radix_sort_without_allocation_matches_the_one_with_a_handle(em
     rng = np.random.default_rng(4)
     h = C.c_void_p()
     assert emu.csa_create(20000, 1, C.byref(h)) == 0
-    for n, b, e in ((17000, 0, 64), (3001, 5, 29), (1, 0, 64), (1024, 8, 24)):
+    for n, b, e in ((9000, 0, 40), (3001, 5, 29), (1, 0, 64), (1024, 8, 24)):
         keys = rng.integers(0, 1 << 63, n).astype(np.uint64) >> np.uint64(rng.integers(0, 40))
         vals = rng.permutation(n).astype(np.uint32)
         k0, v0 = keys.copy(), vals.copy()
@@ -282,15 +282,15 @@ def test_multi_partition_pipeline_through_the_emulated_stage_kernels(emu, p, key
         assert gens >= 6 and sum(step[5] for step in log if step[0] >= 1) > 0  # pills travelled in later generations
 
 
-@pytest.mark.parametrize("p,key_words,sigma,n", [(5, 4, 2, 700), (4, 1, 2, 900)])
+@pytest.mark.parametrize("p,key_words,sigma,n", [(5, 4, 2, 600), (3, 1, 2, 700)])
 def test_multi_partition_pipeline_with_the_emulated_step_entries(emu, p, key_words, sigma, n):
     """The same pipeline with each partition step as one call of csa_sort_init_dev / csa_sort_rerank_dev."""
     import multi_partition
     T = texts.random_text(n, sigma, 13 * p + n, sep_every=0)
     T[-7:] = 0
     if key_words == 1:  # long repeats: many generations, pills forwarded
-        T[300:600] = T[:300]
-        T[650:850] = T[100:300]
+        T[250:450] = T[:200]
+        T[500:650] = T[100:250]
     h = C.c_void_p()
     assert emu.csa_create(n, 1, C.byref(h)) == 0
     log, glue_log = [], []
@@ -305,14 +305,14 @@ def test_multi_partition_pipeline_with_the_emulated_step_entries(emu, p, key_wor
     assert log == glue_log
 
 
-@pytest.mark.parametrize("p,key_words,sigma,n,chunk_cap", [(3, 1, 3, 1400, 4096), (4, 2, 2, 1100, 4096)])
+@pytest.mark.parametrize("p,key_words,sigma,n,chunk_cap", [(3, 1, 3, 900, 4096), (4, 2, 2, 800, 4096)])
 def test_multi_partition_pipeline_through_the_emulated_slab_entries(emu, p, key_words, sigma, n, chunk_cap):
     """csa_sort_init_slabs / csa_sort_rerank_slabs / csa_scatter_slabs: every partition step takes and returns host slabs of
     ragged sizes (several per partition, some empty, the inbox shared out over them), the final permutation comes back cut
     into disk blocks and edges; the suffix array assembled from those pieces is the oracle's."""
     import multi_partition
     T = texts.random_text(n, sigma, 31 * p + n, sep_every=0)
-    T[n // 3:n // 3 + 400] = T[:400]
+    T[n // 3:n // 3 + 250] = T[:250]
     T[-5:] = 0
     h = C.c_void_p()
     assert emu.csa_create(n, 1, C.byref(h)) == 0
