@@ -12,8 +12,8 @@ pytestmark = pytest.mark.gpu
 
 @pytest.mark.timeout(600)
 @pytest.mark.parametrize("config,exclusive,oracle_verifier", [(2, False, True), (3, False, False), (3, True, True), (5, True, True),
-                                                              (4, False, False)],
-                         ids=["C2-arrival-oracle", "C3-arrival", "C3-xcd_chunked-oracle", "C5-xcd_chunked-oracle", "C4-arrival"])
+                                                              (4, True, True)],
+                         ids=["C2-arrival-oracle", "C3-arrival", "C3-xcd_chunked-oracle", "C5-xcd_chunked-oracle", "C4-xcd_chunked-oracle"])
 def test_full_size_configuration_sorts_to_a_verified_suffix_array(config, exclusive, oracle_verifier):
     import torch
     import oracle_lib
