@@ -226,11 +226,18 @@ __global__ __launch_bounds__(256) void stage_slab_kernel(StageArgs a)
     if (a.gen0 && a.keys) {
 #pragma unroll
         for (int w = 0; w < W; ++w) {
+            // one 8-byte load where the four symbols exist (the suffixes of a slab are in no order: every load of a wave
+            // is 64 separate lines, so four narrow loads per word cost four times the requests)
+            const u64 pos = j + 4ull * w;
             u64 k = 0;
+            if (pos + 4 <= a.n) {
+                u64 raw; // little-endian: s0 | s1 << 16 | s2 << 32 | s3 << 48
+                __builtin_memcpy(&raw, a.text + pos, 8);
+                k = (raw << 48) | ((raw & 0xFFFF0000ull) << 16) | ((raw >> 16) & 0xFFFF0000ull) | (raw >> 48);
+            } else {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const u64 pos = j + 4ull * w + q;
-                k = (k << 16) | (pos < a.n ? (u64)a.text[pos] : 0ull);
+                for (int q = 0; q < 4; ++q)
+                    k = (k << 16) | (pos + q < a.n ? (u64)a.text[pos + q] : 0ull);
             }
             a.keys[i * W + w] = k;
         }
