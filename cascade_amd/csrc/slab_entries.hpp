@@ -95,6 +95,9 @@ int check_slabs(const char* who, const csa_handle* h, const csa_slab* slabs, u32
                         (unsigned long long)s.off, (unsigned long long)(s.off + s.size), (unsigned long long)part_sz);
         if (s.size && (!s.key || !s.suf || (need_beta && !s.beta)))
             return fail(CSA_ERR_ARG, "%s: slab %u has a null column", who, c);
+        if (s.size && s.off != covered) // the chunks of a partition follow one another (src/GPU_SACA.cu:1396-1400)
+            return fail(CSA_ERR_ARG, "%s: slab %u starts at suffix %llu, the slabs before it end at %llu", who, c, (unsigned long long)s.off,
+                        (unsigned long long)covered);
         covered += s.size;
     }
     if (covered != part_sz)

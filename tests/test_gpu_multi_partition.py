@@ -126,6 +126,10 @@ def test_slab_entries_refuse_slabs_that_do_not_make_up_the_partition(gpu):
         assert b"slabs hold" in lib.csa_last_error()
         assert lib.csa_sort_init_slabs(h, arr, slab_c, 5096, 1, 3, 4000, end.ctypes.data, C.byref(act), None) == _native.CSA_ERR_ARG
         assert lib.csa_sort_init_slabs(h, arr, slab_c, 20000, 1, 3, 4096, end.ctypes.data, C.byref(act), None) == _native.CSA_ERR_ARG
+        # slabs that overlap although their sizes add up
+        arr3, c3, _ = pool.assemble([(0, 3000), (2000, 2096)])
+        assert lib.csa_sort_init_slabs(h, arr3, c3, 5096, 1, 3, 4096, end.ctypes.data, C.byref(act), None) == _native.CSA_ERR_ARG
+        assert b"starts at suffix" in lib.csa_last_error()
         # an inbox that the slabs do not carry in full
         assert lib.csa_sort_rerank_slabs(h, arr, slab_c, 5096, 77, 8, 3, 4096, end.ctypes.data, C.byref(act), None) == _native.CSA_ERR_ARG
         assert b"inbox" in lib.csa_last_error()
