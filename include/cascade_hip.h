@@ -294,7 +294,8 @@ typedef struct csa_slab {
     uint8_t* msg_target;  /* msg_target(): the slab's chunk of the inbox in (later generations), of the outbox out;
                              scatter out: the unaligned head of the output at [0, ...), its tail at [4096, ...) */
     uint32_t* msg_rank;   /* msg_rank(): likewise */
-    uint64_t off;         /* off(): where the slab's content starts in the partition */
+    uint64_t off;         /* off(): where the slab's content starts in the partition; the slabs of a list follow one
+                           * another (off = the sizes before it summed, src/GPU_SACA.cu:1396-1400) */
     uint64_t size;        /* size(): suffixes in the slab, at most chunk_cap */
     uint32_t inbox_off;   /* inbox_off(), inbox_sz(): the slab's chunk of the partition's inbox (later generations) */
     uint32_t inbox_sz;
