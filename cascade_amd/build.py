@@ -54,10 +54,23 @@ def build_cli():
     return CLI
 
 
+def build_cpp_tests():
+    """tests/cpp/slab_pipeline: a multi-partition build through the slab members of include/cascade_gpu_saca.hpp, in the
+    reference's own language (the GPU suite runs it). Host code; needs the HIP runtime only for its own device buffers."""
+    cxx = os.environ.get("CXX", "g++")
+    root = os.path.dirname(HERE)
+    out = os.path.join(root, "tests", "cpp", "slab_pipeline")
+    _run([cxx, "-std=c++17", "-O2", "-Wall", "-Wextra", "-D__HIP_PLATFORM_AMD__", "-isystem", "/opt/rocm/include", "-o", out,
+          os.path.join(root, "tests", "cpp", "slab_pipeline.cpp"), "-L" + HERE, "-lcascade_hip", "-L/opt/rocm/lib", "-lamdhip64",
+          "-Wl,-rpath,$ORIGIN/../../cascade_amd", "-Wl,-rpath,/opt/rocm/lib"])
+    return out
+
+
 def build_all():
     build_hip()
     build_workloads()
     build_cli()
+    build_cpp_tests()
 
 
 if __name__ == "__main__":
