@@ -544,6 +544,17 @@ def main():
     a_total = sum(per_gen) + a_out
     full_workload = args.n is None and args.key_words == 1
     traffic_source, per_pair, moved_gen, moved_job = measured_traffic(args.config) if full_workload else (None, None, {}, None)
+    # The per-generation bytes of the profile belong to this run only if the profile cut the sort into the same
+    # generations; a share of the peak above 1 is no measurement either. In both cases the per-generation figures of
+    # the profile are dropped (not printed), and the line says why.
+    moved_gen_dropped = None
+    if moved_gen and sorted(moved_gen) != list(range(st["generations"])):
+        moved_gen_dropped = f"the profile holds {len(moved_gen)} generations, the run had {st['generations']}"
+    elif any(st["ms"][g] > 0 and moved_gen[g] / (st["ms"][g] * 1e-3) / 1e9 > HBM_PEAK_GBS for g in moved_gen):
+        moved_gen_dropped = "a generation's bytes over this run's time exceed the HBM peak"
+    if moved_gen_dropped:
+        print(f"[bench] per-generation traffic of {traffic_source} not used: {moved_gen_dropped}", file=sys.stderr)
+        moved_gen = {}
     gen_table = []
     for g in range(st["generations"]):
         gbs = per_gen[g] / (st["ms"][g] * 1e-3) / 1e9 if st["ms"][g] > 0 else 0.0
@@ -600,6 +611,8 @@ def main():
         "job_moved_bytes_per_suffix": round(moved_job / n, 1) if moved_job else None,
         "generations": gen_table,
     }
+    if moved_gen_dropped:
+        result["generation_traffic_dropped"] = moved_gen_dropped
     if args.cpu_sample > 0:
         result["cpu_baseline"] = cpu_baseline(args.config, min(args.cpu_sample, n))
     print(json.dumps(result), flush=True)
