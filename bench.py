@@ -338,14 +338,57 @@ def bench_next_rows(args):
         res["roofline"]["bound"] = "pcie (not an HBM figure: 2 B up + 5 B down per suffix over the host link)"
         res["roofline"]["peak"] = None
         res["roofline"]["frac"] = None
+    elif args.row == "slab_pipeline":
+        # The reference's own calling pattern, PCIe included: a text in 16 partitions, every partition a chain of pinned
+        # host slabs of CHUNK_CAP = 2^21 suffixes (include/GPU_SACA.hpp:99), three dispatcher threads with a buffer set
+        # and a stream each calling the three members concurrently (src/GPU_SACA.cu:1539-1589) through the C++ mirror
+        # (tests/cpp/slab_pipeline.cpp, built by cascade_amd/build.py). The program times the dispatch phases (all
+        # partitions of a generation through their step, uploads and downloads included; host staging between the phases
+        # is not timed) and checks the finished suffix array against the resident sort; here the oracle's O(n) verifier
+        # judges it too. Value: suffixes through generation 0 per second, link traffic included.
+        import subprocess
+        import tempfile
+        exe = os.path.join(ROOT, "tests", "cpp", "slab_pipeline")
+        n = args.n if args.n is not None else 1 << 26
+        parts, threads = 16, 3
+        T = workloads.generate(args.config, n)
+        with tempfile.TemporaryDirectory(dir="/tmp") as tmp:
+            text, out = os.path.join(tmp, "text.u16"), os.path.join(tmp, "sa40")
+            T.tofile(text)
+            infos = []
+            for th in (threads, 1):
+                run = subprocess.run([exe, "0", str(parts), str(args.key_words), str(1 << 21), "7", "1", out, str(th), text],
+                                     capture_output=True, text=True)
+                if run.returncode != 0 or not run.stdout.startswith("OK "):
+                    print(run.stdout, run.stderr, file=sys.stderr)
+                    sys.exit(1)
+                infos.append(dict(kv.split("=") for kv in run.stdout.split() if "=" in kv and not kv.startswith("(")))
+            ok = bool(oracle_lib.is_correct_sa40(np.fromfile(out, dtype=np.uint8), T))
+        info, one = infos
+        ms0, b0 = float(info["gen0_ms"]), int(info["gen0_link_bytes"])
+        res = _row_result("suffixes through a generation-0 partition step/sec at 1 GPU, pinned host slabs in and out",
+                          workloads.NAMES[args.config], n, ms0,
+                          "sort_and_init_rank_and_filter on host slabs, three dispatcher threads (csa_sort_init_slabs)", b0,
+                          {"partitions": parts, "chunk_cap": 1 << 21, "dispatchers": threads, "key_words": args.key_words,
+                           "generations": int(info["generations"]), "largest_partition": int(info["max_part"]),
+                           "device_bytes_three_buffer_sets": int(info["device_bytes"]),
+                           "gen0_link_GBps": round(b0 / ms0 / 1e6, 1),
+                           "all_generations_ms": round(float(info["dispatch_ms"]), 2),
+                           "all_generations_link_GBps": round(int(info["link_bytes"]) / float(info["dispatch_ms"]) / 1e6, 1),
+                           "scatter_ms": round(float(info["scatter_ms"]), 2),
+                           "scatter_link_GBps": round(int(info["scatter_link_bytes"]) / float(info["scatter_ms"]) / 1e6, 1),
+                           "gen0_ms_one_dispatcher": round(float(one["gen0_ms"]), 2),
+                           "all_generations_ms_one_dispatcher": round(float(one["dispatch_ms"]), 2),
+                           "scatter_ms_one_dispatcher": round(float(one["scatter_ms"]), 2)}, 1, 0, ok)
+        res["roofline"]["bound"] = "pcie (not an HBM figure: bytes of the slabs' columns over the host link, both directions)"
+        res["roofline"]["peak"] = None
+        res["roofline"]["frac"] = None
     elif args.row in ("step_init", "step_rerank"):
         # one partition step under the exchange scheme: everything the reference does between the upload of a partition's
         # slabs and their download (src/GPU_SACA.cu:1112-1331 / 1715-1995). The synthetic partition: n suffixes of the
         # workload's text in random order, p partitions by sampled pivots.
         import ctypes as C
-
-        class StepResult(C.Structure):
-            _fields_ = [("active", C.c_uint64), ("messages", C.c_uint64)]
+        StepResult = _native.CsaStepResult
         T = workloads.generate(args.config, n)
         pivots = oracle_lib.sample_pivots(T[:1 << 22], p, 2, rng)
         d_text = torch.from_numpy(T.view(np.int16)).to(dev)
@@ -354,7 +397,7 @@ def bench_next_rows(args):
         lanes = torch.stack([(suf >> (8 * b)) & 0xFF for b in range(5)], dim=1).to(torch.uint8).reshape(-1).contiguous()
         kw = args.key_words
         keys, beta = stage_slab(d_text, lanes, kw, packed, p, 4 * kw, True)
-        sorter = PartitionSorter(n)
+        sorter = PartitionSorter(n, key_words=kw, for_steps=True)  # the steps' own floor plan: csa_step_bytes_per_suffix
         rank_out = torch.empty(n, dtype=torch.int32, device=dev)
         suf_out = torch.empty(5 * n, dtype=torch.uint8, device=dev)
         mt, mr = torch.empty(5 * 2 * n, dtype=torch.uint8, device=dev), torch.empty(2 * n, dtype=torch.int32, device=dev)
@@ -437,7 +480,7 @@ def main():
                     help="check the headline output with the device verifier only (the default also runs the CPU oracle's O(n) "
                          "verifier on it, about 23 bytes of host memory per suffix)")
     ap.add_argument("--generations", action="store_true", help="print the per-generation table to stderr")
-    ap.add_argument("--row", default="sort", choices=["sort", "partition_ids", "stage_slab", "messages", "join", "scatter", "step_init", "step_rerank", "overlap", "pipeline"],
+    ap.add_argument("--row", default="sort", choices=["sort", "partition_ids", "stage_slab", "messages", "join", "scatter", "step_init", "step_rerank", "overlap", "pipeline", "slab_pipeline"],
                     help="which step to measure: the partition sort (the headline, default) or one of the steps around it")
     ap.add_argument("--shared-device", action="store_true",
                     help="measure the headline with the default tile order (safe next to other launches) only")

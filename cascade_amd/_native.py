@@ -22,8 +22,9 @@ EXPORTS = (
     "csa_partition_id_bits", "csa_partition_ids_u16_dev", "csa_scatter_to_rank_order_dev", "csa_output_cut",
     "csa_stage_slab_u16_dev", "csa_count_messages_dev", "csa_message_offsets_dev", "csa_emit_messages_dev",
     "csa_join_messages_dev", "csa_join_messages_sorted_dev", "csa_sort_init_dev", "csa_sort_rerank_dev",
-    "csa_set_device_exclusive", "csa_set_tuning", "csa_radix_sort_pairs_static_dev", "csa_enable_profile_ranges",
-    "csa_slab_bytes_per_suffix", "csa_sort_init_slabs", "csa_sort_rerank_slabs", "csa_scatter_slabs", "csa_sort_partitions_u16",
+    "csa_set_device_exclusive", "csa_set_tuning", "csa_radix_sort_pairs_static_dev", "csa_radix_sort_pairs_static_status", "csa_enable_profile_ranges",
+    "csa_step_bytes_per_suffix", "csa_workspace_bytes", "csa_create_steps", "csa_scratch_high_water", "csa_last_step_result",
+    "csa_sort_init_slabs", "csa_sort_rerank_slabs", "csa_scatter_slabs", "csa_sort_partitions_u16",
 )
 
 
@@ -34,6 +35,12 @@ class CsaSlab(C.Structure):
         ("off", C.c_uint64), ("size", C.c_uint64), ("inbox_off", C.c_uint32), ("inbox_sz", C.c_uint32),
         ("outbox_off", C.c_uint32), ("outbox_sz", C.c_uint32),
     ]
+
+
+class CsaStepResult(C.Structure):
+    """csa_step_result of include/cascade_hip.h: what a per-generation partition step reports."""
+    _fields_ = [("active", C.c_uint64), ("messages", C.c_uint64), ("unserved", C.c_uint64), ("pills", C.c_uint64),
+                ("incoherent_pills", C.c_uint64)]
 
 
 class CsaStats(C.Structure):
@@ -100,6 +107,8 @@ def load():
     lib.csa_radix_sort_pairs_dev.argtypes = [vp, vp, vp, u64, i32, i32, vp]
     lib.csa_radix_sort_pairs_static_dev.restype = i32
     lib.csa_radix_sort_pairs_static_dev.argtypes = [vp, vp, u64, i32, i32, vp]
+    lib.csa_radix_sort_pairs_static_status.restype = i32
+    lib.csa_radix_sort_pairs_static_status.argtypes = [vp]
     lib.csa_verify_sa40_dev.restype = i32
     lib.csa_verify_sa40_dev.argtypes = [vp, vp, u64, u64, vp, vp, C.POINTER(i32)]
     lib.csa_last_error.restype = C.c_char_p
@@ -128,8 +137,16 @@ def load():
     lib.csa_sort_rerank_dev.argtypes = [vp, vp, vp, vp, u64, vp, vp, u32, u64, u32, vp, vp, vp, vp, vp, vp, vp]
     lib.csa_enable_profile_ranges.restype = i32
     lib.csa_enable_profile_ranges.argtypes = [i32]
-    lib.csa_slab_bytes_per_suffix.restype = u64
-    lib.csa_slab_bytes_per_suffix.argtypes = [i32]
+    lib.csa_step_bytes_per_suffix.restype = u64
+    lib.csa_step_bytes_per_suffix.argtypes = [i32]
+    lib.csa_workspace_bytes.restype = u64
+    lib.csa_workspace_bytes.argtypes = [u64]
+    lib.csa_create_steps.restype = i32
+    lib.csa_create_steps.argtypes = [u64, i32, C.POINTER(vp)]
+    lib.csa_scratch_high_water.restype = u64
+    lib.csa_scratch_high_water.argtypes = [vp]
+    lib.csa_last_step_result.restype = i32
+    lib.csa_last_step_result.argtypes = [vp, C.POINTER(CsaStepResult)]
     lib.csa_sort_init_slabs.restype = i32
     lib.csa_sort_init_slabs.argtypes = [vp, C.POINTER(CsaSlab), u32, u64, i32, u32, u64, vp, vp, vp]
     lib.csa_sort_rerank_slabs.restype = i32

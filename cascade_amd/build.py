@@ -62,7 +62,7 @@ def build_cpp_tests():
     out = os.path.join(root, "tests", "cpp", "slab_pipeline")
     _run([cxx, "-std=c++17", "-O2", "-Wall", "-Wextra", "-D__HIP_PLATFORM_AMD__", "-isystem", "/opt/rocm/include", "-o", out,
           os.path.join(root, "tests", "cpp", "slab_pipeline.cpp"), "-L" + HERE, "-lcascade_hip", "-L/opt/rocm/lib", "-lamdhip64",
-          "-Wl,-rpath,$ORIGIN/../../cascade_amd", "-Wl,-rpath,/opt/rocm/lib"])
+          "-Wl,-rpath,$ORIGIN/../../cascade_amd", "-Wl,-rpath,/opt/rocm/lib", "-pthread"])
     return out
 
 

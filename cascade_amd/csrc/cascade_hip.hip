@@ -2,6 +2,7 @@
 // declared in include/cascade_hip.h. gfx950 only.
 #include "../../include/cascade_hip.h"
 
+#include "device_pool.hpp"
 #include "device_utils.hpp"
 #include "doubling.hpp"
 #include "messages.hpp"
@@ -174,6 +175,8 @@ constexpr int SMALL_MAXG_HI = CSA_SMALL_MAXG_HI;
 constexpr u32 SMALL_AVG_LIMIT = CSA_SMALL_AVG_LIMIT;
 static_assert(SMALL_MAXG_HI >= SMALL_MAXG, "the higher group limit is the higher one");
 constexpr u32 TICKET_POOL = 4096;
+constexpr u32 PINNED_HIST = 32;        // host mirror: words [0, 16) mirror the device counters, [16, 32) single values, then the histograms
+constexpr u32 MSG_OFF_WORDS = 32769;   // p + 1 outbox counters, p <= 32768
 constexpr int EVENT_POOL = 2 * CSA_MAX_GENERATIONS * MAX_PASSES * 2;
 
 // Lists of at least this many suffixes update rank[] through two radix passes on the text position instead of
@@ -262,21 +265,28 @@ constexpr u64 STATIC_SCRATCH_BYTES = align256(STATIC_OFF_DIGIT_BASE + MAX_PASSES
 
 static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
 
-namespace {
-struct SlabArena; // device image of a partition's host slabs (slab_entries.hpp)
-void free_slab_arena(csa_handle* h);
-}
+// What a handle was created for (csa_create: everything; csa_create_steps: everything but the resident sort).
+constexpr u32 KIND_RESIDENT = 1u;
 
 struct csa_handle {
     int device = 0;
     u64 cap = 0;
     int key_words = 1;
+    u32 kinds = 0;
+    int cus = 0; // compute units of the device
+    // One block of device memory for everything that scales with the partition. The resident sort uses it under a fixed
+    // carve-up made at creation (the arrays below); every other entry point takes and returns columns of it as it goes
+    // (device_pool.hpp). A handle serves one call at a time, so the two never meet.
+    unsigned char* block = nullptr;
+    DevicePool pool;
+    u64 last_high_water = 0; // of the last call that used the pool
     u64* key[3] = {nullptr, nullptr, nullptr};
     u32* idx[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
     u32* gid = nullptr;
     u32* rank = nullptr;
     u32* gprim[2] = {nullptr, nullptr};
     u32* gstart[2] = {nullptr, nullptr};
+    // The workspace: tables whose size follows the number of tiles, and small fixed ones.
     u64* lookback = nullptr;
     u64 lookback_words = 0;
     u64 lookback_tile_words = 0;
@@ -287,16 +297,18 @@ struct csa_handle {
     u32* digit_base = nullptr; // [MAX_PASSES][256]
     u32* tickets = nullptr;    // [TICKET_POOL]
     u32 ticket_next = 0;
-    u32* counts = nullptr; // [2] error flag; [3] verifier flag; [4] members of large groups
-    u32* h_pinned = nullptr; // host mirror: [0..3] counts/err, [16 ..) histogram
+    u32* counts = nullptr; // [2] error flag; [3] verifier flag; [4] members of large groups; [6..7] tied entries;
+                           // [8..9] active-set size of a step; [10..11] unserved members; [12..13] pill receipts;
+                           // [14] incoherent pill receipts
+    u32* msg_off = nullptr; // [MSG_OFF_WORDS]: the outbox counters of the slab-shaped steps
+    u32* h_pinned = nullptr; // host mirror: [0..15] counts, [16 ..) histogram
     u32 epoch = 0;
     u32 tile_order = TILES_BY_ARRIVAL;           // how the radix passes number their tiles (radix_sort.hpp), in use
     u32 tile_order_exclusive = TILES_BY_ARRIVAL; // the order after csa_set_device_exclusive
     u32 xcd_chunk = XCD_CHUNK;                   // tiles of a radix pass that one XCD takes in a row under TILES_STATIC_CHUNKS
     u32 defer_min = DEFER_MIN; // lists at least this long use the bucketed rank update (csa_set_tuning)
-    u64* step64[2] = {nullptr, nullptr}; // two more 8-byte arrays of the capacity, for the per-generation partition steps
-    SlabArena* slab_arena = nullptr;     // allocated by the first call of a slab-shaped entry
     u32 window_min_changed = WINDOW_MIN_CHANGED; // csa_set_tuning (0xFFFFFFFF: never)
+    csa_step_result last_step = {};              // counters of the last partition step (csa_last_step_result)
     std::vector<hipEvent_t> events;
     hipEvent_t ev_gen[CSA_MAX_GENERATIONS + 2] = {};
     bool ev_gen_ready = false;
@@ -465,7 +477,7 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
     }
     hipLaunchKernelGGL(radix_scan_hist_kernel, dim3(1), dim3(256), 0, s, h->ghist, h->digit_base, plan.num_passes);
     HIP_TRY(hipGetLastError());
-    u32* h_hist = h->h_pinned + 16;
+    u32* h_hist = h->h_pinned + PINNED_HIST;
     HIP_TRY(hipMemcpyAsync(h_hist, h->ghist, plan.num_passes * RADIX_BINS * sizeof(u32), hipMemcpyDeviceToHost, s));
     HIP_TRY(hipStreamSynchronize(s));
     bool run[MAX_PASSES];
@@ -625,7 +637,7 @@ int deferred_rank_update(Launch& L, const DeferBuffers& buf, u32 n)
     }
     const u64* in_recs = buf.recs[0];
     if (n_pass > 0) {
-        u32* h_hist = h->h_pinned + 16;
+        u32* h_hist = h->h_pinned + PINNED_HIST;
         for (int p = 0; p < n_pass; ++p) {
             // positions x in [0, n) whose digit (x >> shift) & mask equals d: whole periods plus a clamped remainder
             const u64 unit = 1ull << xshift[p], period = unit << xbits[p];
@@ -754,7 +766,7 @@ int rank_totals(Launch& L, const RankTables& r, bool gen0, u32 m, u32 n, bool ex
     hipLaunchKernelGGL(rerank_scan_kernel, dim3(r.slabs), dim3(1024), 0, s, r.tile_agg, r.tile_prefix, r.tiles, r.slab,
                        r.slab_total, r.tile_splits);
     HIP_TRY(hipGetLastError());
-    u32* h_slabs = h->h_pinned + 16;
+    u32* h_slabs = h->h_pinned + PINNED_HIST;
     HIP_TRY(hipMemcpyAsync(h_slabs, r.slab_total, r.slabs * 5 * sizeof(u32), hipMemcpyDeviceToHost, s));
     u32 big_seen = 0;
     int rc = read_counts(L, &big_seen);
@@ -1320,21 +1332,39 @@ int csa_join_messages_sorted_dev(csa_handle* h, const uint8_t* d_msg_target, con
     L.stats = nullptr;
     hipStream_t s = L.stream;
     HIP_TRY(hipMemsetAsync(h->counts, 0, 4 * sizeof(u32), s));
-    // (target word, rank) pairs in the handle's arrays, sorted on the 40 target bits
-    hipLaunchKernelGGL(unpack_lanes_kernel, dim3((msg_c + 255u) / 256u), dim3(256), 0, s, d_msg_target, (u64)msg_c, h->key[0]);
-    HIP_TRY(hipMemcpyAsync(h->idx[0], d_msg_rank, (u64)msg_c * sizeof(u32), hipMemcpyDeviceToDevice, s));
+    // (target word, rank) pairs in columns of the handle's block, sorted on the 40 target bits
+    h->pool.reset();
+    u64* K[2];
+    u32* V[2];
+    for (int i = 0; i < 2; ++i) {
+        K[i] = static_cast<u64*>(h->pool.take((u64)msg_c * sizeof(u64)));
+        V[i] = static_cast<u32*>(h->pool.take((u64)msg_c * sizeof(u32)));
+    }
+    if (!K[0] || !V[0] || !K[1] || !V[1])
+        return fail(CSA_ERR_ARG, "csa_join_messages_sorted_dev: the handle's block of %llu bytes has no room for 24 bytes per message",
+                    (unsigned long long)h->pool.bytes());
+    // the directory over the cohort takes what is left, up to an entry per cohort member (a smaller one has longer buckets)
+    u64 dir_room = n < 3 ? 3 : n;
+    u32* dir = nullptr;
+    while (dir_room >= 3 && !(dir = static_cast<u32*>(h->pool.take(dir_room * sizeof(u32)))))
+        dir_room /= 2;
+    if (!dir)
+        dir_room = 0;
+    h->last_high_water = h->pool.high_water();
+    hipLaunchKernelGGL(unpack_lanes_kernel, dim3((msg_c + 255u) / 256u), dim3(256), 0, s, d_msg_target, (u64)msg_c, K[0]);
+    HIP_TRY(hipMemcpyAsync(V[0], d_msg_rank, (u64)msg_c * sizeof(u32), hipMemcpyDeviceToDevice, s));
     int in_out = 0, passes = 0;
     const PassPlan plan = make_plan(0, 40);
-    int rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, h->key[0], h->idx[0], h->key[1], h->idx[1], msg_c, plan, &in_out, &passes);
+    int rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, K[0], V[0], K[1], V[1], msg_c, plan, &in_out, &passes);
     if (rc)
         return rc;
     u32 dir_log2 = 0;
-    rc = build_join_directory(d_sa, n, h->idx[2], h->cap, s, &dir_log2);
+    rc = build_join_directory(d_sa, n, dir, dir_room, s, &dir_log2);
     if (rc)
         return rc;
     hipLaunchKernelGGL(join_messages_kernel, dim3((msg_c + 255u) / 256u), dim3(256), 0, s, (const u8*)nullptr,
-                       (const u64*)h->key[in_out], (const u32*)h->idx[in_out], msg_c, d_sa, d_primary, d_keys, n,
-                       (const u32*)(dir_log2 ? h->idx[2] : nullptr), dir_log2);
+                       (const u64*)K[in_out], (const u32*)V[in_out], msg_c, d_sa, d_primary, d_keys, n,
+                       (const u32*)(dir_log2 ? dir : nullptr), dir_log2);
     HIP_TRY(hipGetLastError());
     return read_counts(L, nullptr);
 }
@@ -1383,297 +1413,59 @@ int csa_stage_slab_u16_dev(const uint16_t* d_text, uint64_t n, const uint8_t* d_
 
 extern "C++" {
 namespace {
-
-// Shared tail of the two partition steps: the list (keys, suffix words, routing tags) sorted by key is ranked and split
-// into active / retired, the cohort's messages are emitted, ranks and lanes are narrowed for the caller.
-template <bool GEN0>
-int finish_partition_step(Launch& L, const u64* sorted_key0, const u64* sorted_key1, const u64* keys_src, const u32* perm, int key_words,
-                          const u64* sorted_words, const u32* sorted_beta, u64 m, u64 ctx, u32 p, u64* key_r, u64* words_r, u32* beta_r, u32* d_rank_out, u8* d_suf40_out,
-                          u8* d_msg_target, u32* d_msg_rank, u32* d_msg_off, csa_step_result* res)
+// The scatter behind csa_scatter_to_rank_order_dev and csa_scatter_slabs; takes its columns from the handle's block as
+// that block stands (the caller has reset it, or holds columns of its own in it). Waits for the stream.
+int scatter_to_rank_order(csa_handle* h, const char* who, const u8* d_suf, const u32* d_rank, u64 part_sz, u8* d_sa40, hipStream_t s)
 {
-    csa_handle* h = L.h;
-    hipStream_t s = L.stream;
-    const RankTables r = rank_tables(h, (u32)m, STEP_TILE);
-    unsigned long long* d_active = reinterpret_cast<unsigned long long*>(h->counts + 8);
-    StepRankArgs ra;
-    ra.key0 = sorted_key0;
-    ra.key1 = sorted_key1;
-    ra.keys_src = keys_src;
-    ra.perm = perm;
-    ra.key_words = key_words;
-    ra.words = sorted_words;
-    ra.beta = sorted_beta;
-    ra.m = m;
-    ra.key_out = key_r;
-    ra.words_out = words_r;
-    ra.beta_out = beta_r;
-    ra.tile_agg = r.tile_agg;
-    ra.tile_splits = r.tile_splits;
-    ra.tile_prefix = r.tile_prefix;
-    ra.slab_total = r.slab_total;
-    ra.slab = r.slab;
-    ra.slabs = r.slabs;
-    ra.active_out = d_active;
-    hipLaunchKernelGGL((step_rank_kernel<GEN0, false>), dim3(r.tiles), dim3(STEP_BLOCK), 0, s, ra);
-    hipLaunchKernelGGL(rerank_scan_kernel, dim3(r.slabs), dim3(1024), 0, s, r.tile_agg, r.tile_prefix, r.tiles, r.slab, r.slab_total,
-                       r.tile_splits);
-    hipLaunchKernelGGL((step_rank_kernel<GEN0, true>), dim3(r.tiles), dim3(STEP_BLOCK), 0, s, ra);
-    HIP_TRY(hipGetLastError());
-    // the cohort's messages, collated by destination (src/GPU_SACA.cu:1266-1287,1930-1951)
-    MessageArgs ma;
-    int rc = fill_message_args(ma, "partition step", key_r ? words_r : nullptr, key_r, beta_r, m, ctx, GEN0 ? 0 : 1, p);
-    if (rc)
-        return rc;
-    HIP_TRY(hipMemsetAsync(d_msg_off, 0, ((u64)p + 1) * sizeof(u32), s));
-    ma.msg_off = d_msg_off;
-    const u32 grid = ma.tiles < 4096u ? ma.tiles : 4096u;
-    hipLaunchKernelGGL(count_messages_kernel, dim3(grid), dim3(MSG_BLOCK), 0, s, ma);
-    hipLaunchKernelGGL(message_offsets_kernel, dim3(1), dim3(1024), 0, s, d_msg_off, p + 1);
-    ma.active_sz = d_active;
-    ma.msg_target = d_msg_target;
-    ma.msg_rank = d_msg_rank;
-    hipLaunchKernelGGL(emit_messages_kernel, dim3(grid), dim3(MSG_BLOCK), 0, s, ma);
-    // what the caller persists: narrowed ranks and lanes (src/GPU_SACA.cu:1289-1305)
-    hipLaunchKernelGGL(narrow_and_pack_kernel, dim3((u32)((m + 255) / 256)), dim3(256), 0, s, (const u64*)key_r, (const u64*)words_r, m,
-                       GEN0 ? 0 : 1, d_rank_out, d_suf40_out);
-    HIP_TRY(hipGetLastError());
-    HIP_TRY(hipMemcpyAsync(h->h_pinned + 8, h->counts + 8, 2 * sizeof(u32), hipMemcpyDeviceToHost, s));
-    HIP_TRY(hipMemcpyAsync(h->h_pinned + 10, d_msg_off + (p - 1), sizeof(u32), hipMemcpyDeviceToHost, s));
-    rc = read_counts(L, nullptr);
-    if (rc)
-        return rc;
-    if (res) {
-        res->active = (u64)h->h_pinned[8] | ((u64)h->h_pinned[9] << 32);
-        res->messages = h->h_pinned[10];
+    HIP_TRY(hipMemsetAsync(h->counts, 0, 4 * sizeof(u32), s));
+    const u32 blocks = (u32)((part_sz + 255) / 256);
+    u64* K[2] = {nullptr, nullptr};
+    u32* V[2] = {nullptr, nullptr};
+    bool windowed = part_sz >= SCATTER_WINDOW_MIN && part_sz <= h->cap;
+    if (windowed) { // (a block without room for the 24 bytes per suffix of the window pass scatters directly)
+        for (int i = 0; i < 2; ++i) {
+            K[i] = static_cast<u64*>(h->pool.take(part_sz * sizeof(u64)));
+            V[i] = static_cast<u32*>(h->pool.take(part_sz * sizeof(u32)));
+        }
+        windowed = K[0] && V[0] && K[1] && V[1];
     }
-    return CSA_OK;
-}
-
-int check_step_args(csa_handle* h, const char* who, u64 m, u32 p, const void* a, const void* b, const void* c, const void* d)
-{
-    if (!h)
-        return fail(CSA_ERR_ARG, "%s: null handle", who);
-    if (p < 1 || p > 32768u)
-        return fail(CSA_ERR_ARG, "%s: p = %u is outside [1, 32768]", who, p);
-    if (m > h->cap)
-        return fail(CSA_ERR_ARG, "%s: %llu suffixes exceed the handle's capacity %llu", who, (unsigned long long)m,
-                    (unsigned long long)h->cap);
-    if (m && (!a || !b || !c || !d))
-        return fail(CSA_ERR_ARG, "%s: null buffer", who);
-    if (!h->step64[0]) { // one block: generation 0 also uses it as one array of 16-byte records
-        const u64 cap = h->cap ? h->cap : 1;
-        const hipError_t e = hipMalloc((void**)&h->step64[0], 2 * cap * sizeof(u64));
-        if (e != hipSuccess)
-            return fail(CSA_ERR_HIP, "%s: %s while allocating the step scratch", who, hipGetErrorString(e));
-        h->step64[1] = h->step64[0] + cap;
+    if (windowed) {
+        // large partition: group the pairs by the window of the output their rank falls into, then write window by window
+        Launch L;
+        L.h = h;
+        L.stream = s;
+        L.flags = 0;
+        L.stats = nullptr;
+        hipLaunchKernelGGL(scatter_window_keys_kernel, dim3(blocks), dim3(256), 0, s, d_suf, d_rank, part_sz, (int)SCATTER_WINDOW_LOG2,
+                           K[0], V[0], h->counts + 3);
+        const int window_bits = bit_length((part_sz - 1) >> SCATTER_WINDOW_LOG2);
+        int in_out = 0, passes = 0;
+        const int rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, K[0], V[0], K[1], V[1], (u32)part_sz,
+                                  make_plan(40, 40 + window_bits), &in_out, &passes);
+        if (rc)
+            return rc;
+        hipLaunchKernelGGL(scatter_window_lanes_kernel, dim3(blocks), dim3(256), 0, s, (const u64*)K[in_out], (const u32*)V[in_out],
+                           part_sz, d_sa40);
+    } else {
+        hipLaunchKernelGGL(scatter_lanes_kernel, dim3(blocks), dim3(256), 0, s, d_suf, d_rank, part_sz, d_sa40, h->counts + 3);
     }
-    return CSA_OK;
+    HIP_TRY(hipGetLastError());
+    for (int i = 0; i < 2; ++i) {
+        h->pool.give(K[i]);
+        h->pool.give(V[i]);
+    }
+    Launch R;
+    R.h = h;
+    R.stream = s;
+    R.flags = 0;
+    R.stats = nullptr;
+    const int rc_counts = read_counts(R, nullptr); // waits for the stream; a failed wait of the bucket pass ends here
+    if (h->h_pinned[3])
+        return fail(CSA_ERR_ARG, "%s: a rank lies outside [0, %llu)", who, (unsigned long long)part_sz);
+    return rc_counts;
 }
-
 } // namespace
 } // extern "C++"
-
-int csa_sort_init_dev(csa_handle* h, const uint64_t* d_keys, int key_words, const uint8_t* d_suf40, const uint32_t* d_beta,
-                      uint64_t m, uint32_t p, uint32_t* d_rank_out, uint8_t* d_suf40_out, uint8_t* d_msg_target,
-                      uint32_t* d_msg_rank, uint32_t* d_msg_off, void* stream, csa_step_result* res)
-{
-    if (key_words < 1 || key_words > 4)
-        return fail(CSA_ERR_ARG, "csa_sort_init_dev: key_words = %d is outside [1, 4]", key_words);
-    int rc = check_step_args(h, "csa_sort_init_dev", m, p, d_keys, d_suf40, d_beta, d_msg_off);
-    if (rc)
-        return rc;
-    if (res)
-        res->active = res->messages = 0;
-    if (m == 0) {
-        HIP_TRY(hipMemsetAsync(d_msg_off, 0, ((u64)p + 1) * sizeof(u32), (hipStream_t)stream));
-        return CSA_OK;
-    }
-    if (!d_rank_out || !d_suf40_out || !d_msg_target || !d_msg_rank)
-        return fail(CSA_ERR_ARG, "csa_sort_init_dev: null output buffer");
-    Launch L;
-    L.h = h;
-    L.stream = (hipStream_t)stream;
-    L.flags = 0;
-    L.stats = nullptr;
-    hipStream_t s = L.stream;
-    const u32 blocks = (u32)((m + 255) / 256);
-    HIP_TRY(hipMemsetAsync(h->counts, 0, 4 * sizeof(u32), s));
-    u64* K[2] = {h->key[0], h->key[1]};
-    u32* P[2] = {h->idx[0], h->idx[1]};
-    int kc = 0, pc = 0; // the arrays that hold the current keys / permutation
-    int in_out = 0, passes = 0;
-    hipLaunchKernelGGL(iota_kernel, dim3(blocks), dim3(256), 0, s, P[pc], m);
-    if (key_words == 1) {
-        // stable LSD sort by (key word, forward tag): the tag first, then the word (src/GPU_SACA.cu:1165-1227), on
-        // (64-bit key, permutation) pairs
-        hipLaunchKernelGGL(tag_keys_kernel, dim3(blocks), dim3(256), 0, s, d_beta, m, K[kc]);
-        rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, K[kc], P[pc], K[kc ^ 1], P[pc ^ 1], (u32)m, make_plan(0, 16), &in_out, &passes);
-        if (rc)
-            return rc;
-        pc ^= in_out;
-        hipLaunchKernelGGL(gather_u64_kernel, dim3(blocks), dim3(256), 0, s, (const u64*)d_keys, (const u32*)P[pc], m, 1u, 0u, K[0]);
-        rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, K[0], P[pc], K[1], P[pc ^ 1], (u32)m, make_plan(0, 64), &in_out, &passes);
-        if (rc)
-            return rc;
-        kc = in_out;
-        pc ^= in_out;
-    } else {
-        // Wider keys: the same order, (key words, forward tag), reached from the most significant word. All suffixes are
-        // sorted by word 0 alone. Only those that tie with a neighbour on it can still change places, and only inside their
-        // run: they are taken out in order, sorted among themselves by (word 0, ..., word W - 1, tag) with the stable LSD
-        // passes of the reference (tag, then the words from the last, src/GPU_SACA.cu:1165-1227) and put back, in that
-        // order, at the places the tied entries held. Sorting every suffix on every word costs 2 + 8 W passes over the
-        // partition; this costs 8, plus 2 + 8 W over the tied ones.
-        hipLaunchKernelGGL(gather_u64_kernel, dim3(blocks), dim3(256), 0, s, (const u64*)d_keys, (const u32*)P[pc], m, (u32)key_words, 0u,
-                           K[0]);
-        rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, K[0], P[pc], K[1], P[pc ^ 1], (u32)m, make_plan(0, 64), &in_out, &passes);
-        if (rc)
-            return rc;
-        kc = in_out;
-        pc ^= in_out;
-        const RankTables r = rank_tables(h, (u32)m, STEP_TILE);
-        TieArgs ta;
-        ta.keys = K[kc];
-        ta.perm = P[pc];
-        ta.m = m;
-        ta.pos_out = h->idx[4];
-        ta.perm_out = h->idx[2];
-        ta.tile_agg = r.tile_agg;
-        ta.tile_splits = r.tile_splits;
-        ta.tile_prefix = r.tile_prefix;
-        ta.slab_total = r.slab_total;
-        ta.slab = r.slab;
-        ta.slabs = r.slabs;
-        ta.total_out = reinterpret_cast<unsigned long long*>(h->counts + 6);
-        hipLaunchKernelGGL((tie_kernel<false>), dim3(r.tiles), dim3(STEP_BLOCK), 0, s, ta);
-        hipLaunchKernelGGL(rerank_scan_kernel, dim3(r.slabs), dim3(1024), 0, s, r.tile_agg, r.tile_prefix, r.tiles, r.slab, r.slab_total,
-                           r.tile_splits);
-        hipLaunchKernelGGL((tie_kernel<true>), dim3(r.tiles), dim3(STEP_BLOCK), 0, s, ta);
-        HIP_TRY(hipGetLastError());
-        rc = read_counts(L, nullptr);
-        if (rc)
-            return rc;
-        const u64 tied = h->h_pinned[6];
-        if (tied > m)
-            return fail(CSA_ERR_INTERNAL, "csa_sort_init_dev: %llu of %llu suffixes counted as tied", (unsigned long long)tied, (unsigned long long)m);
-        if (tied > 0) {
-            const u32 tblocks = (u32)((tied + 255) / 256);
-            u64* SK[2] = {K[kc ^ 1], h->key[2]}; // the sorted word 0 stays in K[kc]
-            u32* SV[2] = {h->idx[2], h->idx[3]};
-            int sv = 0;
-            hipLaunchKernelGGL(gather_tag_keys_kernel, dim3(tblocks), dim3(256), 0, s, d_beta, (const u32*)SV[sv], tied, SK[0]);
-            rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, SK[0], SV[sv], SK[1], SV[sv ^ 1], (u32)tied, make_plan(0, 16), &in_out, &passes);
-            if (rc)
-                return rc;
-            sv ^= in_out;
-            for (int w = key_words - 1; w >= 0; --w) {
-                hipLaunchKernelGGL(gather_u64_kernel, dim3(tblocks), dim3(256), 0, s, (const u64*)d_keys, (const u32*)SV[sv], tied,
-                                   (u32)key_words, (u32)w, SK[0]);
-                rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, SK[0], SV[sv], SK[1], SV[sv ^ 1], (u32)tied, make_plan(0, 64), &in_out, &passes);
-                if (rc)
-                    return rc;
-                sv ^= in_out;
-            }
-            hipLaunchKernelGGL(scatter_u32_kernel, dim3(tblocks), dim3(256), 0, s, (const u32*)SV[sv], (const u32*)h->idx[4], tied, m, P[pc],
-                               h->counts + 2);
-            HIP_TRY(hipGetLastError());
-        }
-    }
-    // sorted: key word 0 in K[kc], the permutation in P[pc]
-    u64* sorted_key1 = nullptr;
-    if (key_words >= 2) {
-        sorted_key1 = K[kc ^ 1];
-        hipLaunchKernelGGL(gather_u64_kernel, dim3(blocks), dim3(256), 0, s, (const u64*)d_keys, (const u32*)P[pc], m, (u32)key_words, 1u,
-                           sorted_key1);
-    }
-    u64* sorted_words = h->key[2];
-    u32* sorted_beta = h->idx[2];
-    // the carried columns follow the permutation: lane and routing tags of a suffix are first put side by side in one
-    // 16-byte record (a streaming pass), so that the gather costs one random line per suffix instead of two
-    uint4* carried = reinterpret_cast<uint4*>(h->step64[0]);
-    hipLaunchKernelGGL(pack_carried_kernel, dim3(blocks), dim3(256), 0, s, d_suf40, d_beta, m, carried);
-    hipLaunchKernelGGL(gather_carried_kernel, dim3(blocks), dim3(256), 0, s, (const uint4*)carried, (const u32*)P[pc], m, sorted_words,
-                       sorted_beta);
-    HIP_TRY(hipGetLastError());
-    return finish_partition_step<true>(L, K[kc], sorted_key1, d_keys, P[pc], key_words, sorted_words, sorted_beta, m, 4ull * (u64)key_words, p, h->step64[0],
-                                       h->step64[1], h->idx[3], d_rank_out, d_suf40_out, d_msg_target, d_msg_rank, d_msg_off, res);
-}
-
-int csa_sort_rerank_dev(csa_handle* h, const uint32_t* d_rank, const uint8_t* d_suf40, const uint32_t* d_beta, uint64_t m,
-                        const uint8_t* d_inbox_target, const uint32_t* d_inbox_rank, uint32_t inbox_sz, uint64_t ctx,
-                        uint32_t p, uint32_t* d_rank_out, uint8_t* d_suf40_out, uint8_t* d_msg_target, uint32_t* d_msg_rank,
-                        uint32_t* d_msg_off, void* stream, csa_step_result* res)
-{
-    int rc = check_step_args(h, "csa_sort_rerank_dev", m, p, d_rank, d_suf40, d_beta, d_msg_off);
-    if (rc)
-        return rc;
-    if (res)
-        res->active = res->messages = 0;
-    if (m == 0) {
-        HIP_TRY(hipMemsetAsync(d_msg_off, 0, ((u64)p + 1) * sizeof(u32), (hipStream_t)stream));
-        return CSA_OK;
-    }
-    if (!d_rank_out || !d_suf40_out || !d_msg_target || !d_msg_rank || (inbox_sz && (!d_inbox_target || !d_inbox_rank)))
-        return fail(CSA_ERR_ARG, "csa_sort_rerank_dev: null buffer");
-    Launch L;
-    L.h = h;
-    L.stream = (hipStream_t)stream;
-    L.flags = 0;
-    L.stats = nullptr;
-    hipStream_t s = L.stream;
-    const u32 blocks = (u32)((m + 255) / 256);
-    HIP_TRY(hipMemsetAsync(h->counts, 0, 4 * sizeof(u32), s));
-    u64* K[2] = {h->key[0], h->key[1]};
-    u32* P[2] = {h->idx[0], h->idx[1]};
-    // 1. the cohort in suffix order, so that messages can be joined by search (src/GPU_SACA.cu:1769-1800)
-    hipLaunchKernelGGL(unpack_words_kernel, dim3(blocks), dim3(256), 0, s, d_suf40, (const u32*)nullptr, (const u32*)nullptr, m, 0, K[0],
-                       (u32*)nullptr);
-    hipLaunchKernelGGL(iota_kernel, dim3(blocks), dim3(256), 0, s, P[0], m);
-    int in_out = 0, passes = 0;
-    rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, K[0], P[0], K[1], P[1], (u32)m, make_plan(0, 40), &in_out, &passes);
-    if (rc)
-        return rc;
-    u64* words_by_suffix = K[in_out];
-    u64* free64 = K[in_out ^ 1];
-    u32* perm = P[in_out];
-    u32* primary_by_suffix = h->idx[2];
-    u32* beta_by_suffix = h->idx[3];
-    hipLaunchKernelGGL(gather_u32_kernel, dim3(blocks), dim3(256), 0, s, d_rank, (const u32*)perm, m, primary_by_suffix);
-    hipLaunchKernelGGL(gather_u32_kernel, dim3(blocks), dim3(256), 0, s, d_beta, (const u32*)perm, m, beta_by_suffix);
-    // 2. composite keys from the inbox: primary << 31 | received rank, all ones where nothing arrives
-    //    (src/GPU_SACA.cu:1803-1835)
-    u64* keys = h->key[2];
-    hipLaunchKernelGGL(fill_u64_kernel, dim3(blocks), dim3(256), 0, s, keys, m, ~0ull);
-    if (inbox_sz) {
-        // the permutation of the suffix-order sort has been consumed: its other buffer holds the directory
-        u32* dir = P[in_out ^ 1];
-        u32 dir_log2 = 0;
-        rc = build_join_directory(words_by_suffix, m, dir, h->cap, s, &dir_log2);
-        if (rc)
-            return rc;
-        hipLaunchKernelGGL(join_messages_kernel, dim3((inbox_sz + 255u) / 256u), dim3(256), 0, s, d_inbox_target, (const u64*)nullptr,
-                           d_inbox_rank, inbox_sz, (const u64*)words_by_suffix, (const u32*)primary_by_suffix, keys, m,
-                           (const u32*)(dir_log2 ? dir : nullptr), dir_log2);
-    }
-    HIP_TRY(hipGetLastError());
-    // 3. sort by (primary, secondary): key bits [0, 62) (src/GPU_SACA.cu:1841-1871)
-    hipLaunchKernelGGL(iota_kernel, dim3(blocks), dim3(256), 0, s, P[0], m);
-    rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, keys, P[0], free64, P[1], (u32)m, make_plan(0, 62), &in_out, &passes);
-    if (rc)
-        return rc;
-    u64* sorted_keys = in_out ? free64 : keys;
-    u64* spare64 = in_out ? keys : free64;
-    perm = P[in_out];
-    u64* sorted_words = h->step64[0];
-    u32* sorted_beta = h->idx[4];
-    hipLaunchKernelGGL(gather_u64_kernel, dim3(blocks), dim3(256), 0, s, (const u64*)words_by_suffix, (const u32*)perm, m, 1u, 0u,
-                       sorted_words);
-    hipLaunchKernelGGL(gather_u32_kernel, dim3(blocks), dim3(256), 0, s, (const u32*)beta_by_suffix, (const u32*)perm, m, sorted_beta);
-    HIP_TRY(hipGetLastError());
-    // 4. refine, split, messages, narrow
-    return finish_partition_step<false>(L, sorted_keys, nullptr, nullptr, nullptr, 1, sorted_words, sorted_beta, m, ctx, p, h->step64[1], spare64,
-                                        primary_by_suffix, d_rank_out, d_suf40_out, d_msg_target, d_msg_rank, d_msg_off, res);
-}
 
 int csa_scatter_to_rank_order_dev(csa_handle* h, const uint8_t* d_suf, const uint32_t* d_rank, uint64_t part_sz,
                                   uint8_t* d_sa40, void* stream)
@@ -1686,39 +1478,10 @@ int csa_scatter_to_rank_order_dev(csa_handle* h, const uint8_t* d_suf, const uin
         return fail(CSA_ERR_ARG, "csa_scatter_to_rank_order_dev: null buffer");
     if (part_sz > CSA_MAX_PART_SZ)
         return fail(CSA_ERR_TOO_LARGE, "csa_scatter_to_rank_order_dev: %llu suffixes exceed a partition", (unsigned long long)part_sz);
-    hipStream_t s = (hipStream_t)stream;
-    HIP_TRY(hipMemsetAsync(h->counts, 0, 4 * sizeof(u32), s));
-    const u32 blocks = (u32)((part_sz + 255) / 256);
-    if (part_sz >= SCATTER_WINDOW_MIN && part_sz <= h->cap) {
-        // large partition: group the pairs by the window of the output their rank falls into, then write window by window
-        Launch L;
-        L.h = h;
-        L.stream = s;
-        L.flags = 0;
-        L.stats = nullptr;
-        hipLaunchKernelGGL(scatter_window_keys_kernel, dim3(blocks), dim3(256), 0, s, d_suf, d_rank, part_sz, (int)SCATTER_WINDOW_LOG2,
-                           h->key[0], h->idx[0], h->counts + 3);
-        const int window_bits = bit_length((part_sz - 1) >> SCATTER_WINDOW_LOG2);
-        int in_out = 0, passes = 0;
-        const int rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, h->key[0], h->idx[0], h->key[1], h->idx[1], (u32)part_sz,
-                                  make_plan(40, 40 + window_bits), &in_out, &passes);
-        if (rc)
-            return rc;
-        hipLaunchKernelGGL(scatter_window_lanes_kernel, dim3(blocks), dim3(256), 0, s, (const u64*)h->key[in_out],
-                           (const u32*)h->idx[in_out], part_sz, d_sa40);
-    } else {
-        hipLaunchKernelGGL(scatter_lanes_kernel, dim3(blocks), dim3(256), 0, s, d_suf, d_rank, part_sz, d_sa40, h->counts + 3);
-    }
-    HIP_TRY(hipGetLastError());
-    Launch R;
-    R.h = h;
-    R.stream = s;
-    R.flags = 0;
-    R.stats = nullptr;
-    const int rc_counts = read_counts(R, nullptr); // waits for the stream; a failed wait of the bucket pass ends here
-    if (h->h_pinned[3])
-        return fail(CSA_ERR_ARG, "csa_scatter_to_rank_order_dev: a rank lies outside [0, %llu)", (unsigned long long)part_sz);
-    return rc_counts;
+    h->pool.reset();
+    const int rc = scatter_to_rank_order(h, "csa_scatter_to_rank_order_dev", d_suf, d_rank, part_sz, d_sa40, (hipStream_t)stream);
+    h->last_high_water = h->pool.high_water();
+    return rc;
 }
 
 void csa_output_cut(uint64_t lo, uint64_t hi, uint64_t chunk_bytes, uint64_t c, uint64_t chunk_c, uint64_t out[6])
@@ -1754,59 +1517,103 @@ uint64_t csa_bytes_per_suffix(int key_words)
     return 3 * 8 + 5 * 4 + 4 + 4 + 4 * 2;
 }
 
-int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
+extern "C++" {
+namespace {
+
+constexpr u64 BLOCK_SLACK = 64u << 10; // what rounding every column up to DevicePool::ALIGN can cost a call
+
+struct WorkspaceSizes {
+    u64 lookback_tile_words, lookback_words, rank_tiles_cap;
+    u64 bytes;
+};
+
+// The workspace: what a handle holds besides its block. It follows the number of tiles, not the number of suffixes.
+WorkspaceSizes workspace_sizes(u64 cap)
+{
+    WorkspaceSizes w;
+    const u64 sort_tiles = (cap + SORT_TILE - 1) / SORT_TILE;
+    const u64 rank_tiles = (cap + RANK_TILE - 1) / RANK_TILE;
+    w.lookback_tile_words = sort_tiles * RADIX_BINS; // the group words of the radix pass follow the tile words
+    w.lookback_words = w.lookback_tile_words + (sort_tiles / LB_GROUP + 1) * RADIX_BINS;
+    if (rank_tiles * 4 > w.lookback_words)
+        w.lookback_words = rank_tiles * 4;
+    w.rank_tiles_cap = rank_tiles + 1;
+    w.bytes = w.lookback_words * 8 + (w.rank_tiles_cap * 9 + RERANK_SLABS * 5) * sizeof(u32) + (MAX_PASSES + 2) * RADIX_BINS * 4 +
+              MAX_PASSES * RADIX_BINS * 4 + TICKET_POOL * 4 + 16 * 4 + MSG_OFF_WORDS * 4;
+    w.bytes += 9 * 4096; // nine allocations, each rounded up by the runtime
+    return w;
+}
+
+u64 resident_block_bytes(u64 cap)
+{
+    const u64 A = DevicePool::ALIGN;
+    auto up = [&](u64 b) { return (b + A - 1) & ~(A - 1); };
+    return 3 * up(cap * 8) + 5 * up(cap * 4) + 2 * up(cap * 4) + 2 * up((cap / 2 + 1) * 4) + 2 * up((cap / 2 + 2) * 4);
+}
+
+int create_handle(const char* who, u64 max_part_sz, int key_words, u32 kinds, csa_handle** out)
 {
     if (!out)
-        return fail(CSA_ERR_ARG, "csa_create: out is null");
+        return fail(CSA_ERR_ARG, "%s: out is null", who);
     *out = nullptr;
     if (key_words < 1 || key_words > 4)
-        return fail(CSA_ERR_ARG, "csa_create: key_words = %d is outside [1, 4]", key_words);
+        return fail(CSA_ERR_ARG, "%s: key_words = %d is outside [1, 4]", who, key_words);
     if (max_part_sz > CSA_MAX_PART_SZ)
-        return fail(CSA_ERR_TOO_LARGE, "csa_create: %llu suffixes exceed the partition limit %llu",
+        return fail(CSA_ERR_TOO_LARGE, "%s: %llu suffixes exceed the partition limit %llu", who,
                     (unsigned long long)max_part_sz, (unsigned long long)CSA_MAX_PART_SZ);
     csa_handle* h = new csa_handle();
     h->cap = max_part_sz ? max_part_sz : 1;
     h->key_words = key_words;
+    h->kinds = kinds;
     const u64 cap = h->cap;
-    const u64 sort_tiles = (cap + SORT_TILE - 1) / SORT_TILE;
-    const u64 rank_tiles = (cap + RANK_TILE - 1) / RANK_TILE;
-    h->lookback_tile_words = sort_tiles * RADIX_BINS; // the group words of the radix pass follow the tile words
-    h->lookback_words = h->lookback_tile_words + (sort_tiles / LB_GROUP + 1) * RADIX_BINS;
-    if (rank_tiles * 4 > h->lookback_words)
-        h->lookback_words = rank_tiles * 4;
+    const WorkspaceSizes ws = workspace_sizes(cap);
+    h->lookback_tile_words = ws.lookback_tile_words;
+    h->lookback_words = ws.lookback_words;
     hipError_t e = hipGetDevice(&h->device);
-    int cus = 0;
     if (e == hipSuccess)
-        e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, h->device);
+        e = hipDeviceGetAttribute(&h->cus, hipDeviceAttributeMultiprocessorCount, h->device);
     // Tile order of the radix passes: by arrival, unless the caller declares the device its own
     // (csa_set_device_exclusive); the XCD-chunked order then needs 8 * XCD_CHUNK workgroups of a pass resident at once
     // and is offered only on a device with room for twice that many (csa_set_tuning changes the chunk length).
     h->tile_order = TILES_BY_ARRIVAL;
-    h->tile_order_exclusive = cus >= 2 * 8 * (int)XCD_CHUNK ? TILES_STATIC_CHUNKS : TILES_BY_ARRIVAL;
+    h->tile_order_exclusive = h->cus >= 2 * 8 * (int)XCD_CHUNK ? TILES_STATIC_CHUNKS : TILES_BY_ARRIVAL;
     h->xcd_chunk = XCD_CHUNK;
     auto alloc = [&](void** p, u64 bytes) {
         if (e == hipSuccess)
             e = hipMalloc(p, bytes ? bytes : 4);
     };
-    for (int i = 0; i < 3; ++i)
-        alloc((void**)&h->key[i], cap * 8);
-    for (int i = 0; i < 5; ++i)
-        alloc((void**)&h->idx[i], cap * 4);
-    alloc((void**)&h->gid, cap * 4);
-    alloc((void**)&h->rank, cap * 4);
-    alloc((void**)&h->gprim[0], (cap / 2 + 1) * 4);
-    alloc((void**)&h->gprim[1], (cap / 2 + 1) * 4);
-    alloc((void**)&h->gstart[0], (cap / 2 + 2) * 4);
-    alloc((void**)&h->gstart[1], (cap / 2 + 2) * 4);
+    // the block: the resident sort's floor plan, or what the steps keep alive at their busiest moment
+    u64 block_bytes = ((kinds & KIND_RESIDENT) ? resident_block_bytes(cap) : csa_step_bytes_per_suffix(key_words) * cap) + BLOCK_SLACK;
+    block_bytes = (block_bytes + DevicePool::ALIGN - 1) & ~(DevicePool::ALIGN - 1);
+    alloc((void**)&h->block, block_bytes);
+    if (e == hipSuccess) {
+        h->pool.attach(h->block, block_bytes);
+        if (kinds & KIND_RESIDENT) { // the fixed carve-up of the resident sort
+            for (int i = 0; i < 3; ++i)
+                h->key[i] = static_cast<u64*>(h->pool.take(cap * 8));
+            for (int i = 0; i < 5; ++i)
+                h->idx[i] = static_cast<u32*>(h->pool.take(cap * 4));
+            h->gid = static_cast<u32*>(h->pool.take(cap * 4));
+            h->rank = static_cast<u32*>(h->pool.take(cap * 4));
+            for (int i = 0; i < 2; ++i)
+                h->gprim[i] = static_cast<u32*>(h->pool.take((cap / 2 + 1) * 4));
+            for (int i = 0; i < 2; ++i)
+                h->gstart[i] = static_cast<u32*>(h->pool.take((cap / 2 + 2) * 4));
+            if (!h->gstart[1])
+                e = hipErrorOutOfMemory; // (cannot happen: the block was sized by the same sum)
+            h->pool.reset();
+        }
+    }
     alloc((void**)&h->lookback, h->lookback_words * 8);
-    h->rank_tiles_cap = rank_tiles + 1;
+    h->rank_tiles_cap = ws.rank_tiles_cap;
     alloc((void**)&h->tile_tables, (h->rank_tiles_cap * 9 + RERANK_SLABS * 5) * sizeof(u32));
     alloc((void**)&h->ghist, (MAX_PASSES + 2) * RADIX_BINS * 4);
     alloc((void**)&h->digit_base, MAX_PASSES * RADIX_BINS * 4);
     alloc((void**)&h->tickets, TICKET_POOL * 4);
     alloc((void**)&h->counts, 16 * 4);
+    alloc((void**)&h->msg_off, MSG_OFF_WORDS * 4);
     if (e == hipSuccess)
-        e = hipHostMalloc((void**)&h->h_pinned, (16 + MAX_PASSES * RADIX_BINS) * 4, hipHostMallocDefault);
+        e = hipHostMalloc((void**)&h->h_pinned, (PINNED_HIST + MAX_PASSES * RADIX_BINS) * 4, hipHostMallocDefault);
     if (e == hipSuccess)
         e = hipMemset(h->lookback, 0, h->lookback_words * 8);
     if (e == hipSuccess)
@@ -1816,13 +1623,27 @@ int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
     if (e == hipSuccess)
         e = hipDeviceSynchronize();
     if (e != hipSuccess) {
-        const int rc = fail(CSA_ERR_HIP, "csa_create: %s while allocating for %llu suffixes", hipGetErrorString(e),
-                            (unsigned long long)cap);
+        const int rc = fail(CSA_ERR_HIP, "%s: %s while allocating for %llu suffixes", who, hipGetErrorString(e), (unsigned long long)cap);
         csa_destroy(h);
         return rc;
     }
     *out = h;
     return CSA_OK;
+}
+
+} // namespace
+} // extern "C++"
+
+uint64_t csa_workspace_bytes(uint64_t max_part_sz) { return workspace_sizes(max_part_sz ? max_part_sz : 1).bytes + BLOCK_SLACK; }
+
+int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out)
+{
+    return create_handle("csa_create", max_part_sz, key_words, KIND_RESIDENT, out);
+}
+
+int csa_create_steps(uint64_t max_part_sz, int key_words, csa_handle** out)
+{
+    return create_handle("csa_create_steps", max_part_sz, key_words, 0u, out);
 }
 
 int csa_set_tuning(csa_handle* h, int knob, uint32_t value)
@@ -1833,6 +1654,11 @@ int csa_set_tuning(csa_handle* h, int knob, uint32_t value)
     case CSA_TUNE_DEFER_MIN: h->defer_min = value; break;
     case CSA_TUNE_WINDOW_MIN_CHANGED: h->window_min_changed = value; break;
     case CSA_TUNE_XCD_CHUNK:
+        // the chunked order waits for workgroups that are dispatched later: 8 * chunk workgroups of a pass must be able
+        // to be resident together, and the device must have room for twice that many (the condition csa_create applies)
+        if (value && 2ull * 8ull * value > (u64)(h->cus > 0 ? h->cus : 0))
+            return fail(CSA_ERR_ARG, "csa_set_tuning: an XCD chunk of %u tiles needs %llu compute units, the device has %d", value,
+                        2ull * 8ull * value, h->cus);
         h->tile_order_exclusive = value ? TILES_STATIC_CHUNKS : TILES_BY_ARRIVAL;
         if (value)
             h->xcd_chunk = value;
@@ -1856,24 +1682,14 @@ void csa_destroy(csa_handle* h)
 {
     if (!h)
         return;
-    free_slab_arena(h);
-    for (int i = 0; i < 3; ++i)
-        (void)hipFree(h->key[i]);
-    for (int i = 0; i < 5; ++i)
-        (void)hipFree(h->idx[i]);
-    (void)hipFree(h->gstart[0]);
-    (void)hipFree(h->gstart[1]);
-    (void)hipFree(h->gid);
-    (void)hipFree(h->rank);
-    (void)hipFree(h->gprim[0]);
-    (void)hipFree(h->gprim[1]);
+    (void)hipFree(h->block);
     (void)hipFree(h->lookback);
     (void)hipFree(h->tile_tables);
     (void)hipFree(h->ghist);
     (void)hipFree(h->digit_base);
     (void)hipFree(h->tickets);
-    (void)hipFree(h->step64[0]); // (both halves)
     (void)hipFree(h->counts);
+    (void)hipFree(h->msg_off);
     if (h->h_pinned)
         (void)hipHostFree(h->h_pinned);
     for (auto& e : h->events)
@@ -1895,6 +1711,9 @@ int csa_sort_partition_u16_dev(csa_handle* h, const uint16_t* d_text, uint64_t n
     if (index_base > CSA_MAX_INDEX || index_base + n > CSA_MAX_INDEX)
         return fail(CSA_ERR_TOO_LARGE, "csa_sort_partition_u16_dev: suffix indices up to %llu do not fit 40 bits",
                     (unsigned long long)(index_base + n));
+    if (!(h->kinds & KIND_RESIDENT))
+        return fail(CSA_ERR_ARG, "csa_sort_partition_u16_dev: the handle was created by csa_create_steps, which leaves out the "
+                    "resident sort's arrays; use csa_create");
     if (n > h->cap)
         return fail(CSA_ERR_ARG, "csa_sort_partition_u16_dev: %llu suffixes exceed the handle's capacity %llu",
                     (unsigned long long)n, (unsigned long long)h->cap);
@@ -1956,15 +1775,21 @@ int csa_radix_sort_pairs_dev(csa_handle* h, uint64_t* d_keys, uint32_t* d_vals, 
     L.flags = 0;
     L.stats = nullptr;
     HIP_TRY(hipMemsetAsync(h->counts, 0, 4 * sizeof(u32), L.stream));
+    h->pool.reset();
+    u64* tmp_keys = static_cast<u64*>(h->pool.take(n * 8));
+    u32* tmp_vals = static_cast<u32*>(h->pool.take(n * 4));
+    h->last_high_water = h->pool.high_water();
+    if (!tmp_keys || !tmp_vals)
+        return fail(CSA_ERR_ARG, "csa_radix_sort_pairs_dev: the handle's block of %llu bytes has no room for 12 bytes per pair",
+                    (unsigned long long)h->pool.bytes());
     int in_out = 0, passes = 0;
     const PassPlan plan = make_plan(begin_bit, end_bit);
-    int rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, d_keys, d_vals, h->key[0], h->idx[0], (u32)n, plan, &in_out,
-                        &passes);
+    int rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, d_keys, d_vals, tmp_keys, tmp_vals, (u32)n, plan, &in_out, &passes);
     if (rc)
         return rc;
     if (in_out) {
-        HIP_TRY(hipMemcpyAsync(d_keys, h->key[0], n * 8, hipMemcpyDeviceToDevice, L.stream));
-        HIP_TRY(hipMemcpyAsync(d_vals, h->idx[0], n * 4, hipMemcpyDeviceToDevice, L.stream));
+        HIP_TRY(hipMemcpyAsync(d_keys, tmp_keys, n * 8, hipMemcpyDeviceToDevice, L.stream));
+        HIP_TRY(hipMemcpyAsync(d_vals, tmp_vals, n * 4, hipMemcpyDeviceToDevice, L.stream));
     }
     return read_counts(L, nullptr);
 }
@@ -2070,6 +1895,22 @@ int csa_radix_sort_pairs_static_dev(uint64_t* d_keys, uint32_t* d_vals, uint64_t
     return CSA_OK;
 }
 
+int csa_radix_sort_pairs_static_status(void* stream)
+{
+    unsigned char* base = nullptr; // (the device address of the scratch array, as in the sort itself)
+    int rc = static_scratch(&base);
+    if (rc)
+        return rc;
+    hipStream_t s = (hipStream_t)stream;
+    u32 err = 0; // one word into the caller's stack: no buffer is allocated for it
+    HIP_TRY(hipMemcpyAsync(&err, base + STATIC_OFF_ERR, sizeof(u32), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    if (err)
+        return fail(CSA_ERR_INTERNAL, "csa_radix_sort_pairs_static_dev: device invariant %u failed in the last sort on this device%s", err,
+                    err == DEV_ERR_LOOKBACK_TIMEOUT ? " (a look-back wait ran into its spin limit): the pairs it left are not sorted" : "");
+    return CSA_OK;
+}
+
 int csa_verify_sa40_dev(csa_handle* h, const uint16_t* d_text, uint64_t n, uint64_t index_base,
                         const uint8_t* d_sa40, void* stream, int* ok)
 {
@@ -2087,11 +1928,17 @@ int csa_verify_sa40_dev(csa_handle* h, const uint16_t* d_text, uint64_t n, uint6
         return fail(CSA_ERR_ARG, "csa_verify_sa40_dev: null pointer");
     hipStream_t s = (hipStream_t)stream;
     const u32 blocks = (u32)((n + 255) / 256);
+    h->pool.reset();
+    u32* inverse = static_cast<u32*>(h->pool.take(n * sizeof(u32))); // the inverse suffix array
+    h->last_high_water = h->pool.high_water();
+    if (!inverse)
+        return fail(CSA_ERR_ARG, "csa_verify_sa40_dev: the handle's block of %llu bytes has no room for 4 bytes per suffix",
+                    (unsigned long long)h->pool.bytes());
     HIP_TRY(hipMemsetAsync(h->counts + 3, 0, sizeof(u32), s));
-    hipLaunchKernelGGL(fill_u32_kernel, dim3(blocks), dim3(256), 0, s, h->rank, n, 0xFFFFFFFFu);
-    hipLaunchKernelGGL(verify_invert_kernel, dim3(blocks), dim3(256), 0, s, d_sa40, (u32)n, index_base, h->rank,
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(blocks), dim3(256), 0, s, inverse, n, 0xFFFFFFFFu);
+    hipLaunchKernelGGL(verify_invert_kernel, dim3(blocks), dim3(256), 0, s, d_sa40, (u32)n, index_base, inverse,
                        h->counts + 3);
-    hipLaunchKernelGGL(verify_order_kernel, dim3(blocks), dim3(256), 0, s, d_sa40, d_text, (u32)n, index_base, h->rank,
+    hipLaunchKernelGGL(verify_order_kernel, dim3(blocks), dim3(256), 0, s, d_sa40, d_text, (u32)n, index_base, inverse,
                        h->counts + 3);
     HIP_TRY(hipGetLastError());
     HIP_TRY(hipMemcpyAsync(h->h_pinned + 3, h->counts + 3, sizeof(u32), hipMemcpyDeviceToHost, s));
@@ -2109,5 +1956,6 @@ int csa_enable_profile_ranges(int enable)
 
 } // extern "C"
 
+#include "step_entries.hpp"
 #include "slab_entries.hpp"
 #include "host_pipeline.hpp"

@@ -1,5 +1,5 @@
 // Partitions that arrive in host memory and leave to host memory: upload, sort and download run as a three-stage
-// pipeline on three streams, so that the transfers of one partition hide behind the sort of another, as the three
+// pipeline on four streams (one up, one for the sort, two down), so that the transfers of one partition hide behind the sort of another, as the three
 // dispatcher threads of the reference overlap them (src/GPU_SACA.cu:1539-1589). Host code only; included by
 // cascade_hip.hip after the C ABI's definitions.
 #pragma once
@@ -7,8 +7,10 @@
 #include <condition_variable>
 #include <thread>
 
-// pieces a transfer is cut into, each on a stream of its own (12 texts of 2^26 symbols, pinned memory, whole job:
-// 152 ms with one piece, where one copy engine brings 29 GB/s down; 106 ms with two, 46 GB/s; 120 ms with four)
+// pieces a download is cut into, each on a stream of its own (12 texts of 2^26 symbols, pinned memory, whole job:
+// 152 ms with one piece, where one copy engine brings 29 GB/s down; 106 ms with two, 46 GB/s; 120 ms with four).
+// The uploads (2 of the 7 bytes per suffix) travel on one stream: with the sort's stream that makes four streams, one
+// per hardware queue a process has by default; a fifth would share a queue with another and wait behind it.
 #ifndef CSA_PIPELINE_COPY_WAYS
 #define CSA_PIPELINE_COPY_WAYS 2
 #endif
@@ -107,8 +109,8 @@ int csa_sort_partitions_u16(uint32_t count, const uint16_t* const* h_texts, cons
     const u32 sets = count > 1 ? 2 : 1;
     u16* d_text[2] = {nullptr, nullptr};
     u8* d_sa[2] = {nullptr, nullptr};
-    constexpr u32 WAYS = CSA_PIPELINE_COPY_WAYS;
-    hipStream_t st_up[WAYS] = {}, st_sort = nullptr, st_down[WAYS] = {};
+    constexpr u32 WAYS = CSA_PIPELINE_COPY_WAYS, UP_WAYS = 1;
+    hipStream_t st_up[UP_WAYS] = {}, st_sort = nullptr, st_down[WAYS] = {};
     hipError_t e = hipSuccess;
     for (u32 b = 0; b < sets && e == hipSuccess; ++b) {
         e = hipMalloc((void**)&d_text[b], max_n ? max_n * 2 : 4);
@@ -116,12 +118,12 @@ int csa_sort_partitions_u16(uint32_t count, const uint16_t* const* h_texts, cons
             e = hipMalloc((void**)&d_sa[b], max_n ? max_n * 5 : 4);
     }
     // (all at the default priority)
-    for (u32 w = 0; w < WAYS; ++w) {
+    for (u32 w = 0; w < UP_WAYS; ++w)
         if (e == hipSuccess)
             e = hipStreamCreateWithFlags(&st_up[w], hipStreamNonBlocking);
+    for (u32 w = 0; w < WAYS; ++w)
         if (e == hipSuccess)
             e = hipStreamCreateWithFlags(&st_down[w], hipStreamNonBlocking);
-    }
     if (e == hipSuccess)
         e = hipStreamCreateWithFlags(&st_sort, hipStreamNonBlocking);
     if (e != hipSuccess)
@@ -137,7 +139,7 @@ int csa_sort_partitions_u16(uint32_t count, const uint16_t* const* h_texts, cons
                 // the buffer of partition k was last read by the sort of partition k - 2
                 if (k >= 2 && !pipe.wait_for(pipe.sorted, k - 1))
                     return;
-                const int c = copy_through(st_up, WAYS, d_text[k % sets], h_texts[k], n[k] * 2, hipMemcpyHostToDevice);
+                const int c = copy_through(st_up, UP_WAYS, d_text[k % sets], h_texts[k], n[k] * 2, hipMemcpyHostToDevice);
                 if (c)
                     return pipe.failed(c);
                 pipe.advance(pipe.uploaded);
@@ -174,12 +176,12 @@ int csa_sort_partitions_u16(uint32_t count, const uint16_t* const* h_texts, cons
         if (pipe.status != CSA_OK)
             rc = fail(pipe.status, "%s", pipe.message);
     }
-    for (u32 w = 0; w < WAYS; ++w) {
+    for (u32 w = 0; w < UP_WAYS; ++w)
         if (st_up[w])
             (void)hipStreamDestroy(st_up[w]);
+    for (u32 w = 0; w < WAYS; ++w)
         if (st_down[w])
             (void)hipStreamDestroy(st_down[w]);
-    }
     if (st_sort)
         (void)hipStreamDestroy(st_sort);
     for (u32 b = 0; b < 2; ++b) {

@@ -190,6 +190,14 @@ __global__ __launch_bounds__(256) void pack_carried_kernel(const u8* __restrict_
     carried[i] = make_uint4((u32)v, (u32)(v >> 32), bt, 0u);
 }
 
+// keys[i] = forward tag of suffix i, from its carried record
+__global__ __launch_bounds__(256) void carried_tag_keys_kernel(const uint4* __restrict__ carried, u64 count, u64* __restrict__ keys)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i < count)
+        keys[i] = carried[i].z >> 16;
+}
+
 // words[i], beta_out[i] = the record of suffix perm[i]
 __global__ __launch_bounds__(256) void gather_carried_kernel(const uint4* __restrict__ carried, const u32* __restrict__ perm, u64 count,
                                                              u64* __restrict__ words, u32* __restrict__ beta_out)
@@ -227,6 +235,12 @@ struct StepRankArgs {
     u32 slab;
     u32 slabs;
     unsigned long long* active_out; // size of the active set
+    // generation t: what the reference counts and checks under -DTESTS (include/GPU_SACA.cuh:234-249): cohort members no
+    // message joined, members a poison pill joined, and neighbours with equal (primary, secondary) of which only one
+    // carries a pill receipt
+    unsigned long long* unserved_out;
+    unsigned long long* pills_out;
+    u32* incoherent_out;
 };
 
 template <bool GEN0>
@@ -253,13 +267,13 @@ template <bool GEN0, bool APPLY>
 __global__ __launch_bounds__(STEP_BLOCK) void step_rank_kernel(StepRankArgs a)
 {
     constexpr int WAVES = STEP_BLOCK / WAVE;
-    __shared__ u32 s_w[WAVES][3];
+    __shared__ u32 s_w[WAVES][5];
     const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
     const u32 tile = blockIdx.x;
     const u64 base = (u64)tile * STEP_TILE + (u64)t * STEP_ITEMS;
     // heads are 1-based positions (0 = none so far)
     bool kh[STEP_ITEMS + 1], ph[STEP_ITEMS];
-    u32 la = 0, lb = 0, lact = 0;
+    u32 la = 0, lb = 0, lact = 0, lun = 0, lpill = 0;
 #pragma unroll
     for (int k = 0; k < STEP_ITEMS + 1; ++k) {
         const u64 i = base + k;
@@ -275,13 +289,31 @@ __global__ __launch_bounds__(STEP_BLOCK) void step_rank_kernel(StepRankArgs a)
             if (ph[k])
                 lb = (u32)i + 1u;
             lact += (kh[k] && kh[k + 1]) ? 0u : 1u;
+            if (!GEN0 && !APPLY) {
+                const u64 key = a.key0[i];
+                if ((key & STEP_SECONDARY) == STEP_SECONDARY)
+                    lun++;
+                else if (key & MSG_PILL_RECEIPT)
+                    lpill++;
+                if (i > 0) {
+                    const u64 differ = key ^ a.key0[i - 1];
+                    if ((differ & STEP_KEY62) == 0 && (differ & MSG_PILL_RECEIPT))
+                        atomicAdd(a.incoherent_out, 1u);
+                }
+            }
         }
     }
     const u32 ia = wave_incl_max(la), ib = wave_incl_max(lb), ic = wave_incl_sum(lact);
+    if (!GEN0 && !APPLY) {
+        lun = wave_reduce_sum(lun);
+        lpill = wave_reduce_sum(lpill);
+    }
     if (lane == 63u) {
         s_w[w][0] = ia;
         s_w[w][1] = ib;
         s_w[w][2] = ic;
+        s_w[w][3] = lun;
+        s_w[w][4] = lpill;
     }
     __syncthreads();
     u32 xa = __shfl_up(ia, 1), xb = __shfl_up(ib, 1), xc = __shfl_up(ic, 1);
@@ -300,11 +332,16 @@ __global__ __launch_bounds__(STEP_BLOCK) void step_rank_kernel(StepRankArgs a)
     }
     if (!APPLY) {
         if (t == 0) {
+            u32 tun = 0, tpill = 0;
+            for (u32 ww = 0; ww < WAVES; ++ww) {
+                tun += s_w[ww][3];
+                tpill += s_w[ww][4];
+            }
             a.tile_agg[(u64)tile * 4 + 0] = ta;
             a.tile_agg[(u64)tile * 4 + 1] = tb;
             a.tile_agg[(u64)tile * 4 + 2] = tc;
-            a.tile_agg[(u64)tile * 4 + 3] = 0;
-            a.tile_splits[tile] = 0;
+            a.tile_agg[(u64)tile * 4 + 3] = tun;  // summed by the scan like the active count
+            a.tile_splits[tile] = tpill;          // at most STEP_TILE: the scan adds the low 16 bits up per slab
         }
         return;
     }
@@ -314,9 +351,19 @@ __global__ __launch_bounds__(STEP_BLOCK) void step_rank_kernel(StepRankArgs a)
     pre_a = pre_a > sp.max0 ? pre_a : sp.max0;
     pre_b = pre_b > sp.max1 ? pre_b : sp.max1;
     pre_c += sp.sum2;
-    const u32 total_active = slabs_before(a.slab_total, a.slabs).sum2;
-    if (tile == 0 && t == 0)
-        *a.active_out = total_active;
+    const SlabPrefix all = slabs_before(a.slab_total, a.slabs);
+    const u32 total_active = all.sum2;
+    if (tile == 0 && w == 0) {
+        u32 pills = lane < a.slabs ? a.slab_total[lane * 5 + 4] : 0u; // one slab per lane
+        pills = wave_reduce_sum(pills);
+        if (lane == 0) {
+            *a.active_out = total_active;
+            if (!GEN0) {
+                *a.unserved_out = all.sum3;
+                *a.pills_out = pills;
+            }
+        }
+    }
     u32 ra = xa > pre_a ? xa : pre_a, rb = xb > pre_b ? xb : pre_b;
     u32 act_before = pre_c + xc; // active entries before this thread's first
 #pragma unroll

@@ -37,12 +37,15 @@ def stats_to_dict(st):
 
 
 class PartitionSorter:
-    """Owns the device scratch for partitions of up to `max_part_sz` suffixes (csa_create / csa_destroy)."""
+    """Owns the device scratch for partitions of up to `max_part_sz` suffixes (csa_create / csa_destroy).
+    for_steps: the handle is made by csa_create_steps instead: sized for the per-generation steps
+    (csa_step_bytes_per_suffix), without the arrays of the resident sort, which then refuses it."""
 
-    def __init__(self, max_part_sz, key_words=1, device_exclusive=False):
+    def __init__(self, max_part_sz, key_words=1, device_exclusive=False, for_steps=False):
         self._lib = _native.load()
         self._h = C.c_void_p()
-        _native.check(self._lib.csa_create(int(max_part_sz), int(key_words), C.byref(self._h)))
+        create = self._lib.csa_create_steps if for_steps else self._lib.csa_create
+        _native.check(create(int(max_part_sz), int(key_words), C.byref(self._h)))
         self.max_part_sz = int(max_part_sz)
         self.key_words = int(key_words)
         self.last_stats = None
@@ -79,6 +82,14 @@ class PartitionSorter:
     @staticmethod
     def bytes_per_suffix(key_words=1):
         return int(_native.load().csa_bytes_per_suffix(int(key_words)))
+
+    @staticmethod
+    def step_bytes_per_suffix(key_words=1):
+        return int(_native.load().csa_step_bytes_per_suffix(int(key_words)))
+
+    def scratch_high_water(self):
+        """Bytes of the handle's block that the last call held at its busiest moment (csa_scratch_high_water)."""
+        return int(self._lib.csa_scratch_high_water(self._h))
 
     def sort_ptr(self, d_text, n, d_sa40, index_base=0, stream=0, flags=0):
         """Raw device pointers in, statistics out (csa_sort_partition_u16_dev)."""

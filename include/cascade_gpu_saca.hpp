@@ -111,21 +111,47 @@ public:
         for (idx_t b = 0; b < STREAM_C; ++b)
             if (csa_[b])
                 csa_destroy(csa_[b]);
+        for (idx_t b = 0; b < STREAM_C; ++b)
+            if (resident_[b])
+                csa_destroy(resident_[b]);
     }
 
-    // Largest partition that STREAM_C buffer sets of the library's floor plan fit into free_device_bytes (the
-    // reference balances three partitions over the device memory the same way, src/GPU_SACA.cu:372,557).
+    static constexpr double MEM_SAFETY_MARGIN = 0.1;        // spared for the runtime (include/GPU_SACA.hpp:44)
+    static constexpr double PART_SZ_IMBALANCE_SLACK = 1.20; // partitions may come out larger than planned (include/GPU_SACA.hpp:61)
+
+    // Largest partition such that STREAM_C handles of the steps' floor plan, workspaces included, fit into
+    // free_device_bytes with the reference's margins (src/GPU_SACA.cu:365-403): a host that creates its partitions no
+    // larger than this finds that allocate_device_space() succeeds and that no step runs out of device memory, because
+    // the steps allocate nothing.
     idx_t partition_size_upper_bound(std::size_t free_device_bytes) const
     {
-        const idx_t by_memory = free_device_bytes / (STREAM_C * csa_bytes_per_suffix(key_words_));
-        return by_memory < CSA_MAX_PART_SZ ? by_memory : CSA_MAX_PART_SZ;
+        const double budget_f = static_cast<double>(free_device_bytes) * (1.0 - MEM_SAFETY_MARGIN) / PART_SZ_IMBALANCE_SLACK;
+        const std::size_t budget = static_cast<std::size_t>(budget_f);
+        const std::size_t per_suffix = csa_step_bytes_per_suffix(key_words_);
+        idx_t p_sz_max = budget / (STREAM_C * per_suffix);
+        if (p_sz_max > CSA_MAX_PART_SZ)
+            p_sz_max = CSA_MAX_PART_SZ;
+        // the workspace follows the partition size: shrink until block and workspace fit together
+        while (p_sz_max > 0 && STREAM_C * (p_sz_max * per_suffix + csa_workspace_bytes(p_sz_max)) > budget) {
+            const std::size_t ws = STREAM_C * csa_workspace_bytes(p_sz_max);
+            const idx_t next = ws >= budget ? 0 : (budget - ws) / (STREAM_C * per_suffix);
+            p_sz_max = next < p_sz_max ? next : p_sz_max - 1;
+        }
+        return p_sz_max;
     }
 
-    // One handle per buffer set; false if the device has no room (the reference returns the same way).
+    // What allocate_device_space() takes from the device for partitions of up to part_sz suffixes.
+    std::size_t device_bytes_required(idx_t part_sz) const
+    {
+        return STREAM_C * (part_sz * csa_step_bytes_per_suffix(key_words_) + csa_workspace_bytes(part_sz));
+    }
+
+    // One handle per buffer set, each with everything the three members will ever use; false if the device has no
+    // room (the reference returns the same way, src/GPU_SACA.cu:550-560).
     bool allocate_device_space()
     {
         for (idx_t b = 0; b < STREAM_C; ++b)
-            if (!csa_[b] && csa_create(max_part_sz_, key_words_, &csa_[b]) != CSA_OK) {
+            if (!csa_[b] && csa_create_steps(max_part_sz_, key_words_, &csa_[b]) != CSA_OK) {
                 std::cerr << csa_last_error() << "\n";
                 return false;
             }
@@ -168,6 +194,16 @@ public:
         check(csa_sort_rerank_slabs(csa_[buf_id], slabs.data(), static_cast<std::uint32_t>(slabs.size()), total(slabs), inbox_sz, ctx_,
                                     p_, chunk_cap_, msg_off(p_id), active_slot(p_id), stream_[buf_id]));
         spread(slabs, p_assembly);
+#ifdef TESTS
+        // what the reference checks after a generation under -DTESTS (src/GPU_SACA.cu:2055-2063; the device trap of
+        // include/GPU_SACA.cuh:246-249)
+        csa_step_result r{};
+        check(csa_last_step_result(csa_[buf_id], &r));
+        if (r.unserved > 0)
+            fail("Active suffixes with no message received: " + std::to_string(r.unserved));
+        if (r.incoherent_pills > 0)
+            fail("Incoherent poison-pill receipts: " + std::to_string(r.incoherent_pills));
+#endif
     }
 
     // Lanes and final ranks in the slabs -> the partition's stretch of the output, cut for the output file whose
@@ -205,11 +241,15 @@ public:
         check(csa_scatter_to_rank_order_dev(csa_[buf_id], suf, rank, part_sz, sa40, stream_[buf_id]));
     }
 
-    // A partition whose symbols are a window of the text resident in HBM: every generation inside one call.
+    // A partition whose symbols are a window of the text resident in HBM: every generation inside one call. The handles
+    // of allocate_device_space() are made for the steps; this member keeps handles of its own (csa_create), made on
+    // first use.
     void sort_partition(const T_sym_* d_text, idx_t part_sz, idx_t index_base, std::uint8_t* d_sa40, idx_t buf_id,
                         csa_stats* stats = nullptr)
     {
-        check(csa_sort_partition_u16_dev(csa_[buf_id], reinterpret_cast<const std::uint16_t*>(d_text), part_sz, index_base, d_sa40,
+        if (!resident_[buf_id])
+            check(csa_create(max_part_sz_, key_words_, &resident_[buf_id]));
+        check(csa_sort_partition_u16_dev(resident_[buf_id], reinterpret_cast<const std::uint16_t*>(d_text), part_sz, index_base, d_sa40,
                                          stream_[buf_id], 0, stats));
     }
 
@@ -279,6 +319,7 @@ private:
     std::vector<idx_t> active_sz_;
     idx_t ctx_ = 0, gen_ = 0;
     csa_handle* csa_[STREAM_C] = {};
+    csa_handle* resident_[STREAM_C] = {};
     void* stream_[STREAM_C] = {};
     csa_stats stats_{};
 };

@@ -69,18 +69,49 @@ typedef struct csa_stats {
 
 typedef struct csa_handle csa_handle;
 
-/* Device bytes the handle holds per suffix of capacity (text and output excluded).
- * Replaces the sizing of the reference's GPU_SACA::partition_size_upper_bound / allocate_device_space
- * (include/GPU_SACA.hpp:209,221; src/GPU_SACA.cu:372,535-590). */
+/* ---- sizing: what a handle holds on the device ----
+ * A handle owns one block of device memory that scales with its capacity, and a workspace that follows the number of
+ * tiles (look-back words, per-tile tables, digit counts, the outbox counters). Both are allocated by csa_create /
+ * csa_create_steps and nothing is allocated afterwards: every entry point that takes a handle works inside them.
+ * Replaces the sizing of the reference's GPU_SACA::partition_size_upper_bound / allocate_device_space / cub_workspace_size
+ * (include/GPU_SACA.hpp:209,217,221; src/GPU_SACA.cu:365-380,457-531,535-590), whose floor plan is
+ * 2 * (max(8 * key_words, 16) + 8 + 4 + 4) + 1 = 65 / 65 / 81 / 97 bytes per suffix for key_words = 1 / 2 / 3 / 4. */
+
+/* Block bytes per suffix of a handle made by csa_create (text and output excluded): the floor plan of the sort that
+ * keeps the partition resident, 60 whatever the key width. Such a handle serves every entry point; the per-generation
+ * steps find room in it for partitions of up to capacity * 60 / csa_step_bytes_per_suffix(key_words) suffixes. */
 uint64_t csa_bytes_per_suffix(int key_words);
 
-/* Allocates the scratch for partitions of up to max_part_sz suffixes on the current device.
+/* Block bytes per suffix of a handle made by csa_create_steps: what the per-generation steps (csa_sort_init_*,
+ * csa_sort_rerank_*, csa_scatter_*), their slab-shaped forms included, need for a partition, inputs and outputs on the
+ * device included: 48 with one-word keys, 65 with two words, 8 * key_words + 52 = 76 / 84 with three / four.
+ * Every column of a step has a fixed place in the block and columns whose lives do not overlap share a place, which is
+ * how the reference reaches its own figure (src/GPU_SACA.cu:1268-1270,1292,1301,1805-1806). */
+uint64_t csa_step_bytes_per_suffix(int key_words);
+
+/* Bytes of the workspace of a handle for partitions of up to max_part_sz suffixes, rounding slack of the block
+ * included (about 0.3 bytes per suffix plus 0.6 MB): what a host adds per handle when it sizes partitions against free
+ * device memory, as the reference adds cub's workspace (src/GPU_SACA.cu:385-403). */
+uint64_t csa_workspace_bytes(uint64_t max_part_sz);
+
+/* Allocates block and workspace for partitions of up to max_part_sz suffixes on the current device; fails with
+ * CSA_ERR_HIP if the device has no room (nothing stays allocated then).
  * key_words: 64-bit words of the generation-0 key, 1 to 4 (4 to 16 uint16 symbols; the reference's
  * PREF_KEY_WORDS, include/Packed_Prefix.hpp:20-24, whose default is 4). The suffix array does not depend on it,
- * only the number of generations and their sizes do; every width costs the same time (wide keys are resolved by
- * doubling steps on one-word keys, which are reported as generation 0).
+ * only the number of generations and their sizes do; for csa_sort_partition_u16_dev every width costs the same time
+ * (wide keys are resolved by doubling steps on one-word keys, which are reported as generation 0).
  * Replaces GPU_SACA::allocate_device_space (src/GPU_SACA.cu:535-590). */
 int csa_create(uint64_t max_part_sz, int key_words, csa_handle** out);
+
+/* The same for a host pipeline that drives partitions through the per-generation steps only, one handle per
+ * dispatcher thread (STREAM_C of them, include/GPU_SACA.hpp:90-91): the block is csa_step_bytes_per_suffix(key_words)
+ * per suffix and csa_sort_partition_u16_dev refuses the handle. Every other entry point works on it. */
+int csa_create_steps(uint64_t max_part_sz, int key_words, csa_handle** out);
+
+/* Bytes of the block that the last call on this handle held at its busiest moment (0 for the resident sort, whose
+ * carve-up is fixed). For tests and for sizing; the reference prints its device-memory high-water mark the same way
+ * (include/utility.cuh:68-131). */
+uint64_t csa_scratch_high_water(const csa_handle* h);
 
 /* Declares whether calls on this handle have the device to themselves (exclusive != 0): no other handle, stream or
  * process launches work on it while such a call runs. Only then may the radix passes number their tiles by
@@ -100,7 +131,8 @@ int csa_set_device_exclusive(csa_handle* h, int exclusive);
  *                                0xFFFFFFFF: never)
  *   CSA_TUNE_XCD_CHUNK           tiles (of 8192 pairs) that one XCD takes in a row under csa_set_device_exclusive
  *                                (default 16; 0: the exclusive order is the default order); call before
- *                                csa_set_device_exclusive
+ *                                csa_set_device_exclusive. 8 chunks of that many workgroups must be resident
+ *                                together with room to spare: values above compute units / 16 fail with CSA_ERR_ARG
  * No counterpart in the reference. */
 enum { CSA_TUNE_DEFER_MIN = 0, CSA_TUNE_WINDOW_MIN_CHANGED = 1, CSA_TUNE_XCD_CHUNK = 2 };
 int csa_set_tuning(csa_handle* h, int knob, uint32_t value);
@@ -124,7 +156,7 @@ int csa_sort_partition_u16_dev(csa_handle* h, const uint16_t* d_text, uint64_t n
 int csa_sort_partition_u16(const uint16_t* h_text, uint64_t n, int key_words, uint8_t* h_sa40, csa_stats* stats);
 
 /* The same for `count` independent partitions in host memory, pipelined: one handle sized for the largest of them, two
- * sets of device buffers, three streams. While partition k is sorted, the text of partition k + 1 is uploaded and the
+ * sets of device buffers, four streams (one up, one for the sort, two down). While partition k is sorted, the text of partition k + 1 is uploaded and the
  * suffix array of partition k - 1 is downloaded (an upload thread and a download thread beside the calling one), which is
  * how the reference's three dispatcher threads overlap transfers and device work (src/GPU_SACA.cu:1539-1589).
  * h_texts[k]: n[k] symbols; h_sa40[k]: room for 5 * n[k] bytes; index_base (may be NULL = all zero): the suffix index of
@@ -154,7 +186,8 @@ int csa_radix_sort_pairs_dev(csa_handle* h, uint64_t* d_keys, uint32_t* d_vals, 
  * ends: 8 * CSA_STATIC_SORT_MAX_PAIRS + 4 * CSA_STATIC_SORT_MAX_PAIRS bytes of pairs + 2.3 MB of control words, 14.3 MB
  * in all. n > CSA_STATIC_SORT_MAX_PAIRS fails with CSA_ERR_TOO_LARGE. All calls on one device share that one array:
  * calls that overlap on a device (two streams, two threads) race; serialise them. Every pass of the bit range runs
- * (passes over a constant digit are not skipped: that needs the counts on the host). The stream's device must be the
+ * (passes over a constant digit are not skipped: that needs the counts on the host). A failure on the device is not
+ * reported by this call: ask csa_radix_sort_pairs_static_status afterwards. The stream's device must be the
  * current one. The first call on a device looks the array's address up (hipGetSymbolAddress); make that call, with
  * n = 0 if need be, before any stream capture begins.
  * No counterpart in the reference (its sorts go through cub's workspace, allocated once by allocate_device_space). */
@@ -162,6 +195,13 @@ int csa_radix_sort_pairs_dev(csa_handle* h, uint64_t* d_keys, uint32_t* d_vals, 
 #define CSA_STATIC_SORT_MAX_PAIRS (1u << 20)
 #endif
 int csa_radix_sort_pairs_static_dev(uint64_t* d_keys, uint32_t* d_vals, uint64_t n, int begin_bit, int end_bit, void* stream);
+
+/* csa_radix_sort_pairs_static_dev cannot report a failure on the device (it returns before its kernels run): a
+ * look-back wait that runs into its spin limit makes the remaining workgroups leave, and the pairs are then not sorted.
+ * This call waits for the stream and returns CSA_ERR_INTERNAL if the last such sort on the current device ended that
+ * way, CSA_OK otherwise. It copies one word to the host and allocates nothing; not for use inside a stream capture
+ * (ask after the graph's launch has finished). No counterpart in the reference. */
+int csa_radix_sort_pairs_static_status(void* stream);
 
 /* O(n) suffix-array check on the device: d_sa40 is a permutation of [index_base, index_base + n) and every
  * adjacent pair is in order (first symbols, then ranks of the successors; a successor past the end sorts
@@ -248,7 +288,19 @@ int csa_join_messages_sorted_dev(csa_handle* h, const uint8_t* d_msg_target, con
 typedef struct csa_step_result {
     uint64_t active;   /* size of the partition's new active set: entries [0, active) of the outputs */
     uint64_t messages; /* messages in the outbox */
+    /* Generations t >= 1, counted on the device in every call (the reference counts and checks them under -DTESTS,
+     * include/GPU_SACA.cuh:234-249, src/GPU_SACA.cu:2055-2068): */
+    uint64_t unserved; /* cohort members that no message joined: they sorted with an all-ones secondary. The exchange
+                          scheme guarantees 0; the reference aborts otherwise ("Active suffixes with no message received") */
+    uint64_t pills;    /* cohort members that a poison pill joined (their source's rank is final) */
+    uint64_t incoherent_pills; /* neighbours of the sorted cohort with equal (primary, secondary) of which only one carries
+                                  a pill receipt (test::validate_coherent_pill_receipts, test/tests.hpp:106-111; the
+                                  reference traps). 0 in a coherent exchange */
 } csa_step_result;
+
+/* The counters of the last csa_sort_init_* / csa_sort_rerank_* call on the handle (the slab-shaped entries return
+ * them this way). */
+int csa_last_step_result(const csa_handle* h, csa_step_result* out);
 
 /* Generation 0 of one partition of m suffixes (m <= the handle's capacity), everything resident in HBM:
  *   in : d_keys[i * key_words + w] packed K-gram words (key_words 1 to 4), d_suf40 5-byte lanes, d_beta routing-tag pairs (forward tag in
@@ -258,7 +310,8 @@ typedef struct csa_step_result {
  *        the outbox: 5-byte targets, ranks (MSB = the sender retired), d_msg_off[q] = exclusive END of the group bound
  *        for partition q (p + 1 counters); ctx = 4 * key_words symbols were resolved.
  * The outbox needs room for m messages. The call returns after the stream has finished; res may be NULL.
- * The handle lends its sort scratch and, from the first call on, two more 8-byte arrays of its capacity.
+ * The step works inside the handle's block and allocates nothing (csa_step_bytes_per_suffix covers it with the
+ * caller's buffers counted in).
  * Replaces GPU_SACA::sort_and_init_rank_and_filter (include/GPU_SACA.hpp:272, src/GPU_SACA.cu:1112-1331) between the
  * upload of the slabs and their download. */
 int csa_sort_init_dev(csa_handle* h, const uint64_t* d_keys, int key_words, const uint8_t* d_suf40, const uint32_t* d_beta,
@@ -272,7 +325,7 @@ int csa_sort_init_dev(csa_handle* h, const uint64_t* d_keys, int key_words, cons
  *   out: as csa_sort_init_dev, ranks refined by (primary, received rank); the outbox needs room for 2 * m messages
  *        (payloads and forwarded pills).
  * A cohort member that received no message sorts with an all-ones secondary, as in the reference (the exchange
- * scheme guarantees there is none).
+ * scheme guarantees there is none; res->unserved counts them).
  * Replaces GPU_SACA::sort_and_re_rank_and_filter (include/GPU_SACA.hpp:279, src/GPU_SACA.cu:1715-1995). */
 int csa_sort_rerank_dev(csa_handle* h, const uint32_t* d_rank, const uint8_t* d_suf40, const uint32_t* d_beta, uint64_t m,
                         const uint8_t* d_inbox_target, const uint32_t* d_inbox_rank, uint32_t inbox_sz, uint64_t ctx,
@@ -303,11 +356,6 @@ typedef struct csa_slab {
     uint32_t outbox_sz;   /* messages [2 * c * chunk_cap, ...) for the c-th slab of the list */
 } csa_slab;
 
-/* Device bytes the slab-shaped entries add to a handle per suffix of its capacity (the device image of the slabs going
- * in and coming out), on top of csa_bytes_per_suffix and the 16 bytes of the step entries. Allocated by the first such
- * call, kept until csa_destroy. */
-uint64_t csa_slab_bytes_per_suffix(int key_words);
-
 /* GPU_SACA::sort_and_init_rank_and_filter(p_id, p_assembly, buf_id) (include/GPU_SACA.hpp:272, src/GPU_SACA.cu:1112-1331)
  * as the dispatcher calls it: uploads key(), suf(), beta() of every slab to the slab's off() (:1125-1133), runs
  * csa_sort_init_dev, then downloads into every slab its share of the ranks (over key()) and lanes, active suffixes
@@ -315,7 +363,8 @@ uint64_t csa_slab_bytes_per_suffix(int key_words);
  * h_msg_off receives the p exclusive END offsets of the destinations' groups (backend_->msg_off(p_id)), *h_active_slot
  * the new active-set size (backend_->active_slot(p_id)); either may be NULL. part_sz = the slabs' sizes summed <= the
  * handle's capacity. The call returns after the stream has finished (the reference's caller synchronises right after,
- * src/GPU_SACA.cu:1582). */
+ * src/GPU_SACA.cu:1582); when it returns an error, nothing is still being copied into the slabs or h_msg_off either.
+ * The device image of the slabs lives in the handle's block: no memory is allocated. */
 int csa_sort_init_slabs(csa_handle* h, csa_slab* slabs, uint32_t slab_c, uint64_t part_sz, int key_words, uint32_t p,
                         uint64_t chunk_cap, uint32_t* h_msg_off, uint64_t* h_active_slot, void* stream);
 

@@ -1,25 +1,40 @@
-// slab_pipeline <n> <p> <key_words> <chunk_cap> <seed> <sigma> [suffix-array-file]
+// slab_pipeline <n> <p> <key_words> <chunk_cap> <seed> <sigma> [suffix-array-file|-] [threads] [text-file|-] [budget-bytes]
 // A multi-partition suffix-array build driven the way the reference's dispatcher drives its builder class
 // (src/GPU_SACA.cu:1354-1600, 2190-2370), through the three per-partition members of include/cascade_gpu_saca.hpp:
 // every partition step takes a Partition_Assembly of pinned host slabs (chunks of chunk_cap suffixes, each with its chunk
 // of the partition's inbox) and returns ranks, lanes and the outbox in them; partitions exchange ranks only as messages;
 // the final permutation comes back cut for the output file. Everything that the reference's backend keeps (partition
 // contents, inboxes, the packed partition-id map with its retirement flags) is plain host memory here.
+//   threads      dispatcher threads (1 to 3 = STREAM_C), each with its own buffer set and stream, that take the
+//                partitions of a generation from a shared counter and call the members concurrently
+//                (src/GPU_SACA.cu:1539-1589); default 1
+//   text-file    uint16 symbols to build the suffix array of (n = its length; sigma is ignored) instead of the built-in
+//                random text with a planted repeat
+//   budget-bytes device memory the builder may plan with: the partitions must not exceed partition_size_upper_bound of
+//                it, allocate_device_space must take no more than its share, and no step may allocate beyond that
+//                (checked with hipMemGetInfo). With n = 0 the text length is that bound itself (use p = 1: one partition
+//                of exactly the largest size the floor plan admits)
 // The result is compared, byte for byte, with the suffix array of the same text sorted as one resident partition
-// (csa_sort_partition_u16); exit status 0 if they agree. A test program: it is not part of the library.
+// (csa_sort_partition_u16); exit status 0 if they agree. The last line also reports what the dispatch phases took and
+// moved over the link (host staging and message routing between the phases are not in those times).
+// A test program: it is not part of the library.
 #include "../../include/cascade_gpu_saca.hpp"
 
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
 #include <array>
+#include <atomic>
+#include <chrono>
 #include <cstring>
 #include <memory>
 #include <random>
+#include <thread>
 
 namespace {
 
 using namespace cascade_hip;
+using Builder = GPU_SACA<std::uint16_t>;
 
 [[noreturn]] void die(const std::string& what)
 {
@@ -51,6 +66,13 @@ template <typename T> T* pinned_alloc(std::size_t count)
     T* p = nullptr;
     hip_check(hipHostMalloc(reinterpret_cast<void**>(&p), (count ? count : 1) * sizeof(T), hipHostMallocDefault), "hipHostMalloc");
     return p;
+}
+
+std::size_t device_free_bytes()
+{
+    std::size_t free_b = 0, total_b = 0;
+    hip_check(hipMemGetInfo(&free_b, &total_b), "hipMemGetInfo");
+    return free_b;
 }
 
 void put_lane(std::uint8_t* lanes, std::size_t i, std::uint64_t v)
@@ -85,6 +107,14 @@ struct Partition {
     std::vector<std::uint64_t> suf; // its suffixes, active ones first
     std::vector<p_sz_t> rank;       // their partition-local ranks
     idx_t active = 0;
+    std::vector<std::unique_ptr<Slab_Buffers>> slabs; // the partition's own slabs, kept over the generations
+    Partition_Assembly assembly;                      // the chain handed to the members in this phase
+    Staging_Slab& slab_of(std::size_t c, idx_t chunk_cap, int key_words)
+    {
+        while (slabs.size() <= c)
+            slabs.push_back(std::make_unique<Slab_Buffers>(chunk_cap, key_words));
+        return slabs[c]->slab;
+    }
 };
 
 struct Inbox {
@@ -92,30 +122,74 @@ struct Inbox {
     std::vector<p_sz_t> rank;
 };
 
+// Runs job(q, buf_id) for every listed partition on `threads` dispatcher threads, buffer set = thread index; returns
+// the seconds the phase took.
+template <typename Job> double dispatch(const std::vector<std::uint32_t>& todo, unsigned threads, Job job)
+{
+    const auto t0 = std::chrono::steady_clock::now();
+    if (threads <= 1) {
+        for (const std::uint32_t q : todo)
+            job(q, 0);
+    } else {
+        std::atomic<std::size_t> next{0};
+        std::vector<std::thread> pool;
+        for (unsigned b = 0; b < threads; ++b)
+            pool.emplace_back([&, b] {
+                for (std::size_t i = next.fetch_add(1); i < todo.size(); i = next.fetch_add(1))
+                    job(todo[i], b);
+            });
+        for (auto& t : pool)
+            t.join();
+    }
+    return std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+}
+
 } // namespace
 
 int main(int argc, char** argv)
 {
     if (argc < 7)
-        die("usage: slab_pipeline <n> <p> <key_words> <chunk_cap> <seed> <sigma> [suffix-array-file]");
-    const idx_t n = std::strtoull(argv[1], nullptr, 10);
+        die("usage: slab_pipeline <n> <p> <key_words> <chunk_cap> <seed> <sigma> [suffix-array-file|-] [threads] [text-file|-] [budget-bytes]");
+    idx_t n = std::strtoull(argv[1], nullptr, 10);
     const std::uint32_t p = static_cast<std::uint32_t>(std::strtoul(argv[2], nullptr, 10));
     const int key_words = std::atoi(argv[3]);
     const idx_t chunk_cap = std::strtoull(argv[4], nullptr, 10);
     const std::uint64_t seed = std::strtoull(argv[5], nullptr, 10);
     const std::uint32_t sigma = static_cast<std::uint32_t>(std::strtoul(argv[6], nullptr, 10));
-    if (n < 16 || p < 1 || p > 32768 || key_words < 1 || key_words > 4 || chunk_cap % 4096 != 0 || chunk_cap == 0 || sigma < 1)
+    const std::string sa_path = argc > 7 && std::string(argv[7]) != "-" ? argv[7] : "";
+    const unsigned threads = argc > 8 ? static_cast<unsigned>(std::atoi(argv[8])) : 1u;
+    const std::string text_path = argc > 9 && std::string(argv[9]) != "-" ? argv[9] : "";
+    const std::size_t budget = argc > 10 ? std::strtoull(argv[10], nullptr, 10) : 0;
+    if (p < 1 || p > 32768 || key_words < 1 || key_words > 4 || chunk_cap % 4096 != 0 || chunk_cap == 0 || sigma < 1 || threads < 1 ||
+        threads > Builder::STREAM_C)
         die("bad arguments");
     const idx_t ell = 4 * static_cast<idx_t>(key_words);
+    if (budget && n == 0) // one partition of exactly the size the floor plan admits for this budget
+        n = Builder(1, static_cast<p_id_t>(p), key_words, chunk_cap).partition_size_upper_bound(budget);
 
-    // ---- the text: random symbols, a long repeat (many generations, pills in flight), a zero tail ----
+    // ---- the text: a file, or random symbols with a long repeat (many generations, pills in flight) and a zero tail ----
     std::mt19937_64 rng(seed);
-    std::vector<std::uint16_t> text(n);
-    for (auto& s : text)
-        s = static_cast<std::uint16_t>(rng() % sigma);
-    std::copy(text.begin(), text.begin() + n / 3, text.begin() + n / 2);
-    for (idx_t i = n - 9; i < n; ++i)
-        text[i] = 0;
+    std::vector<std::uint16_t> text;
+    if (!text_path.empty()) {
+        std::ifstream in(text_path, std::ios::binary | std::ios::ate);
+        if (!in)
+            die("cannot open " + text_path);
+        n = static_cast<idx_t>(in.tellg()) / 2;
+        text.resize(n);
+        in.seekg(0);
+        in.read(reinterpret_cast<char*>(text.data()), static_cast<std::streamsize>(2 * n));
+    } else {
+        if (n < 16)
+            die("bad arguments: n < 16");
+        text.resize(n);
+        for (auto& s : text)
+            s = static_cast<std::uint16_t>(rng() % sigma);
+        std::copy(text.begin(), text.begin() + n / 3, text.begin() + n / 2);
+        for (idx_t i = n - 9; i < n; ++i)
+            text[i] = 0;
+    }
+    if (n < 16)
+        die("the text is shorter than 16 symbols");
     std::uint16_t* d_text = dev_alloc<std::uint16_t>(n);
     hip_check(hipMemcpy(d_text, text.data(), n * 2, hipMemcpyHostToDevice), "text upload");
 
@@ -155,6 +229,9 @@ int main(int argc, char** argv)
     hip_check(hipMemcpy(pid.data(), d_pid, n * 2, hipMemcpyDeviceToHost), "pid download");
     hip_check(hipMemcpy(map.data(), d_map, map_words * 8, hipMemcpyDeviceToHost), "map download");
     hip_check(hipMemcpy(psz.data(), d_psz, p * 8, hipMemcpyDeviceToHost), "sizes download");
+    hip_check(hipFree(d_pid), "free");
+    hip_check(hipFree(d_piv), "free");
+    hip_check(hipFree(d_psz), "free");
     std::vector<idx_t> P_off(p + 1, 0);
     idx_t max_part = 1;
     for (std::uint32_t q = 0; q < p; ++q) {
@@ -165,9 +242,8 @@ int main(int argc, char** argv)
         die("the partition sizes do not add up to n");
 
     std::vector<Partition> part(p);
-    for (std::uint32_t q = 0; q < p; ++q) {
+    for (std::uint32_t q = 0; q < p; ++q)
         part[q].suf.reserve(psz[q]);
-    }
     for (idx_t j = 0; j < n; ++j)
         part[pid[j]].suf.push_back(j);
     for (std::uint32_t q = 0; q < p; ++q) {
@@ -175,17 +251,6 @@ int main(int argc, char** argv)
         part[q].rank.assign(part[q].suf.size(), 0);
         part[q].active = part[q].suf.size();
     }
-
-    // ---- the builder and its slabs ----
-    GPU_SACA<std::uint16_t> saca(max_part, static_cast<p_id_t>(p), key_words, chunk_cap);
-    if (!saca.allocate_device_space())
-        die("no device space");
-    std::vector<std::unique_ptr<Slab_Buffers>> pool;
-    auto slab_of = [&](std::size_t c) -> Staging_Slab& {
-        while (pool.size() <= c)
-            pool.push_back(std::make_unique<Slab_Buffers>(chunk_cap, key_words));
-        return pool[c]->slab;
-    };
     std::uint8_t* d_lanes = dev_alloc<std::uint8_t>(5 * max_part);
     std::uint64_t* d_keys = dev_alloc<std::uint64_t>(max_part * key_words);
     std::uint32_t* d_beta = dev_alloc<std::uint32_t>(max_part);
@@ -193,26 +258,53 @@ int main(int argc, char** argv)
     std::vector<std::uint64_t> keys(max_part * key_words);
     std::vector<std::uint32_t> beta(max_part);
 
+    // ---- the builder: sized by its own bound when a budget is given; everything it will ever hold is allocated here ----
+    Builder saca(max_part, static_cast<p_id_t>(p), key_words, chunk_cap);
+    if (budget && max_part > saca.partition_size_upper_bound(budget))
+        die("the largest partition (" + std::to_string(max_part) + ") exceeds partition_size_upper_bound(" + std::to_string(budget) +
+            ") = " + std::to_string(saca.partition_size_upper_bound(budget)));
+    const std::size_t free_before = device_free_bytes();
+    if (!saca.allocate_device_space())
+        die("no device space");
+    const std::size_t free_after = device_free_bytes();
+    const std::size_t taken = free_before - free_after;
+    if (budget && taken > static_cast<std::size_t>(static_cast<double>(budget) * (1.0 - Builder::MEM_SAFETY_MARGIN)))
+        die("allocate_device_space took " + std::to_string(taken) + " bytes, more than the budget's share");
+    if (taken > saca.device_bytes_required(max_part) + (64u << 20))
+        die("allocate_device_space took " + std::to_string(taken) + " bytes, the floor plan says " +
+            std::to_string(saca.device_bytes_required(max_part)));
+    hipStream_t streams[Builder::STREAM_C] = {};
+    for (unsigned b = 0; b < threads; ++b) {
+        hip_check(hipStreamCreateWithFlags(&streams[b], hipStreamNonBlocking), "stream");
+        saca.set_stream(b, streams[b]);
+    }
+    // No step may take device memory of its own. The level is read after the streams exist (the runtime keeps a few MB
+    // per stream), and what the runtime sets up on a stream's first use is allowed for below; a column of a partition
+    // would be far more.
+    const std::size_t free_ready = device_free_bytes();
+    std::size_t free_lowest = free_ready;
+
+    double dispatch_s = 0, gen0_s = 0;
+    std::uint64_t link_bytes = 0, gen0_bytes = 0;
     std::vector<Inbox> inbox(p);
     idx_t gen = 0, ctx = ell;
     for (;; ++gen, ctx *= 2) {
-        bool any = false;
-        for (const auto& pt : part)
-            any = any || pt.active > 0;
-        if (!any)
+        std::vector<std::uint32_t> todo;
+        for (std::uint32_t q = 0; q < p; ++q)
+            if (part[q].active > 0)
+                todo.push_back(q);
+        if (todo.empty())
             break;
         if (gen >= 64)
             die("64 generations and still active suffixes");
         saca.set_context(ctx, gen);
         hip_check(hipMemcpy(d_map, map.data(), map_words * 8, hipMemcpyHostToDevice), "map upload");
-        std::vector<Inbox> next(p);
-        std::vector<std::uint64_t> retired_now;
-        for (std::uint32_t q = 0; q < p; ++q) {
+        // ---- phase 1, host (the reference's readers and stagers, src/GPU_SACA.cu:1412-1500, 1611-1692): every
+        //      partition and its inbox cut into chunks of chunk_cap (:1396-1400), keys at generation 0, routing tags ----
+        std::uint64_t bytes_up = 0;
+        for (const std::uint32_t q : todo) {
             Partition& pt = part[q];
             const idx_t a = pt.active;
-            if (a == 0)
-                continue;
-            // staging (src/GPU_SACA.cu:1611-1692): keys at generation 0, routing tags always
             for (idx_t i = 0; i < a; ++i)
                 put_lane(lanes.data(), i, pt.suf[i]);
             hip_check(hipMemcpy(d_lanes, lanes.data(), 5 * a, hipMemcpyHostToDevice), "lane upload");
@@ -223,13 +315,12 @@ int main(int argc, char** argv)
             hip_check(hipMemcpy(beta.data(), d_beta, a * 4, hipMemcpyDeviceToHost), "beta download");
             if (gen == 0)
                 hip_check(hipMemcpy(keys.data(), d_keys, a * key_words * 8, hipMemcpyDeviceToHost), "key download");
-            // the partition and its inbox, cut into chunks of chunk_cap (src/GPU_SACA.cu:1396-1400)
             const Inbox& in = inbox[q];
             const idx_t inbox_sz = gen == 0 ? 0 : in.target.size();
             const std::size_t chunk_c = std::max<std::size_t>(1, std::max((a + chunk_cap - 1) / chunk_cap, (inbox_sz + chunk_cap - 1) / chunk_cap));
-            Partition_Assembly pa;
+            pt.assembly.slab.clear();
             for (std::size_t c = 0; c < chunk_c; ++c) {
-                Staging_Slab& s = slab_of(c);
+                Staging_Slab& s = pt.slab_of(c, chunk_cap, key_words);
                 const idx_t off = c * chunk_cap;
                 const idx_t sz = off < a ? std::min(chunk_cap, a - off) : 0;
                 const idx_t msg_sz = off < inbox_sz ? std::min(chunk_cap, inbox_sz - off) : 0;
@@ -244,13 +335,26 @@ int main(int argc, char** argv)
                     put_lane(s.msg_target(), i, in.target[off + i]);
                 if (msg_sz)
                     std::memcpy(s.msg_rank(), in.rank.data() + off, msg_sz * 4);
-                pa.slab.push_back(&s);
+                pt.assembly.slab.push_back(&s);
             }
+            bytes_up += a * (gen == 0 ? 8 * key_words + 9 : 13) + inbox_sz * 9;
+        }
+        // ---- phase 2, the dispatchers (src/GPU_SACA.cu:1539-1589): the members, concurrently, one buffer set each ----
+        const double secs = dispatch(todo, threads, [&](std::uint32_t q, unsigned buf_id) {
             if (gen == 0)
-                saca.sort_and_init_rank_and_filter(static_cast<p_id_t>(q), pa, q % GPU_SACA<std::uint16_t>::STREAM_C);
+                saca.sort_and_init_rank_and_filter(static_cast<p_id_t>(q), part[q].assembly, buf_id);
             else
-                saca.sort_and_re_rank_and_filter(static_cast<p_id_t>(q), pa, q % GPU_SACA<std::uint16_t>::STREAM_C);
-            // what the backend takes back (src/GPU_SACA.cu:1305-1331): ranks over key(), lanes, the outbox by destination
+                saca.sort_and_re_rank_and_filter(static_cast<p_id_t>(q), part[q].assembly, buf_id);
+        });
+        free_lowest = std::min(free_lowest, device_free_bytes());
+        // ---- phase 3, host (the reference's writers, src/GPU_SACA.cu:1305-1331, 1503-1530, 1695-1711): ranks over
+        //      key(), lanes, the outbox split by destination, retirement flags ----
+        std::vector<Inbox> next(p);
+        std::vector<std::uint64_t> retired_now;
+        std::uint64_t bytes_down = 0;
+        for (const std::uint32_t q : todo) {
+            Partition& pt = part[q];
+            const idx_t a = pt.active;
             const idx_t a_new = *saca.active_slot(static_cast<p_id_t>(q));
             const p_sz_t* end = saca.msg_off(static_cast<p_id_t>(q));
             const idx_t total = end[p - 1];
@@ -258,8 +362,8 @@ int main(int argc, char** argv)
                 die("more active suffixes after a step than before");
             std::vector<std::uint64_t> m_target(total);
             std::vector<p_sz_t> m_rank(total);
-            for (std::size_t c = 0; c < chunk_c; ++c) {
-                const Staging_Slab& s = *pa.slab[c];
+            for (std::size_t c = 0; c < pt.assembly.slab.size(); ++c) {
+                const Staging_Slab& s = *pt.assembly.slab[c];
                 for (idx_t i = 0; i < s.size(); ++i) {
                     pt.suf[s.off() + i] = get_lane(s.suf(), i);
                     pt.rank[s.off() + i] = reinterpret_cast<const p_sz_t*>(s.key())[i];
@@ -285,56 +389,75 @@ int main(int argc, char** argv)
             for (idx_t i = a_new; i < a; ++i)
                 retired_now.push_back(pt.suf[i]);
             pt.active = a_new;
+            bytes_down += a * 9 + total * 9;
         }
-        // retirement flags of this generation's retirees (GPU_SACA::destage_slab, src/GPU_SACA.cu:1695-1711)
         for (const std::uint64_t j : retired_now) {
             const std::uint64_t bit = j * bits + (bits - 1);
             map[bit / 64] |= std::uint64_t(1) << (bit % 64);
         }
         inbox.swap(next);
+        dispatch_s += secs;
+        link_bytes += bytes_up + bytes_down;
+        if (gen == 0) {
+            gen0_s = secs;
+            gen0_bytes = bytes_up + bytes_down;
+        }
     }
 
-    // ---- every partition to rank order, as cut for the output file (src/GPU_SACA.cu:2107-2164) ----
+    // ---- every partition to rank order, as cut for the output file (src/GPU_SACA.cu:2107-2164, 2337-2365) ----
     std::vector<std::uint8_t> file(5 * n, 0xEE);
+    std::vector<std::uint32_t> todo;
     for (std::uint32_t q = 0; q < p; ++q) {
-        const Partition& pt = part[q];
+        Partition& pt = part[q];
         const idx_t m = pt.suf.size();
         if (m == 0)
             continue;
+        todo.push_back(q);
         const std::size_t chunk_c = (m + chunk_cap - 1) / chunk_cap + 1; // one more: the partition need not start on a disk block
-        Partition_Assembly pa;
+        pt.assembly.slab.clear();
         for (std::size_t c = 0; c < chunk_c; ++c) {
-            Staging_Slab& s = slab_of(c);
+            Staging_Slab& s = pt.slab_of(c, chunk_cap, key_words);
             const idx_t off = c * chunk_cap;
             const idx_t sz = off < m ? std::min(chunk_cap, m - off) : 0;
             s.assign(sz ? off : m, sz, 0, 0);
             for (idx_t i = 0; i < sz; ++i)
                 put_lane(s.suf(), i, pt.suf[off + i]);
             std::memcpy(s.key(), pt.rank.data() + off, sz * 4);
-            pa.slab.push_back(&s);
+            pt.assembly.slab.push_back(&s);
         }
-        const idx_t lo = 5 * P_off[q];
-        saca.scatter_to_rank_order(static_cast<p_id_t>(q), pa, q % GPU_SACA<std::uint16_t>::STREAM_C, lo);
+    }
+    const double scatter_s = dispatch(todo, threads, [&](std::uint32_t q, unsigned buf_id) {
+        saca.scatter_to_rank_order(static_cast<p_id_t>(q), part[q].assembly, buf_id, 5 * P_off[q]);
+    });
+    free_lowest = std::min(free_lowest, device_free_bytes());
+    for (const std::uint32_t q : todo) {
+        const Partition& pt = part[q];
+        const idx_t m = pt.suf.size(), lo = 5 * P_off[q];
+        const std::size_t chunk_c = pt.assembly.slab.size();
         for (std::size_t c = 0; c < chunk_c; ++c) {
             std::uint64_t cut[6];
             csa_output_cut(lo, lo + 5 * m, 5 * chunk_cap, static_cast<std::uint32_t>(c), static_cast<std::uint32_t>(chunk_c), cut);
-            const Staging_Slab& s = *pa.slab[c];
+            const Staging_Slab& s = *pt.assembly.slab[c];
             std::memcpy(file.data() + cut[0], s.suf(), cut[1] - cut[0]);
             std::memcpy(file.data() + cut[2], s.msg_target(), cut[3] - cut[2]);
             std::memcpy(file.data() + cut[4], s.msg_target() + 4096, cut[5] - cut[4]);
         }
     }
+    if (free_lowest + (32u << 20) < free_ready)
+        die("a step took device memory of its own: " + std::to_string(free_ready - free_lowest) + " bytes below the level after allocate_device_space");
 
+    if (!sa_path.empty()) {
+        std::ofstream out(sa_path, std::ios::binary | std::ios::trunc);
+        out.write(reinterpret_cast<const char*>(file.data()), static_cast<std::streamsize>(file.size()));
+        if (text_path.empty()) {
+            std::ofstream txt(sa_path + ".text", std::ios::binary | std::ios::trunc);
+            txt.write(reinterpret_cast<const char*>(text.data()), static_cast<std::streamsize>(2 * n));
+        }
+    }
     // ---- the same text as one resident partition ----
     std::vector<std::uint8_t> want(5 * n);
     csa_stats st{};
     csa_check(csa_sort_partition_u16(text.data(), n, key_words, want.data(), &st), "resident sort");
-    if (argc > 7) {
-        std::ofstream out(argv[7], std::ios::binary | std::ios::trunc);
-        out.write(reinterpret_cast<const char*>(file.data()), static_cast<std::streamsize>(file.size()));
-        std::ofstream txt(std::string(argv[7]) + ".text", std::ios::binary | std::ios::trunc);
-        txt.write(reinterpret_cast<const char*>(text.data()), static_cast<std::streamsize>(2 * n));
-    }
     if (file != want) {
         idx_t at = 0;
         while (at < 5 * n && file[at] == want[at])
@@ -343,6 +466,8 @@ int main(int argc, char** argv)
         return 1;
     }
     std::cout << "OK n=" << n << " p=" << p << " key_words=" << key_words << " generations=" << gen << " (resident sort: " << st.generations
-              << ")\n";
+              << ") threads=" << threads << " max_part=" << max_part << " device_bytes=" << taken << " gen0_ms=" << gen0_s * 1e3
+              << " gen0_link_bytes=" << gen0_bytes << " dispatch_ms=" << dispatch_s * 1e3 << " link_bytes=" << link_bytes
+              << " scatter_ms=" << scatter_s * 1e3 << " scatter_link_bytes=" << 14 * n << "\n";
     return 0;
 }

@@ -228,7 +228,14 @@ inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
 template <typename T>
 inline hipError_t hipGetSymbolAddress(void** p, T& symbol) { *p = &symbol; return hipSuccess; }
 enum hipDeviceAttribute_t { hipDeviceAttributeMultiprocessorCount = 63 };
-inline hipError_t hipDeviceGetAttribute(int* v, hipDeviceAttribute_t, int) { *v = 1; return hipSuccess; } // one "CU"
+// one "CU", unless a test has the device claim more (HIPEMU_CU_COUNT): workgroups still run one at a time, which makes it
+// the extreme case of a device shared with other launches
+inline hipError_t hipDeviceGetAttribute(int* v, hipDeviceAttribute_t, int)
+{
+    const char* claimed = std::getenv("HIPEMU_CU_COUNT");
+    *v = claimed ? std::atoi(claimed) : 1;
+    return hipSuccess;
+}
 inline hipError_t hipMalloc(void** p, size_t bytes)
 {
     *p = std::malloc(bytes ? bytes : 1);

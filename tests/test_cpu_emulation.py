@@ -40,7 +40,24 @@ def emu():
     lib.csa_sort_init_slabs.argtypes = [vp, C.POINTER(_native.CsaSlab), u32, u64, i32, u32, u64, vp, vp, vp]
     lib.csa_sort_rerank_slabs.argtypes = [vp, C.POINTER(_native.CsaSlab), u32, u64, u64, u64, u32, u64, vp, vp, vp]
     lib.csa_scatter_slabs.argtypes = [vp, C.POINTER(_native.CsaSlab), u32, u64, u64, u64, vp]
+    lib.csa_create_steps.argtypes = [u64, i32, C.POINTER(vp)]
+    lib.csa_step_bytes_per_suffix.restype = u64
+    lib.csa_step_bytes_per_suffix.argtypes = [i32]
+    lib.csa_workspace_bytes.restype = u64
+    lib.csa_workspace_bytes.argtypes = [u64]
+    lib.csa_scratch_high_water.restype = u64
+    lib.csa_scratch_high_water.argtypes = [vp]
+    lib.csa_last_step_result.argtypes = [vp, C.POINTER(_native.CsaStepResult)]
     return lib
+
+
+def steps_handle(lib, key_words):
+    """For multi_partition.build_sa: a handle of exactly the largest partition's capacity, made for the steps."""
+    def make(max_part_sz):
+        h = C.c_void_p()
+        assert lib.csa_create_steps(max_part_sz, key_words, C.byref(h)) == 0, lib.csa_last_error()
+        return h
+    return make
 
 
 def emu_sort(lib, T, key_words):
@@ -291,14 +308,9 @@ def test_multi_partition_pipeline_with_the_emulated_step_entries(emu, p, key_wor
     if key_words == 1:  # long repeats: many generations, pills forwarded
         T[250:450] = T[:200]
         T[500:650] = T[100:250]
-    h = C.c_void_p()
-    assert emu.csa_create(n, 1, C.byref(h)) == 0
     log, glue_log = [], []
-    try:
-        sa, gens = multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, p, key_words=key_words,
-                                            log=log, step_handle=h)
-    finally:
-        emu.csa_destroy(h)
+    sa, gens = multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, p, key_words=key_words,
+                                        log=log, step_handle=steps_handle(emu, key_words))
     assert np.array_equal(sa, oracle_lib.sa40_to_u64(oracle_lib.build_sa40(T))), (p, key_words, gens)
     # the same run with numpy glue between the stages: the same cohorts, survivors and message counts at every step
     multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, p, key_words=key_words, log=glue_log)
@@ -314,16 +326,53 @@ def test_multi_partition_pipeline_through_the_emulated_slab_entries(emu, p, key_
     T = texts.random_text(n, sigma, 31 * p + n, sep_every=0)
     T[n // 3:n // 3 + 250] = T[:250]
     T[-5:] = 0
-    h = C.c_void_p()
-    assert emu.csa_create(n, 1, C.byref(h)) == 0
-    try:
-        # slabs far smaller than the reference's: a partition of a few thousand suffixes still spans several
-        sa, gens = multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, p, key_words=key_words,
-                                            slab_handle=h, host_buf=lambda nbytes: np.zeros(nbytes, dtype=np.uint8), chunk_cap=chunk_cap)
-    finally:
-        emu.csa_destroy(h)
+    # slabs far smaller than the reference's: a partition of a few thousand suffixes still spans several
+    sa, gens = multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, p, key_words=key_words,
+                                        slab_handle=steps_handle(emu, key_words), host_buf=lambda nbytes: np.zeros(nbytes, dtype=np.uint8),
+                                        chunk_cap=chunk_cap)
     want, _ = oracle_lib.prefix_doubling(T, key_words)
     assert np.array_equal(sa, want) and gens >= 5
+
+
+@pytest.mark.parametrize("key_words,p,slabs", [(1, 1, True), (2, 1, True), (3, 2, False), (4, 1, True)])
+def test_the_steps_stay_inside_the_floor_plan(emu, key_words, p, slabs):
+    """A handle made by csa_create_steps for exactly the largest partition holds csa_step_bytes_per_suffix(key_words)
+    bytes per suffix and nothing more is ever allocated: every step of a whole build, slab traffic included, must find
+    its columns in that block (a step that does not returns an error naming the column). Texts with long ties on the
+    first key word, so that the wide-key path sorts nearly every suffix a second time (its busiest moment). The
+    reference's own floor plan is 65 / 65 / 81 / 97 bytes per suffix (src/GPU_SACA.cu:372)."""
+    import multi_partition
+    per_suffix = int(emu.csa_step_bytes_per_suffix(key_words))
+    assert per_suffix == {1: 48, 2: 65, 3: 76, 4: 84}[key_words]
+    assert per_suffix <= 2 * (max(8 * key_words, 16) + 8 + 4 + 4) + 1  # the reference's own figure
+    for n, sigma in ((420, 2),):
+        T = texts.random_text(n, sigma, 5 * n + key_words, sep_every=0)
+        kw = {"slab_handle": steps_handle(emu, key_words), "host_buf": lambda nbytes: np.zeros(nbytes, dtype=np.uint8),
+              "chunk_cap": 4096} if slabs else {"step_handle": steps_handle(emu, key_words)}
+        sa, gens = multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, p, key_words=key_words, **kw)
+        want, _ = oracle_lib.prefix_doubling(T, key_words)
+        assert np.array_equal(sa, want), (n, sigma, gens)
+        if slabs and p == 1:
+            # the busiest step held no more than the documented figure (the partition's size is rounded up to 256 suffixes)
+            assert multi_partition.build_sa.high_water <= per_suffix * (n + 255), (multi_partition.build_sa.high_water, per_suffix * n)
+
+
+def test_sizing_by_the_mirrors_bound_never_exceeds_the_device(emu):
+    """What include/cascade_gpu_saca.hpp's partition_size_upper_bound computes (restated here): STREAM_C handles of the
+    bound's size, workspaces included, fit into the free memory with the reference's margins."""
+    STREAM_C, MARGIN, SLACK = 3, 0.1, 1.20
+    for key_words in (1, 2, 3, 4):
+        per_suffix = int(emu.csa_step_bytes_per_suffix(key_words))
+        for free in (1 << 24, 5 << 30, 96 << 30, 288 << 30):
+            budget = int(free * (1.0 - MARGIN) / SLACK)
+            sz = min(budget // (STREAM_C * per_suffix), _native.CSA_MAX_PART_SZ)
+            while sz > 0 and STREAM_C * (sz * per_suffix + int(emu.csa_workspace_bytes(sz))) > budget:
+                ws = STREAM_C * int(emu.csa_workspace_bytes(sz))
+                nxt = 0 if ws >= budget else (budget - ws) // (STREAM_C * per_suffix)
+                sz = nxt if nxt < sz else sz - 1
+            assert STREAM_C * (sz * per_suffix + int(emu.csa_workspace_bytes(sz))) <= budget < free
+            if free >= 5 << 30:
+                assert sz > 0.8 * budget / (STREAM_C * per_suffix)  # the workspace is a small share
 
 
 def test_step_entries_on_a_text_of_one_symbol(emu):
@@ -331,12 +380,7 @@ def test_step_entries_on_a_text_of_one_symbol(emu):
     one partition are empty. Closed form: the shorter suffix comes first."""
     import multi_partition
     T = np.full(100, 9, dtype=np.uint16)
-    h = C.c_void_p()
-    assert emu.csa_create(T.size, 1, C.byref(h)) == 0
-    try:
-        sa, gens = multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, 3, step_handle=h)
-    finally:
-        emu.csa_destroy(h)
+    sa, gens = multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, 3, step_handle=steps_handle(emu, 1))
     assert np.array_equal(sa, np.arange(T.size - 1, -1, -1, dtype=np.uint64)), gens
 
 
@@ -350,12 +394,21 @@ def test_chunked_tile_order_without_resident_workgroups_ends_in_an_error_not_a_h
     T = texts.random_text(140000, 5, 3, sep_every=0)  # 137 tiles of 1024 keys: one whole group of 8 chunks of 16
     n = T.size
     h = C.c_void_p()
-    assert emu.csa_create(n, 1, C.byref(h)) == 0
+    # the emulated device has one compute unit: the chunked order is neither offered nor accepted as a tuning value
+    assert emu.csa_create(16, 1, C.byref(h)) == 0
+    assert emu.csa_set_tuning(h, _native.CSA_TUNE_XCD_CHUNK, 16) == _native.CSA_ERR_ARG and b"compute units" in emu.csa_last_error()
+    emu.csa_destroy(h)
+    # a device that claims 256 compute units while its workgroups still run one at a time
+    os.environ["HIPEMU_CU_COUNT"] = "256"
+    try:
+        assert emu.csa_create(n, 1, C.byref(h)) == 0
+    finally:
+        del os.environ["HIPEMU_CU_COUNT"]
     out = np.zeros(5 * n + 8, dtype=np.uint8)
     st = _native.CsaStats()
     try:
-        # (the emulated device has too few compute units for the chunked order to be offered by itself)
         assert emu.csa_set_tuning(h, _native.CSA_TUNE_XCD_CHUNK, 16) == 0
+        assert emu.csa_set_tuning(h, _native.CSA_TUNE_XCD_CHUNK, 17) == _native.CSA_ERR_ARG  # 2 * 8 * 17 > 256
         assert emu.csa_set_device_exclusive(h, 1) == 0
         rc = emu.csa_sort_partition_u16_dev(h, T.ctypes.data, n, 0, out.ctypes.data, None, 0, C.byref(st))
         assert rc == -4 and b"spin limit" in emu.csa_last_error(), (rc, emu.csa_last_error())

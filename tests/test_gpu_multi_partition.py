@@ -33,6 +33,16 @@ def gpu():
     return _native.load(), to_dev, to_host
 
 
+def steps_handle(lib, key_words):
+    """For multi_partition.build_sa: a handle made for the steps (csa_create_steps) with exactly the largest partition's
+    capacity, the tightest the floor plan admits: a step that needs a byte more than csa_step_bytes_per_suffix fails."""
+    def make(max_part_sz):
+        h = C.c_void_p()
+        assert lib.csa_create_steps(max_part_sz, key_words, C.byref(h)) == 0, lib.csa_last_error()
+        return h
+    return make
+
+
 @pytest.mark.parametrize("p,key_words,sorted_join,steps", [(3, 1, False, False), (16, 1, True, False), (33, 2, False, False),
                                                            (3, 1, False, True), (16, 2, False, True), (40, 1, False, True),
                                                            (9, 3, False, True), (16, 4, False, True), (5, 4, False, False)])
@@ -50,7 +60,8 @@ def test_partitions_that_only_exchange_messages_build_the_oracles_suffix_array(g
     try:
         print(f"  multi-partition n={n} p={p} key_words={key_words} steps={steps}", flush=True)
         sa, gens = multi_partition.build_sa(lib, to_dev, to_host, T, p, key_words=key_words, log=log,
-                                            join_handle=h if sorted_join else None, step_handle=h if steps else None)
+                                            join_handle=h if sorted_join else None,
+                                            step_handle=steps_handle(lib, key_words) if steps else None)
     finally:
         lib.csa_destroy(h)
     want, _ = oracle_lib.prefix_doubling(T, key_words)
@@ -76,14 +87,12 @@ def test_slab_shaped_entries_from_pinned_host_slabs_build_the_oracles_suffix_arr
     T[30000:70000] = T[:40000]
     T[-9:] = 0
     log = []
-    h = C.c_void_p()
-    assert lib.csa_create(n, 1, C.byref(h)) == 0
-    try:
-        print(f"  slab entries n={n} p={p} key_words={key_words} chunk_cap={chunk_cap}", flush=True)
-        sa, gens = multi_partition.build_sa(lib, to_dev, to_host, T, p, key_words=key_words, log=log, slab_handle=h,
-                                            host_buf=pinned_host_buf, chunk_cap=chunk_cap)
-    finally:
-        lib.csa_destroy(h)
+    print(f"  slab entries n={n} p={p} key_words={key_words} chunk_cap={chunk_cap}", flush=True)
+    sa, gens = multi_partition.build_sa(lib, to_dev, to_host, T, p, key_words=key_words, log=log, slab_handle=steps_handle(lib, key_words),
+                                        host_buf=pinned_host_buf, chunk_cap=chunk_cap)
+    per_suffix = int(lib.csa_step_bytes_per_suffix(key_words))
+    assert per_suffix == {1: 48, 2: 65, 3: 76, 4: 84}[key_words]
+    assert multi_partition.build_sa.high_water <= per_suffix * (n + 255)  # (the partition's size is rounded up to 256 suffixes)
     want, _ = oracle_lib.prefix_doubling(T, key_words)
     assert np.array_equal(sa, want)
     assert gens >= 10 and (p == 1 or sum(step[5] for step in log if step[0] >= 1) > 0)
@@ -99,14 +108,10 @@ def test_slab_shaped_entries_report_what_the_device_entries_report(gpu):
     logs = []
     for mode in ("dev", "slabs"):
         log = []
-        h = C.c_void_p()
-        assert lib.csa_create(n, 1, C.byref(h)) == 0
-        try:
-            print(f"  {mode} entries n={n} p={p}", flush=True)
-            kw = {"step_handle": h} if mode == "dev" else {"slab_handle": h, "host_buf": pinned_host_buf, "chunk_cap": 8192}
-            sa, _ = multi_partition.build_sa(lib, to_dev, to_host, T, p, log=log, seed=5, **kw)
-        finally:
-            lib.csa_destroy(h)
+        print(f"  {mode} entries n={n} p={p}", flush=True)
+        make = steps_handle(lib, 1)
+        kw = {"step_handle": make} if mode == "dev" else {"slab_handle": make, "host_buf": pinned_host_buf, "chunk_cap": 8192}
+        sa, _ = multi_partition.build_sa(lib, to_dev, to_host, T, p, log=log, seed=5, **kw)
         assert np.array_equal(sa, oracle_lib.prefix_doubling(T, 1)[0])
         logs.append(log)
     assert logs[0] == logs[1]
@@ -162,13 +167,8 @@ def test_step_entries_on_hard_shapes(gpu, shape, p):
     lib, to_dev, to_host = gpu
     T = _shape(shape)
     n = T.size
-    h = C.c_void_p()
-    assert lib.csa_create(n, 1, C.byref(h)) == 0
-    try:
-        print(f"  step entries on {shape}: n={n} p={p}", flush=True)
-        sa, gens = multi_partition.build_sa(lib, to_dev, to_host, T, p, step_handle=h)
-    finally:
-        lib.csa_destroy(h)
+    print(f"  step entries on {shape}: n={n} p={p}", flush=True)
+    sa, gens = multi_partition.build_sa(lib, to_dev, to_host, T, p, step_handle=steps_handle(lib, 1))
     want, _ = oracle_lib.prefix_doubling(T, 1)
     assert np.array_equal(sa, want), (shape, gens)
     if shape == "one_symbol":
@@ -191,12 +191,10 @@ def test_random_pipelines_through_the_step_entries(gpu):
             T[-int(rng.integers(1, 30)):] = 0
         p = int(rng.choice([1, 2, 3, 7, 16, 50, 200]))
         key_words = 1 + case % 4
-        h = C.c_void_p()
-        assert lib.csa_create(n, 1, C.byref(h)) == 0
-        try:
-            print(f"  random pipeline case={case} n={n} sigma={sigma} p={p} key_words={key_words}", flush=True)
-            sa, _ = multi_partition.build_sa(lib, to_dev, to_host, T, p, key_words=key_words, seed=case, step_handle=h)
-        finally:
-            lib.csa_destroy(h)
+        print(f"  random pipeline case={case} n={n} sigma={sigma} p={p} key_words={key_words}", flush=True)
+        # half of the cases through the slab-shaped entries; the handle is sized exactly for the largest partition
+        kw = {"step_handle": steps_handle(lib, key_words)} if (case // 4) % 2 == 0 else {
+            "slab_handle": steps_handle(lib, key_words), "host_buf": pinned_host_buf, "chunk_cap": 4096}
+        sa, _ = multi_partition.build_sa(lib, to_dev, to_host, T, p, key_words=key_words, seed=case, **kw)
         want, _ = oracle_lib.prefix_doubling(T, 1)
         assert np.array_equal(sa, want), (case, n, sigma, p, key_words)

@@ -38,6 +38,7 @@ def test_sort_without_allocation_equals_the_sort_with_a_handle():
             _native.check(lib.csa_radix_sort_pairs_static_dev(k1.data_ptr(), v1.data_ptr(), n, b, e, stream or None))
             torch.cuda.synchronize()
             assert torch.cuda.mem_get_info()[0] == free_before  # nothing was allocated on the device
+            assert lib.csa_radix_sort_pairs_static_status(stream or None) == 0, lib.csa_last_error()
             assert torch.equal(k1, k0) and torch.equal(v1, v0), (n, b, e)
             if n <= 300001:
                 wk, wv = oracle_lib.stable_sort_pairs(keys, vals, b, e)
@@ -47,3 +48,39 @@ def test_sort_without_allocation_equals_the_sort_with_a_handle():
     v = torch.zeros(limit + 1, dtype=torch.int32, device="cuda")
     rc = lib.csa_radix_sort_pairs_static_dev(k.data_ptr(), v.data_ptr(), limit + 1, 0, 64, None)
     assert rc == _native.CSA_ERR_TOO_LARGE and b"exceed" in lib.csa_last_error()
+
+
+def test_sort_without_allocation_recorded_into_a_graph_and_replayed():
+    """The callers this entry point is for include code recorded into a HIP graph: the call only enqueues kernels (its
+    control words are cleared by a fill kernel, not a memset node), so a captured call can be replayed on new data in the
+    same buffers. Replays alternate with eager work and synchronisations of the program's own; every replay is compared with
+    the handle's sort of the same pairs."""
+    import torch
+    from cascade_amd import PartitionSorter, _native
+    lib = _native.load()
+    rng = np.random.default_rng(5)
+    n = 200000
+    # the first call on a device looks the scratch address up: before any capture
+    _native.check(lib.csa_radix_sort_pairs_static_dev(None, None, 0, 0, 64, None))
+    keys = torch.zeros(n, dtype=torch.int64, device="cuda")
+    vals = torch.zeros(n, dtype=torch.int32, device="cuda")
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            _native.check(lib.csa_radix_sort_pairs_static_dev(keys.data_ptr(), vals.data_ptr(), n, 0, 40, side.cuda_stream))
+    torch.cuda.synchronize()
+    with PartitionSorter(n) as s:
+        for replay in range(4):
+            hk = rng.integers(0, 1 << 40, n, dtype=np.uint64)
+            hv = rng.permutation(n).astype(np.uint32)
+            print(f"  graph replay {replay}", flush=True)
+            keys.copy_(_dev(torch, hk))
+            vals.copy_(_dev(torch, hv))
+            want_k, want_v = keys.clone(), vals.clone()
+            s.radix_sort_pairs(want_k, want_v, 0, 40)  # eager work between the replays
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert lib.csa_radix_sort_pairs_static_status(None) == 0, lib.csa_last_error()
+            assert torch.equal(keys, want_k) and torch.equal(vals, want_v), replay
