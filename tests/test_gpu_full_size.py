@@ -52,10 +52,11 @@ def test_full_size_configuration_sorts_to_a_verified_suffix_array(config, exclus
         s.close()
 
 
-@pytest.mark.timeout(300)
+@pytest.mark.timeout(600)
 def test_largest_partition_at_the_largest_index_base():
     """n = 2^31 - 1 suffixes (MAX_PART_SZ, include/bit-layout.hpp:63-68) ending at suffix index 2^40 - 1, the last
-    one a 5-byte entry can hold (include/sa40.hpp:72-75): uniform random symbols, generated on the device."""
+    one a 5-byte entry can hold (include/sa40.hpp:72-75): uniform random symbols, generated on the device. The suffix array
+    from index 0 goes through the oracle's verifier on the host; the one at the largest base must be that array shifted."""
     import torch
     from cascade_amd import PartitionSorter
     n = (1 << 31) - 1
@@ -66,7 +67,24 @@ def test_largest_partition_at_the_largest_index_base():
     d_text = torch.randint(-32768, 32768, (n,), dtype=torch.int16, device="cuda", generator=g)
     s = PartitionSorter(n, key_words=1)
     try:
+        # the same partition from index 0 is judged by the CPU oracle's O(n) verifier (the reference's rule,
+        # test/end-to-end.cpp:46-80; about 23 bytes of host memory per suffix, 49 GB here)
+        import oracle_lib
+        out0 = s.sort(d_text)
+        print("  oracle verifier on the host", flush=True)
+        assert oracle_lib.is_correct_sa40(out0.cpu().numpy(), d_text.cpu().numpy().view(np.uint16))
         out = s.sort(d_text, index_base=base)
+        # ... and at the largest base every entry is the verified one plus the base (compared in pieces of 2^26 entries)
+
+        def entries(lanes):
+            e = lanes[:, 0].to(torch.int64)
+            for k in range(1, 5):
+                e |= lanes[:, k].to(torch.int64) << (8 * k)
+            return e
+        for lo in range(0, n, 1 << 26):
+            hi = min(n, lo + (1 << 26))
+            assert bool((entries(out.view(n, 5)[lo:hi]) == entries(out0.view(n, 5)[lo:hi]) + base).all()), lo
+        del out0
         assert s.last_stats["n"] == n and s.last_stats["generations"] >= 1
         assert s.verify(d_text, out, index_base=base)
         assert not s.verify(d_text, out, index_base=base - 1)
