@@ -605,7 +605,7 @@ def main():
         # as a share of the HBM peak. It is NOT a roofline fraction: generations whose groups are sorted inside LDS move far
         # fewer bytes than the yardstick charges and come out above 1. frac_moved is the roofline fraction: bytes the
         # counters saw this generation move (from the committed profile of this workload) over this run's time.
-        row = {"g": g, "active": st["active"][g], "groups": st["groups"][g], "big": st["big"][g], "passes": st["passes"][g],
+        row = {"g": g, "active": st["active"][g], "groups": st["groups"][g], "big": st["big"][g], "presorted": st["presorted"][g], "passes": st["passes"][g],
                "rank_update": st["rank_update"][g], "small_only": st["small_only"][g], "dense": st["dense"][g], "ms": round(st["ms"][g], 3),
                "alg_GBps": round(gbs, 1), "alg_over_peak": round(gbs / HBM_PEAK_GBS, 4)}
         if g in moved_gen and st["ms"][g] > 0:

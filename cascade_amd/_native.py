@@ -61,6 +61,7 @@ class CsaStats(C.Structure):
         ("radix_launches", C.c_uint64),
         ("radix_pairs", C.c_uint64),
         ("radix_ms", C.c_double),
+        ("presorted", C.c_uint64 * CSA_MAX_GENERATIONS),
     ]
 
 

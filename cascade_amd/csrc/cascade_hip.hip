@@ -387,10 +387,15 @@ void launch_onesweep_shape(const TileOrder& o, OnesweepArgs& a, hipStream_t s)
         hipLaunchKernelGGL((onesweep_kernel<u64, BLOCK, SORT_ITEMS, SRC, 0, VALS>), dim3(a.tiles), dim3(BLOCK), 0, s, a);
 }
 
+// the first pass of generation 0 (keys built from the text) may take the other shape
+#ifndef CSA_TEXT_WIDE
+#define CSA_TEXT_WIDE 1
+#endif
+
 template <int SRC, bool VALS = true>
 void launch_onesweep(const csa_handle* h, OnesweepArgs& a, hipStream_t s)
 {
-    if (wide_workgroups(a))
+    if (wide_workgroups(a) && (SRC != SRC_TEXT || CSA_TEXT_WIDE))
         launch_onesweep_shape<SRC, SORT_WIDE_BLOCK, VALS>(tile_order_of(h), a, s);
     else
         launch_onesweep_shape<SRC, SORT_BLOCK, VALS>(tile_order_of(h), a, s);
@@ -988,7 +993,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
         sa.nr_out = nr_list;
         sa.big_keys = bkey[0];
         sa.big_sufs = bx[0];
-        sa.big_count = h->counts + 4;
+        sa.big_first = reinterpret_cast<const u32*>(bkey[1]); // (free until the radix sort, which starts after the kernel that reads it)
         sa.tile_agg = r.tile_agg;
         sa.tile_splits = r.tile_splits;
         passes = 0;
@@ -1006,21 +1011,78 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
             HIP_TRY(hipGetLastError());
             st->small_only[gen] = 1;
         } else {
-            HIP_TRY(hipMemsetAsync(h->counts + 4, 0, sizeof(u32), s));
+            HIP_TRY(hipMemsetAsync(h->counts + 4, 0, 2 * sizeof(u32), s));
+            // marks of the large groups whose gathered ranks are out of order, in the tables the next generation's groups
+            // will be written to (free until the apply step)
+            sa.big_sec = bx[1];
+            sa.not_asc = h->gprim[gp ^ 1];
+            sa.not_desc = h->gstart[gp ^ 1];
             high_limit = (u64)m_in <= (u64)groups * SMALL_AVG_LIMIT;
+            const u32 maxg = high_limit ? (u32)SMALL_MAXG_HI : (u32)SMALL_MAXG;
+            const u32 marks = m_in / maxg + 2u; // one mark index per large group at most
+            HIP_TRY(hipMemsetAsync(sa.not_asc, 0, (u64)marks * sizeof(u32), s));
+            HIP_TRY(hipMemsetAsync(sa.not_desc, 0, (u64)marks * sizeof(u32), s));
+            {
+                // where every large group's members start in the list of large-group members, and how many there are
+                // (counts[4]): a prefix sum over the group table
+                u32* big_first = reinterpret_cast<u32*>(bkey[1]);
+                const RankTables gr = rank_tables(h, groups, 1024);
+                hipLaunchKernelGGL((big_prefix_kernel<false>), dim3(gr.tiles), dim3(256), 0, s, (const u32*)h->gstart[gp], groups, maxg, big_first,
+                                   gr.tile_agg, gr.tile_splits, (const u32*)gr.tile_prefix, (const u32*)gr.slab_total, gr.slab, gr.slabs,
+                                   h->counts + 4);
+                hipLaunchKernelGGL(rerank_scan_kernel, dim3(gr.slabs), dim3(1024), 0, s, gr.tile_agg, gr.tile_prefix, gr.tiles, gr.slab,
+                                   gr.slab_total, gr.tile_splits);
+                hipLaunchKernelGGL((big_prefix_kernel<true>), dim3(gr.tiles), dim3(256), 0, s, (const u32*)h->gstart[gp], groups, maxg, big_first,
+                                   gr.tile_agg, gr.tile_splits, (const u32*)gr.tile_prefix, (const u32*)gr.slab_total, gr.slab, gr.slabs,
+                                   h->counts + 4);
+            }
             if (high_limit)
                 hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG_HI, false>), dim3(r.tiles), dim3(SMALL_BLOCK), 0,
                                    s, sa);
             else
                 hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG, false>), dim3(r.tiles), dim3(SMALL_BLOCK), 0, s,
                                    sa);
+            hipLaunchKernelGGL(group_order_kernel, dim3((marks + 255u) / 256u), dim3(256), 0, s, (const u32*)sa.not_asc, (const u32*)sa.not_desc,
+                               marks, h->counts + 5);
             HIP_TRY(hipGetLastError());
             rc = read_counts(L, &big);
             if (rc)
                 return rc;
             all_small = big == 0;
+            const u32 unordered = h->h_pinned[5];
+            if (big > 0 && unordered == 0) {
+                // 2a. every large group is in order as it stands (runs of one token, periodic stretches: the gathered ranks
+                //     rise or fall along the list): no sort, the members are ranked by their runs of equal gathered ranks
+                PresortedArgs pa;
+                pa.sufs = ax;
+                pa.gids = agid;
+                pa.big_sec = sa.big_sec;
+                pa.gstart = h->gstart[gp];
+                pa.gprim = h->gprim[gp];
+                pa.big_first = sa.big_first;
+                pa.not_asc = sa.not_asc;
+                pa.m = m_in;
+                pa.n = n;
+                pa.groups = groups;
+                pa.maxg = maxg;
+                pa.sufs_out = x_out;
+                pa.nr_out = nr_list;
+                pa.err = h->counts + 2;
+                const RankTables pr = rank_tables(h, m_in, RANK_TILE);
+                pa.tile_agg = pr.tile_agg;
+                pa.tile_splits = pr.tile_splits;
+                pa.tile_prefix = pr.tile_prefix;
+                pa.slab_total = pr.slab_total;
+                pa.slab = pr.slab;
+                hipLaunchKernelGGL((place_presorted_kernel<RANK_BLOCK, RANK_ITEMS, false>), dim3(pr.tiles), dim3(RANK_BLOCK), 0, s, pa);
+                hipLaunchKernelGGL(rerank_scan_kernel, dim3(pr.slabs), dim3(1024), 0, s, pr.tile_agg, pr.tile_prefix, pr.tiles, pr.slab,
+                                   pr.slab_total, pr.tile_splits);
+                hipLaunchKernelGGL((place_presorted_kernel<RANK_BLOCK, RANK_ITEMS, true>), dim3(pr.tiles), dim3(RANK_BLOCK), 0, s, pa);
+                HIP_TRY(hipGetLastError());
+                st->presorted[gen] = big;
+            }
             // 2. the large groups: radix sort on (group id, rank[x + h]), then back into the list as (suffix, refined rank)
-            if (big > 0) {
+            if (big > 0 && unordered != 0) {
                 const int gid_bits = bit_length(groups > 1 ? groups - 1 : 0);
                 const PassPlan plan = make_plan(0, sec_bits + gid_bits);
                 rc = radix_sort(L, SRC_PAIRS, nullptr, n, 0, 0, bkey[0], bx[0], bkey[1], bx[1], big, plan, &in_out, &passes);
@@ -1127,6 +1189,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
             st->active[g] = st->active[g + merged];
             st->groups[g] = st->groups[g + merged];
             st->big[g] = st->big[g + merged];
+            st->presorted[g] = st->presorted[g + merged];
             st->passes[g] = st->passes[g + merged];
             st->rank_update[g] = st->rank_update[g + merged];
             st->small_only[g] = st->small_only[g + merged];
@@ -1134,7 +1197,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
             st->ms[g] = st->ms[g + merged];
         }
         for (int g = gen - merged; g < gen; ++g) {
-            st->active[g] = st->groups[g] = st->big[g] = 0;
+            st->active[g] = st->groups[g] = st->big[g] = st->presorted[g] = 0;
             st->passes[g] = st->rank_update[g] = st->small_only[g] = st->dense[g] = 0;
             st->ms[g] = 0.0f;
         }

@@ -512,8 +512,10 @@ __global__ __launch_bounds__(256) void scatter_ranks_kernel(const u32* __restric
 //                                     (reference: include/GPU_SACA.cuh:277, new = old + key-run head - group head);
 // and writes (suffix, refined rank) to its place of the sorted list. Equal refined ranks are equal keys: a group owns
 // the rank range [gprim, gprim + size), so ranks of different groups cannot meet. No key is written at all.
-// Members of larger groups are appended, in no particular order, to a list of (key, suffix) pairs that goes through
-// the radix sort instead (place_big_kernel brings them back in the same (suffix, refined rank) form).
+// Members of larger groups go, in list order, to a list of (key, suffix) pairs that goes through the radix sort
+// instead (place_big_kernel brings them back in the same (suffix, refined rank) form). List order matters: the sort
+// is stable, so members that tie keep the order they had, here as in the small groups; a list whose large groups are
+// in order of rank[x + h] already (place_presorted_kernel) stays recognisable as such generation after generation.
 // Replaces, for small groups, the 62-bit key sort of the reference (src/GPU_SACA.cu:1841-1871).
 //
 // COUNT instantiation (lists known to hold small groups only): the kernel also adds, to the tile of the sorted list
@@ -533,11 +535,19 @@ struct SmallSortArgs {
     u32* err; // set to a DEV_ERR_* code if an invariant of the group tables is violated
     u32* sufs_out; // sorted active list: suffix ...
     u32* nr_out;   // ... and its refined rank, bit 31 set if it differs from the old rank
-    u64* big_keys; // elements of groups larger than MAXG: (group id << sec_bits) | rank[x + h]
-    u32* big_sufs;
-    u32* big_count; // zero before the launch
+    u64* big_keys; // elements of groups larger than MAXG: (group id << sec_bits) | rank[x + h], in list order:
+    u32* big_sufs; // the member at list place e of large group g goes to big_first[g] + (e - gstart[g])
+    const u32* big_first; // [groups]: members of large groups before group g (big_prefix_kernel)
     u32* tile_agg;    // COUNT: [tiles][4], zero before the launch: [2] survivors, [3] new groups per tile of the sorted list
     u32* tile_splits; // COUNT: [tiles], zero before the launch: changed ranks
+    // !COUNT: is the list already in order inside its large groups? The gathered rank of every member of a large group
+    // is kept at its list place in big_sec, and a large group in which some member's gathered rank is below (above) its
+    // predecessor's gets its size written to not_asc (not_desc) at the group's mark index, big_first[g] / MAXG: a large
+    // group has more than MAXG members, so no two share an index, and m / MAXG + 2 entries cover every list. Both zero
+    // before the launch.
+    u32* big_sec;
+    u32* not_asc;
+    u32* not_desc;
 };
 
 template <int BLOCK, int ITEMS, int MAXG, bool COUNT>
@@ -567,12 +577,20 @@ __global__ __launch_bounds__(BLOCK) void smallsort_kernel(SmallSortArgs a)
     }
     // A halo element matters only if its group reaches into the tile, i.e. if it shares the group of the tile's
     // first (left halo) or last (right halo) element; the others would be random reads for nothing.
+    // A member of a large group needs no other member's rank, except the one before it in the list (is the group in
+    // order already?): of a large group at the tile's border only that one element of the halo is read.
     const long long last_own = t0 + TILE - 1 < (long long)a.m - 1 ? t0 + TILE - 1 : (long long)a.m - 1;
     const u32 gid_first = a.gids[t0], gid_last = a.gids[last_own];
+    bool first_small = true, last_small = true;
+    if (gid_first < a.groups && gid_last < a.groups) { // (checked again, and reported, below)
+        first_small = a.gstart[gid_first + 1] - a.gstart[gid_first] <= (u32)MAXG;
+        last_small = a.gstart[gid_last + 1] - a.gstart[gid_last] <= (u32)MAXG;
+    }
     for (int i = t; i < 2 * MAXG; i += BLOCK) {
         const int slot = i < MAXG ? i : TILE + i; // [0, MAXG) and [MAXG + TILE, SPAN)
         const long long e = lo + slot;
-        if (e >= 0 && e < (long long)a.m && a.gids[e] == (i < MAXG ? gid_first : gid_last)) {
+        const bool wanted = i < MAXG ? (first_small || (!COUNT && i == MAXG - 1)) : last_small;
+        if (wanted && e >= 0 && e < (long long)a.m && a.gids[e] == (i < MAXG ? gid_first : gid_last)) {
             const u64 src = (u64)a.sufs[e] + a.h;
             s_sec[slot] = src < a.n ? a.rank[src] : 0u;
         }
@@ -584,7 +602,6 @@ __global__ __launch_bounds__(BLOCK) void smallsort_kernel(SmallSortArgs a)
     // when most of the list is in large groups)
     u32 g[ITEMS], gs[ITEMS], ge[ITEMS];
     u32 kind = 0; // 2 bits per item: 0 = not mine, 1 = small group, 2 = large group
-    u32 n_big = 0;
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         const long long e = t0 + k * BLOCK + t;
@@ -601,33 +618,12 @@ __global__ __launch_bounds__(BLOCK) void smallsort_kernel(SmallSortArgs a)
                 atomicExch(a.err, DEV_ERR_SMALLSORT_TABLES); // the element is not inside its group's range
             } else if (ge[k] - gs[k] > (u32)MAXG) {
                 kind |= 2u << (2 * k);
-                n_big++;
             } else {
                 kind |= 1u << (2 * k);
             }
         }
     }
-    const u32 lane = t & 63u, w = t >> 6;
-    u32 slot = 0;
-    if constexpr (!COUNT) {
-        __shared__ u32 s_wbig[BLOCK / WAVE];
-        __shared__ u32 s_bigbase;
-        const u32 incl = wave_incl_sum(n_big);
-        if (lane == 63u)
-            s_wbig[w] = incl;
-        __syncthreads();
-        slot = incl - n_big; // exclusive prefix inside the block
-        u32 block_big = 0;
-        for (u32 ww = 0; ww < BLOCK / WAVE; ++ww) {
-            if (ww < w)
-                slot += s_wbig[ww];
-            block_big += s_wbig[ww];
-        }
-        if (t == 0)
-            s_bigbase = block_big ? atomicAdd(a.big_count, block_big) : 0u;
-        __syncthreads();
-        slot += s_bigbase;
-    }
+    const u32 lane = t & 63u;
 
     // COUNT: survivors, new groups, changed ranks bound for the own tile (registers) or, for a group that straddles
     // a tile border, for the tile before / after (LDS)
@@ -649,9 +645,20 @@ __global__ __launch_bounds__(BLOCK) void smallsort_kernel(SmallSortArgs a)
             if constexpr (COUNT) {
                 atomicExch(a.err, DEV_ERR_UNEXPECTED_LARGE_GROUP); // groups only split: cannot happen after an all-small list
             } else {
+                const u32 first = a.big_first[g[k]];
+                const u32 slot = first + ((u32)e - gs[k]);
                 a.big_keys[slot] = ((u64)g[k] << a.sec_bits) | (u64)sec[k];
                 a.big_sufs[slot] = x[k];
-                slot++;
+                a.big_sec[e] = sec[k];
+                if (e > (long long)gs[k]) { // the member before it in the list belongs to the same group
+                    const u32 before = s_sec[MAXG + (e - 1 - t0)]; // an own element, or the last one of the left halo
+                    const u32 mark = first / (u32)MAXG;
+                    // (plain stores of one value by whoever sees it first: no atomics, and soon only cached reads)
+                    if (before > sec[k] && a.not_asc[mark] == 0)
+                        a.not_asc[mark] = ge[k] - gs[k];
+                    if (before < sec[k] && a.not_desc[mark] == 0)
+                        a.not_desc[mark] = ge[k] - gs[k];
+                }
             }
             continue;
         }
@@ -910,6 +917,196 @@ __global__ __launch_bounds__(BLOCK) void apply_small_kernel(ApplySmallArgs a)
             a.gids_out[tile_rc + rc] = tile_rh + rh - 1;
             rc++;
         }
+    }
+}
+
+// big_first[g] = members of groups larger than maxg among the groups before g, the place of g's first member in the list
+// of large-group members; *total = that count over all groups. From the group table alone (4 bytes per group), in the
+// three launches of the rank step: per-tile sums, rerank_scan_kernel, the pass that writes the prefixes.
+template <bool APPLY>
+__global__ __launch_bounds__(256) void big_prefix_kernel(const u32* __restrict__ gstart, u32 groups, u32 maxg, u32* __restrict__ big_first,
+                                                         u32* __restrict__ tile_agg, u32* __restrict__ tile_splits,
+                                                         const u32* __restrict__ tile_prefix, const u32* __restrict__ slab_total, u32 slab,
+                                                         u32 slabs, u32* __restrict__ total)
+{
+    constexpr int ITEMS = 4, TILE = 256 * ITEMS, WAVES = 256 / WAVE;
+    __shared__ u32 s_w[WAVES];
+    const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
+    const u32 tile = blockIdx.x;
+    const u64 base = (u64)tile * TILE + (u64)t * ITEMS;
+    u32 size[ITEMS], mine = 0;
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const u64 g = base + k;
+        size[k] = 0;
+        if (g < groups) {
+            const u32 sz = gstart[g + 1] - gstart[g];
+            size[k] = sz > maxg ? sz : 0u;
+        }
+        mine += size[k];
+    }
+    const u32 incl = wave_incl_sum(mine);
+    if (lane == 63u)
+        s_w[w] = incl;
+    __syncthreads();
+    u32 before = incl - mine, tile_total = 0;
+    for (u32 ww = 0; ww < WAVES; ++ww) {
+        if (ww < w)
+            before += s_w[ww];
+        tile_total += s_w[ww];
+    }
+    if (!APPLY) {
+        if (t == 0) {
+            tile_agg[(u64)tile * 4 + 0] = 0;
+            tile_agg[(u64)tile * 4 + 1] = 0;
+            tile_agg[(u64)tile * 4 + 2] = tile_total;
+            tile_agg[(u64)tile * 4 + 3] = 0;
+            tile_splits[tile] = 0;
+        }
+        return;
+    }
+    before += tile_prefix[(u64)tile * 4 + 2] + slabs_before(slab_total, tile / slab).sum2;
+    const u32 all = slabs_before(slab_total, slabs).sum2;
+    if (tile == 0 && t == 0)
+        *total = all;
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const u64 g = base + k;
+        if (g < groups)
+            big_first[g] = before;
+        before += size[k];
+    }
+}
+
+// Members of large groups whose gathered ranks are out of order: the sizes of the large groups that carry both marks
+// (`marks` entries of the two mark arrays of the small-group kernel). Zero means every large group of the list is in
+// non-decreasing or in non-increasing order of rank[x + h] as it stands, and none of them needs the radix sort.
+__global__ __launch_bounds__(256) void group_order_kernel(const u32* __restrict__ not_asc, const u32* __restrict__ not_desc, u32 marks,
+                                                          u32* __restrict__ unordered)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    u32 mine = (i < marks && not_asc[i] && not_desc[i]) ? not_asc[i] : 0u;
+    mine = wave_reduce_sum(mine);
+    if ((threadIdx.x & 63u) == 0 && mine)
+        atomicAdd(unordered, mine);
+}
+
+// The large groups of a list in which every one of them is in order already (group_order_kernel counted nothing):
+// no sort. Place p of a large group g takes the member at list place p if the group's gathered ranks do not decrease
+// along the list, and the member at the mirrored place gstart[g] + gstart[g + 1] - 1 - p if they do not increase (a
+// token run followed by a smaller symbol: the deeper into the run, the smaller); its refined rank is gprim[g] + (head
+// of its run of equal gathered ranks - gstart[g]), the heads being a running maximum over the places, found in the
+// three launches of the rank step (per-tile maxima, rerank_scan_kernel, apply). Members that tie keep whatever mutual
+// order this leaves them in: they share a rank, and the next generation sorts them by what it gathers.
+// Replaces, for such lists, the sort of the reference's 62-bit keys (src/GPU_SACA.cu:1841-1871).
+struct PresortedArgs {
+    const u32* sufs; // the active list ...
+    const u32* gids; // ... its groups ...
+    const u32* big_sec; // ... and, at the places of large groups, the gathered ranks
+    const u32* gstart;
+    const u32* gprim;
+    const u32* big_first; // members of large groups before each group: big_first[g] / maxg is the group's mark index
+    const u32* not_asc;   // set at the mark index where the group's gathered ranks decrease somewhere (then they never increase)
+    u32 m, n, groups, maxg;
+    u32* sufs_out;
+    u32* nr_out;
+    u32* tile_agg;    // [tiles][4]: [0] last run head of the tile, as place + 1 (0: none)
+    u32* tile_splits; // [tiles]: zeroed for the scan
+    const u32* tile_prefix;
+    const u32* slab_total;
+    u32 slab;
+    u32* err;
+};
+
+template <int BLOCK, int ITEMS, bool APPLY>
+__global__ __launch_bounds__(BLOCK) void place_presorted_kernel(PresortedArgs a)
+{
+    constexpr int TILE = BLOCK * ITEMS;
+    constexpr int WAVES = BLOCK / WAVE;
+    __shared__ u32 s_wagg[WAVES];
+    const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
+    const u32 tile = blockIdx.x;
+    const u64 base = (u64)tile * TILE + (u64)t * ITEMS;
+    u32 g[ITEMS], gs[ITEMS], src[ITEMS], sec[ITEMS];
+    u32 big = 0, heads = 0; // one bit per item
+    u32 lh = 0;             // last run head among this thread's places, as place + 1
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const u64 p = base + k;
+        g[k] = gs[k] = src[k] = sec[k] = 0;
+        if (p >= a.m)
+            continue;
+        g[k] = a.gids[p];
+        if (g[k] >= a.groups) {
+            atomicExch(a.err, DEV_ERR_SMALLSORT_TABLES);
+            continue;
+        }
+        gs[k] = a.gstart[g[k]];
+        const u32 ge = a.gstart[g[k] + 1];
+        if (!(gs[k] <= p && p < ge && ge <= a.m)) {
+            atomicExch(a.err, DEV_ERR_SMALLSORT_TABLES);
+            continue;
+        }
+        if (ge - gs[k] <= a.maxg)
+            continue; // a small group: the small-group kernel has placed it
+        big |= 1u << k;
+        const bool mirrored = a.not_asc[a.big_first[g[k]] / a.maxg] != 0;
+        src[k] = mirrored ? gs[k] + (ge - 1u - (u32)p) : (u32)p;
+        sec[k] = a.big_sec[src[k]];
+        bool head = p == gs[k];
+        if (!head) { // the member at the place before this one, in the same order
+            const u32 before = (k > 0 && (big & (1u << (k - 1))) && g[k - 1] == g[k]) ? sec[k - 1]
+                                                                                     : a.big_sec[mirrored ? src[k] + 1u : src[k] - 1u];
+            head = before != sec[k];
+        }
+        if (head) {
+            heads |= 1u << k;
+            lh = (u32)p + 1u;
+        }
+    }
+    const u32 ih = wave_incl_max(lh);
+    if (lane == 63u)
+        s_wagg[w] = ih;
+    __syncthreads();
+    if (!APPLY) {
+        if (t == 0) {
+            u32 ah = 0;
+            for (int ww = 0; ww < WAVES; ++ww)
+                ah = ah > s_wagg[ww] ? ah : s_wagg[ww];
+            a.tile_agg[(u64)tile * 4 + 0] = ah;
+            a.tile_agg[(u64)tile * 4 + 1] = 0;
+            a.tile_agg[(u64)tile * 4 + 2] = 0;
+            a.tile_agg[(u64)tile * 4 + 3] = 0;
+            a.tile_splits[tile] = 0;
+        }
+        return;
+    }
+    u32 xh = __shfl_up(ih, 1);
+    if (lane == 0)
+        xh = 0;
+    for (u32 ww = 0; ww < w; ++ww)
+        xh = xh > s_wagg[ww] ? xh : s_wagg[ww];
+    u32 pre = a.tile_prefix[(u64)tile * 4 + 0];
+    const SlabPrefix sp = slabs_before(a.slab_total, tile / a.slab);
+    pre = pre > sp.max0 ? pre : sp.max0;
+    u32 head_at = xh > pre ? xh : pre; // place + 1 of the last run head before this thread's places
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const u64 p = base + k;
+        if (p >= a.m || !(big & (1u << k)))
+            continue;
+        if (heads & (1u << k))
+            head_at = (u32)p + 1u;
+        // (a large group opens with a head of its own, so the running maximum never reaches back into another group)
+        const u32 khead = head_at - 1u;
+        const u32 x = a.sufs[src[k]];
+        const u32 nr = a.gprim[g[k]] + (khead - gs[k]);
+        if (head_at == 0 || khead < gs[k] || khead > (u32)p || nr >= a.n || x >= a.n) {
+            atomicExch(a.err, DEV_ERR_PLACE_RANGE);
+            continue;
+        }
+        a.sufs_out[p] = x;
+        a.nr_out[p] = nr | (khead != gs[k] ? 0x80000000u : 0u);
     }
 }
 

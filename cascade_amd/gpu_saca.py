@@ -23,6 +23,7 @@ def stats_to_dict(st):
         "active": [int(st.active[i]) for i in range(g)],
         "groups": [int(st.groups[i]) for i in range(g)],
         "big": [int(st.big[i]) for i in range(g)],
+        "presorted": [int(st.presorted[i]) for i in range(g)],
         "passes": [int(st.passes[i]) for i in range(g)],
         "rank_update": [int(st.rank_update[i]) for i in range(g)],
         "small_only": [int(st.small_only[i]) for i in range(g)],

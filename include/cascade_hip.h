@@ -65,6 +65,9 @@ typedef struct csa_stats {
     uint64_t radix_launches;
     uint64_t radix_pairs; /* (key, index) pairs moved, summed over launches */
     double radix_ms;
+    uint64_t presorted[CSA_MAX_GENERATIONS]; /* of big[g], members that skipped the radix sort: every large group of the
+                                                list was in order of rank[x + h] already (rising or falling along the
+                                                list, as in runs of one token and periodic stretches) */
 } csa_stats;
 
 typedef struct csa_handle csa_handle;

@@ -26,9 +26,27 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), name
 
 
-def test_stats_struct_layout_matches_header():
-    # 8 + 4 + 4 + 3 * 64*8 + 5 * 64*4 + 4 + 4 + 8 + 8 + 8
-    assert C.sizeof(_native.CsaStats) == 8 + 4 + 4 + 512 + 512 + 512 + 256 + 256 + 256 + 256 + 256 + 4 + 4 + 8 + 8 + 8
+def test_struct_layouts_match_the_header(tmp_path):
+    """The ctypes structures have the sizes and field offsets the C compiler gives the header's structs."""
+    import subprocess
+    src = tmp_path / "layout.c"
+    src.write_text('''#include <stddef.h>
+#include <stdio.h>
+#include "cascade_hip.h"
+int main(void) {
+    printf("%zu %zu %zu %zu\\n", sizeof(csa_stats), offsetof(csa_stats, ms), offsetof(csa_stats, radix_ms), offsetof(csa_stats, presorted));
+    printf("%zu %zu\\n", sizeof(csa_step_result), offsetof(csa_step_result, incoherent_pills));
+    printf("%zu %zu %zu\\n", sizeof(csa_slab), offsetof(csa_slab, off), offsetof(csa_slab, outbox_sz));
+    return 0;
+}
+''')
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c11", "-I", os.path.join(ROOT, "include"), "-o", str(exe), str(src)], check=True)
+    lines = subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split("\n")
+    st, sr, sl = _native.CsaStats, _native.CsaStepResult, _native.CsaSlab
+    assert [int(v) for v in lines[0].split()] == [C.sizeof(st), st.ms.offset, st.radix_ms.offset, st.presorted.offset]
+    assert [int(v) for v in lines[1].split()] == [C.sizeof(sr), sr.incoherent_pills.offset]
+    assert [int(v) for v in lines[2].split()] == [C.sizeof(sl), sl.off.offset, sl.outbox_sz.offset]
 
 
 def test_argument_errors_need_no_gpu():

@@ -73,6 +73,7 @@ def emu_sort(lib, T, key_words):
     emu_sort.rank_update = [int(st.rank_update[i]) for i in range(st.generations)]
     emu_sort.small_only = [int(st.small_only[i]) for i in range(st.generations)]
     emu_sort.dense = [int(st.dense[i]) for i in range(st.generations)]
+    emu_sort.presorted = [int(st.presorted[i]) for i in range(st.generations)]
     return out[:5 * n], [int(st.active[i]) for i in range(st.generations)], [int(st.big[i]) for i in range(st.generations)]
 
 
@@ -121,6 +122,25 @@ def test_text_at_every_alignment_inside_an_eight_byte_word(emu, key_words):
             assert (T.ctypes.data % 8) == 2 * off
             got, _, _ = emu_sort(emu, T, key_words)
             assert np.array_equal(got, oracle_lib.build_sa40(np.array(T))), (off, n)
+
+
+@pytest.mark.parametrize("after_run", [2, 9])
+def test_large_groups_that_are_in_order_already_skip_the_sort(emu, after_run):
+    # A run of one token and a periodic stretch: from the second generation on, the gathered ranks of every large group
+    # rise or fall along the list (falling in the run when a smaller symbol follows it, rising when a larger one does),
+    # so the generation ranks them where they stand instead of sorting them. Random text around them keeps small groups
+    # in the same lists; the two-letter stretch gives generation 1 large groups that are out of order, which it sorts.
+    T = np.concatenate([texts.random_text(1300, 2, 21, sep_every=0) + 6, np.full(700, 5, dtype=np.uint16),
+                        np.array([after_run], dtype=np.uint16), np.tile(np.array([3, 1, 4, 1, 5, 9, 2], dtype=np.uint16), 150),
+                        texts.random_text(400, 3, 22, sep_every=0)])
+    got, active, big = emu_sort(emu, T, 1)
+    assert np.array_equal(got, oracle_lib.build_sa40(T))
+    _, counts = oracle_lib.prefix_doubling(T, 1)
+    assert active == counts
+    presorted = emu_sort.presorted
+    assert any(p > 0 for p in presorted), (big, presorted)
+    assert all(p in (0, b) for p, b in zip(presorted, big))        # all of a generation's large groups, or none
+    assert any(b > 0 and p == 0 for p, b in zip(presorted, big))   # and some generation did sort its large groups
 
 
 def test_small_and_large_groups_take_both_paths(emu):
