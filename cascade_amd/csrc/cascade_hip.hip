@@ -417,10 +417,11 @@ void launch_onesweep32(const csa_handle* hh, OnesweepArgs& a, hipStream_t s)
 // (pairs kin/vin, or the text); passes alternate between the (kin, vin) and (kout, vout) sets, the
 // very first one writing to (kout, vout). *result_in_out = 1 if the sorted pairs ended in (kout, vout).
 // Passes whose digit is the same for every pair are skipped (they would be the identity).
-// src = SRC_RANKS: pair i is ((rank_src[i], rank_src[i + hop]), i), i < n, built by the first pass that runs.
+// src = SRC_RANKS: pair i is ((rank_src[i], rank_src[i + hop]), i), i < n, built by the first pass that runs; the two
+// ranks are combined as rank_pair_key says for `radix`.
 int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 word, u64* kin, u32* vin, u64* kout,
                u32* vout, u32 n, const PassPlan& plan, int* result_in_out, int* passes_run, const u32* rank_src = nullptr,
-               u32 hop = 0)
+               u32 hop = 0, u32 radix = 0)
 {
     csa_handle* h = L.h;
     hipStream_t s = L.stream;
@@ -443,11 +444,12 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
         if (src == SRC_RANKS) {
             ha.rank = rank_src;
             ha.hop = hop;
+            ha.radix = radix;
         }
         // the two halves of a (rank[i], rank[i + hop]) key are the same array, one shifted by hop: when the plan takes
         // the same digits from both halves, one histogram of rank[] and one of its first hop entries give them all
         const int half = plan.num_passes / 2;
-        bool mirrored = src == SRC_RANKS && plan.num_passes == 2 * half && half >= 1 && half <= RANK_HIST_PASSES;
+        bool mirrored = src == SRC_RANKS && radix == 0 && plan.num_passes == 2 * half && half >= 1 && half <= RANK_HIST_PASSES;
         for (int p = 0; mirrored && p < half; ++p)
             mirrored = plan.shift[p] + plan.bits[p] <= 32 && plan.shift[half + p] == 32 + plan.shift[p] && plan.bits[half + p] == plan.bits[p];
         if (mirrored) {
@@ -523,6 +525,7 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
         a.err = h->counts + 2;
         a.rank = rank_src;
         a.hop = hop;
+        a.radix = radix;
         int rc = next_ticket(L, &a.ticket);
         if (rc)
             return rc;
@@ -796,6 +799,15 @@ int rank_totals(Launch& L, const RankTables& r, bool gen0, u32 m, u32 n, bool ex
     return CSA_OK;
 }
 
+// A dense generation: most of the partition is still active and its groups are long (a small alphabet, a periodic
+// text), so nearly every member would go through the radix sort anyway; the whole partition is then sorted again by
+// keys read in text order. Decided from the size of the active list and the number of its groups alone, so that the
+// generation before already knows it (and leaves ordinals in rank[], which such a generation sorts in fewer passes).
+bool dense_generation(u32 m, u32 groups, u32 n)
+{
+    return (u64)m * 5 >= (u64)n * 3 && (u64)m > (u64)groups * SMALL_MAXG_HI && (u64)m >= DENSE_MIN;
+}
+
 // Generation 0: ranks the sorted list described by `ra`: counts per tile, scans the counts, reads the totals back, then
 // applies them and brings rank[] up to date, directly from the kernel or through the two-pass bucketed update.
 int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivors, u32* groups, int* rank_update)
@@ -814,6 +826,8 @@ int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivo
     int rc = rank_totals(L, r, true, ra.m, ra.n, false, survivors, groups, rank_update);
     if (rc)
         return rc;
+    // what the list becomes decides what rank[] is to hold: ordinals for a dense generation, ranks otherwise
+    ra.ordinals = dense_generation(*survivors, *groups, ra.n) ? 1u : 0u;
     if (*rank_update != 0)
         ra.rank_recs = buf.recs[0];
     hipLaunchKernelGGL((rerank_kernel<RANK_BLOCK, RANK_ITEMS>), dim3(r.tiles), dim3(RANK_BLOCK), 0, s, ra);
@@ -898,6 +912,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     range_gen0.close();
     if (rc)
         return rc;
+    bool ordinals_in_rank = ra.ordinals != 0; // rank[] holds run ordinals instead of ranks: the coming generation is dense
     st->passes[0] = passes;
     st->active[0] = n;
     st->groups[0] = 0;
@@ -924,18 +939,20 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
         // two coalesced streams instead of one random gather per member; the ranks come out of the same run ranking as
         // in generation 0 and go back to rank[] through the bucketed update instead of scattered writes. Suffixes that had
         // retired are alone with their rank: they sort to the place they hold already and keep their rank.
-        const bool dense = (u64)m_in * 5 >= (u64)n * 3 && (u64)m_in > (u64)groups * SMALL_MAXG_HI && (u64)m_in >= DENSE_MIN;
+        const bool dense = dense_generation(m_in, groups, n);
         if (dense) {
-            PassPlan plan; // the digits of the two ranks of a key: bits [0, sec_bits) and [32, 32 + sec_bits)
-            plan.num_passes = 0;
-            for (int half = 0; half < 2; ++half)
-                for (int b = 0; b < sec_bits; b += RADIX_BITS) {
-                    plan.shift[plan.num_passes] = 32 * half + b;
-                    plan.bits[plan.num_passes] = sec_bits - b < RADIX_BITS ? sec_bits - b : RADIX_BITS;
-                    plan.num_passes++;
-                }
+            // The generation before knew this one would be dense (the same test on the same numbers) and left ordinals in
+            // rank[]: the key runs of its sorted list numbered 0, 1, 2, ...; there are as many as it had groups and
+            // singletons. Two ordinals make a key of 2 log2(runs) bits: 17 bits after generation 0 of a four-letter
+            // text (256 groups and the last four suffixes), three passes where two 31-bit ranks take eight.
+            if (!ordinals_in_rank)
+                return fail(CSA_ERR_INTERNAL, "generation %d is dense but the one before it left ranks, not ordinals", gen);
+            const u64 runs = (u64)groups + ((u64)n - m_in);
+            const u32 radix = (u32)runs;
+            const PassPlan plan = make_plan(0, runs > 1 ? bit_length(runs * runs - 1) : 1);
             passes = 0;
-            rc = radix_sort(L, SRC_RANKS, nullptr, n, 0, 0, bkey[0], bx[0], bkey[1], bx[1], n, plan, &in_out, &passes, h->rank, (u32)hop);
+            rc = radix_sort(L, SRC_RANKS, nullptr, n, 0, 0, bkey[0], bx[0], bkey[1], bx[1], n, plan, &in_out, &passes, h->rank, (u32)hop,
+                            radix);
             if (rc)
                 return rc;
             RerankArgs rd;
@@ -958,6 +975,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
             rc = rerank_step(L, rd, db, &m, &groups, &st->rank_update[gen]);
             if (rc)
                 return rc;
+            ordinals_in_rank = rd.ordinals != 0;
             // the freshly sorted index array is the suffix array under construction from here on; the old one is scratch
             u32* const old_sa32 = sa32;
             sa32 = bx[in_out];
@@ -973,6 +991,8 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
             ctx += hop;
             continue;
         }
+        if (ordinals_in_rank)
+            return fail(CSA_ERR_INTERNAL, "generation %d reads ranks but the one before it left ordinals", gen);
         const RankTables r = rank_tables(h, m_in, SMALL_TILE);
         u32* nr_list = reinterpret_cast<u32*>(key_out); // refined rank at every place of the sorted list
         // 1. gather rank[x + h]; small groups are sorted and ranked inside their tile, members of large groups set aside

@@ -67,6 +67,12 @@ struct RerankArgs {
     // (x << 32) | r at rank_recs[c] (a coalesced stream). The records then go through radix passes on the high bits of
     // x before they are written to rank[], so that those writes fall into one window of rank[] at a time.
     u64* rank_recs; // null: write rank[x] directly
+    // 0: the value kept for suffix x is its rank (index of the head of its key run). 1: it is the run's ordinal, the
+    // number of key runs before it (the ranks renumbered 0, 1, 2, ...): what the next generation wants when it sorts the
+    // whole partition again by pairs of these values read in text order (rank_pair_key with a radix). Counted without
+    // a scan of its own: runs before a place = groups begun before it + singletons before it, and an element that is
+    // not a survivor is a singleton.
+    u32 ordinals;
     u32* sufs_out;  // first active list
     u32* gids_out;
     u32* gprim_out;
@@ -292,10 +298,15 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
                 atomicExch(a.err, DEV_ERR_RERANK_RANGE);
                 continue;
             }
+            // runs before this element's own: (groups begun before its run) + (singletons before its run); for a group
+            // member at place c with S survivors before it, S - (c - head) of them precede the head
+            const u32 begun = tile_rh + rh + ((!single && ka) ? 1u : 0u); // group heads up to and including its own run's
+            const u32 ordinal = (single ? begun : begun - 1u) + ((u32)c - (tile_rc + rc));
+            const u32 value = a.ordinals ? ordinal : nr;
             if (a.rank_recs)
-                rec[k] = ((u64)x << 32) | nr;
+                rec[k] = ((u64)x << 32) | value;
             else
-                a.rank[x] = nr;
+                a.rank[x] = value;
             if (!single) {
                 if (ka) {
                     s_oprim[rh] = nr;

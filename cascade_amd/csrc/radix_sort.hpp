@@ -31,11 +31,15 @@ enum : int {
 };
 
 // Key of text position i in a dense generation: its rank, then the rank of the suffix `hop` symbols on (0 past the
-// end of the text; no tied suffix reaches there).
-__device__ __forceinline__ u64 rank_pair_key(const u32* __restrict__ rank, u32 n, u32 hop, u32 i)
+// end of the text; no tied suffix reaches there). radix = 0: the two ranks side by side in the two halves of the key.
+// radix = D > 0: rank[] holds ordinals below D (the ranks renumbered 0, 1, 2, ... in their order), and the key is the
+// two-digit number rank[i] * D + rank[i + hop], which takes as few bits as two ordinals can: the passes of the sort
+// follow the bits in use, and a partition whose suffixes share a few hundred ranks sorts in three passes instead of eight.
+__device__ __forceinline__ u64 rank_pair_key(const u32* __restrict__ rank, u32 n, u32 hop, u32 i, u32 radix)
 {
     const u64 j = (u64)i + hop;
-    return ((u64)rank[i] << 32) | (u64)(j < (u64)n ? rank[j] : 0u);
+    const u64 second = j < (u64)n ? rank[j] : 0u;
+    return radix ? (u64)rank[i] * radix + second : ((u64)rank[i] << 32) | second;
 }
 
 // Generation 0 feeds the suffixes in the order (n-1, n-2, ..., n-tail, 0, 1, ..., n-tail-1): the last
@@ -57,8 +61,9 @@ struct HistArgs {
     u32 word;   // key word to build from the text
     PassPlan plan;
     u32* ghist; // [MAX_PASSES][256], zeroed by the caller
-    const u32* rank = nullptr; // non-null: the keys are rank_pair_key(rank, n, hop, i) instead of keys[i]
+    const u32* rank = nullptr; // non-null: the keys are rank_pair_key(rank, n, hop, i, radix) instead of keys[i]
     u32 hop = 0;
+    u32 radix = 0;
 };
 
 // Digit counters live in LDS as hist[pass][bin][copy]: a lane adds to copy (lane % COPIES), so the lanes of
@@ -89,7 +94,7 @@ __global__ __launch_bounds__(256) void radix_hist_kernel(HistArgs a)
         } else {
 #pragma unroll
             for (int k = 0; k < 4; ++k)
-                key[k] = k < have ? (a.rank ? rank_pair_key(a.rank, a.n, a.hop, (u32)(i + k)) : a.keys[i + k]) : 0;
+                key[k] = k < have ? (a.rank ? rank_pair_key(a.rank, a.n, a.hop, (u32)(i + k), a.radix) : a.keys[i + k]) : 0;
         }
         for (int p = 0; p < a.plan.num_passes; ++p) {
             const int sh = a.plan.shift[p];
@@ -287,7 +292,8 @@ struct OnesweepArgs {
     u32 epoch;
     u32* err;
     const u32* rank = nullptr; // SRC_RANKS: rank[] by text position ...
-    u32 hop = 0;               // ... and the distance to the second rank of a key
+    u32 hop = 0;               // ... the distance to the second rank of a key ...
+    u32 radix = 0;             // ... and how the two make the key (rank_pair_key)
 };
 
 // How the workgroups of a radix pass come by their tiles (one each). Whatever the order, a tile waits for the tiles
@@ -347,7 +353,7 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
     constexpr int WAVES = BLOCK / WAVE;
     static_assert(BLOCK >= RADIX_BINS, "one thread per digit is assumed");
     static_assert(sizeof(KeyT) == 8 || (SRC == SRC_PAIRS && HI == 0), "narrow keys are plain pairs");
-    auto rank_key = [&](u32 i) -> u64 { return rank_pair_key(a.rank, a.n, a.hop, i); }; // SRC_RANKS: pair i is text position i
+    auto rank_key = [&](u32 i) -> u64 { return rank_pair_key(a.rank, a.n, a.hop, i, a.radix); }; // SRC_RANKS: pair i is text position i
     const KeyT* __restrict__ keys_in = static_cast<const KeyT*>(a.keys_in);
     KeyT* __restrict__ keys_out = static_cast<KeyT*>(a.keys_out);
 
