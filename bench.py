@@ -608,6 +608,8 @@ def main():
         row = {"g": g, "active": st["active"][g], "groups": st["groups"][g], "big": st["big"][g], "presorted": st["presorted"][g], "passes": st["passes"][g],
                "rank_update": st["rank_update"][g], "small_only": st["small_only"][g], "dense": st["dense"][g], "ms": round(st["ms"][g], 3),
                "alg_GBps": round(gbs, 1), "alg_over_peak": round(gbs / HBM_PEAK_GBS, 4)}
+        if 1 <= g < st["first_sort_generations"]:
+            row["covered_by_first_sort"] = True  # its list is counted on the sorted keys; no time or passes of its own
         if g in moved_gen and st["ms"][g] > 0:
             mv = moved_gen[g] / (st["ms"][g] * 1e-3) / 1e9
             row["moved_GBps"] = round(mv, 1)
@@ -644,7 +646,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u64 keys / u32 ranks", "data": "synthetic",
         "config": {"workload": workloads.NAMES[args.config], "n": n, "key_words": args.key_words,
-                   "generations": st["generations"], "bit_exact_verified": verified, "verified_by": verified_by,
+                   "generations": st["generations"], "key_symbols": st["key_symbols"],
+                   "first_sort_generations": st["first_sort_generations"], "bit_exact_verified": verified, "verified_by": verified_by,
                    "tile_order": "by arrival" if args.shared_device else "XCD-chunked (device declared exclusive)",
                    "ms_per_step_tiles_by_arrival": round(ms_by_arrival, 3)},
         "roofline": roofline,

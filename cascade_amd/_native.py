@@ -13,7 +13,7 @@ CSA_MAX_PART_SZ = 2147483647
 CSA_MAX_INDEX = 1 << 40
 CSA_OK, CSA_ERR_ARG, CSA_ERR_TOO_LARGE, CSA_ERR_HIP, CSA_ERR_INTERNAL = 0, -1, -2, -3, -4
 CSA_FLAG_KERNEL_TIMING = 1
-CSA_TUNE_DEFER_MIN, CSA_TUNE_WINDOW_MIN_CHANGED, CSA_TUNE_XCD_CHUNK = 0, 1, 2
+CSA_TUNE_DEFER_MIN, CSA_TUNE_WINDOW_MIN_CHANGED, CSA_TUNE_XCD_CHUNK, CSA_TUNE_PACK_SYMBOLS = 0, 1, 2, 3
 
 # every symbol include/cascade_hip.h declares
 EXPORTS = (
@@ -62,6 +62,8 @@ class CsaStats(C.Structure):
         ("radix_pairs", C.c_uint64),
         ("radix_ms", C.c_double),
         ("presorted", C.c_uint64 * CSA_MAX_GENERATIONS),
+        ("key_symbols", C.c_uint32),
+        ("first_sort_generations", C.c_uint32),
     ]
 
 

@@ -308,6 +308,7 @@ struct csa_handle {
     u32 xcd_chunk = XCD_CHUNK;                   // tiles of a radix pass that one XCD takes in a row under TILES_STATIC_CHUNKS
     u32 defer_min = DEFER_MIN; // lists at least this long use the bucketed rank update (csa_set_tuning)
     u32 window_min_changed = WINDOW_MIN_CHANGED; // csa_set_tuning (0xFFFFFFFF: never)
+    u32 pack_symbols = 1; // csa_set_tuning: texts over small alphabets start from keys of many symbols (packed_text.hpp)
     csa_step_result last_step = {};              // counters of the last partition step (csa_last_step_result)
     std::vector<hipEvent_t> events;
     hipEvent_t ev_gen[CSA_MAX_GENERATIONS + 2] = {};
@@ -419,9 +420,17 @@ void launch_onesweep32(const csa_handle* hh, OnesweepArgs& a, hipStream_t s)
 // Passes whose digit is the same for every pair are skipped (they would be the identity).
 // src = SRC_RANKS: pair i is ((rank_src[i], rank_src[i + hop]), i), i < n, built by the first pass that runs; the two
 // ranks are combined as rank_pair_key says for `radix`.
+// src = SRC_PACKED: the first pass cuts its keys from the code stream `packed` describes; the caller has filled
+// ghist already (hist_ready = 2). hist_ready = 1 (SRC_TEXT): the byte histograms of the text are in place.
+struct PackedSource {
+    const u32* stream;
+    u64 words;
+    u32 sym_bits, key_bits;
+};
+
 int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 word, u64* kin, u32* vin, u64* kout,
                u32* vout, u32 n, const PassPlan& plan, int* result_in_out, int* passes_run, const u32* rank_src = nullptr,
-               u32 hop = 0, u32 radix = 0)
+               u32 hop = 0, u32 radix = 0, const PackedSource* packed = nullptr, int hist_ready = 0)
 {
     csa_handle* h = L.h;
     hipStream_t s = L.stream;
@@ -430,8 +439,12 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
     if (n == 0)
         return CSA_OK;
     // ghist[MAX_PASSES][256] followed by the two byte histograms of the text
-    HIP_TRY(hipMemsetAsync(h->ghist, 0, (MAX_PASSES + 2) * RADIX_BINS * sizeof(u32), s));
-    if (src == SRC_PAIRS || src == SRC_RANKS) {
+    if (hist_ready == 0)
+        HIP_TRY(hipMemsetAsync(h->ghist, 0, (MAX_PASSES + 2) * RADIX_BINS * sizeof(u32), s));
+    if (src == SRC_PACKED) {
+        if (!packed || hist_ready != 2)
+            return fail(CSA_ERR_INTERNAL, "radix_sort: packed keys come with their histograms");
+    } else if (src == SRC_PAIRS || src == SRC_RANKS) {
         HistArgs ha;
         ha.keys = kin;
         ha.vals = vin;
@@ -478,8 +491,9 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
         // every suffix of the text takes part and the plan is the eight bytes of one key word: the digit
         // histograms follow from the byte histogram of the text, whatever order the pairs are in
         u32* bytehist = h->ghist + MAX_PASSES * RADIX_BINS;
-        hipLaunchKernelGGL(text_byte_hist_kernel, dim3(hist_blocks(256 * 8 * 16, text_n)), dim3(256), 0, s, text, text_n,
-                           bytehist);
+        if (hist_ready == 0)
+            hipLaunchKernelGGL(text_byte_hist_kernel, dim3(hist_blocks(256 * 8 * 16, text_n)), dim3(256), 0, s, text, text_n,
+                               bytehist);
         hipLaunchKernelGGL(text_hist_expand_kernel, dim3(1), dim3(256), 0, s, text, text_n, word, bytehist, h->ghist);
     }
     hipLaunchKernelGGL(radix_scan_hist_kernel, dim3(1), dim3(256), 0, s, h->ghist, h->digit_base, plan.num_passes);
@@ -526,6 +540,12 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
         a.rank = rank_src;
         a.hop = hop;
         a.radix = radix;
+        if (packed) {
+            a.stream = packed->stream;
+            a.stream_words = packed->words;
+            a.sym_bits = packed->sym_bits;
+            a.key_bits = packed->key_bits;
+        }
         int rc = next_ticket(L, &a.ticket);
         if (rc)
             return rc;
@@ -537,6 +557,8 @@ int radix_sort(Launch& L, int src, const u16* text, u32 text_n, u32 tail, u32 wo
             launch_onesweep<SRC_PAIRS>(h, a, s);
         else if (use_src == SRC_RANKS)
             launch_onesweep<SRC_RANKS>(h, a, s);
+        else if (use_src == SRC_PACKED)
+            launch_onesweep<SRC_PACKED>(h, a, s);
         else
             launch_onesweep<SRC_TEXT>(h, a, s);
         if (timed) {
@@ -808,6 +830,50 @@ bool dense_generation(u32 m, u32 groups, u32 n)
     return (u64)m * 5 >= (u64)n * 3 && (u64)m > (u64)groups * SMALL_MAXG_HI && (u64)m >= DENSE_MIN;
 }
 
+// Whether, and how, the first sort of a partition takes keys of many packed symbols (packed_text.hpp). From the byte
+// histograms of the text: a symbol's code is made of the ranks of its two bytes among the byte values that occur, zero
+// (the padding) included; with nhi * nlo <= 256 codes the text qualifies. The key takes the largest context the doubling
+// of the caller's key width reaches inside 64 bits: S = 4 W 2^j symbols, which covers j generations after the first.
+struct PackedPlan {
+    bool enabled;
+    SymbolCodes codes;
+    u32 skipped; // j
+};
+
+PackedPlan plan_packed_text(const u32* bytehist, u32 n, int key_words, u64 room_bytes)
+{
+    PackedPlan pp;
+    memset(&pp, 0, sizeof(pp));
+    u32 nlo = 0, nhi = 0;
+    for (u32 d = 0; d < 256; ++d) {
+        if (d == 0 || bytehist[d] != 0)
+            pp.codes.lo[d] = (u8)nlo++;
+        if (d == 0 || bytehist[256 + d] != 0)
+            pp.codes.hi[d] = (u8)nhi++;
+    }
+    const u32 codes = nlo * nhi;
+    if (codes > 256)
+        return pp;
+    const u32 b = codes <= 2 ? 1u : codes <= 4 ? 2u : codes <= 16 ? 4u : 8u;
+    u32 S = 4u * (u32)key_words;
+    if (S * b > 64)
+        return pp;
+    u32 j = 0;
+    while (2 * S * b <= 64) {
+        S *= 2;
+        ++j;
+    }
+    const u64 words = ((u64)n * b + 31) / 32 + 4;
+    if (words * 4 > room_bytes)
+        return pp;
+    pp.codes.nlo = nlo;
+    pp.codes.bits = b;
+    pp.codes.key_syms = S;
+    pp.skipped = j;
+    pp.enabled = true;
+    return pp;
+}
+
 // Generation 0: ranks the sorted list described by `ra`: counts per tile, scans the counts, reads the totals back, then
 // applies them and brings rank[] up to date, directly from the kernel or through the two-pass bucketed update.
 int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivors, u32* groups, int* rank_update)
@@ -837,6 +903,23 @@ int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivo
     return CSA_OK;
 }
 
+// Survivors and groups of the sorted list of `ra` when only the key bits above ra.key_drop and a context of ra.ell symbols
+// count: what a generation that had stopped at that context would have left.
+int count_step(Launch& L, RerankArgs ra, u32* survivors, u32* groups)
+{
+    csa_handle* h = L.h;
+    const RankTables r = rank_tables(h, ra.m, RANK_TILE);
+    ra.tile_agg = r.tile_agg;
+    ra.tile_prefix = r.tile_prefix;
+    ra.tile_splits = r.tile_splits;
+    ra.slab_total = r.slab_total;
+    ra.slab = r.slab;
+    ra.err = h->counts + 2;
+    hipLaunchKernelGGL((rerank_count_kernel<RANK_BLOCK, RANK_ITEMS>), dim3(r.tiles), dim3(RANK_BLOCK), 0, L.stream, ra);
+    int how = 0;
+    return rank_totals(L, r, true, ra.m, ra.n, false, survivors, groups, &how);
+}
+
 int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_sa40)
 {
     csa_handle* h = L.h;
@@ -850,12 +933,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     // and doubles from there. Every reported generation then has the context, the ranks and the active set of the wide-key
     // generation it stands for. A 4-word key sorted word by word costs 32 radix passes over all suffixes (316 ms on the
     // 1B-token workload); this way it costs what the one-word key costs.
-    const u32 ell = 4u;
     const u64 wide_ell = 4ull * (u64)h->key_words;
-    int folded = 0; // generations after the first that still belong to the reported generation 0
-    for (u64 c = ell; c < wide_ell; c += (c < wide_ell - c ? c : wide_ell - c))
-        ++folded;
-    const u32 tail = n < ell ? n : ell;
 
     RangeScope range_sort("sort_partition n=%u", n);
     HIP_TRY(hipMemsetAsync(h->counts, 0, 4 * sizeof(u32), s));
@@ -863,14 +941,52 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
 
     // ---- generation 0: sort every suffix by its K-gram key, ties of tail suffixes broken by length ----
     RangeScope range_gen0("generation 0 m=%u", n);
+    // The byte histograms of the text come first: they give the digit counts of the passes and tell whether the alphabet
+    // is small enough for keys of more than four symbols.
+    HIP_TRY(hipMemsetAsync(h->ghist, 0, (MAX_PASSES + 2) * RADIX_BINS * sizeof(u32), s));
+    u32* const bytehist = h->ghist + MAX_PASSES * RADIX_BINS;
+    hipLaunchKernelGGL(text_byte_hist_kernel, dim3(hist_blocks(256 * 8 * 16, n)), dim3(256), 0, s, d_text, n, bytehist);
+    PackedPlan pp;
+    memset(&pp, 0, sizeof(pp));
+    if (h->pack_symbols) {
+        u32* h_bytes = h->h_pinned + PINNED_HIST;
+        HIP_TRY(hipMemcpyAsync(h_bytes, bytehist, 2 * RADIX_BINS * sizeof(u32), hipMemcpyDeviceToHost, s));
+        HIP_TRY(hipStreamSynchronize(s));
+        pp = plan_packed_text(h_bytes, n, h->key_words, (u64)h->cap * sizeof(u32));
+    }
+    const u32 ell = pp.enabled ? pp.codes.key_syms : 4u; // symbols the first sort resolves
+    int folded = 0; // generations after the first that still belong to the reported generation 0
+    for (u64 c = ell; c < wide_ell; c += (c < wide_ell - c ? c : wide_ell - c))
+        ++folded;
+    const u32 tail = n < ell ? n : ell;
     int passes = 0, p1 = 0, in_out = 0;
-    const PassPlan full = make_plan(0, 64);
     u64* K[2] = {h->key[0], h->key[1]};
     u32* V[2] = {h->idx[0], h->idx[1]};
     int cur; // the (K, V) set that holds the sorted pairs
     int rc;
     cur = 0;
-    rc = radix_sort(L, SRC_TEXT, d_text, n, tail, 0, K[0], V[0], K[1], V[1], n, full, &in_out, &p1);
+    if (pp.enabled) {
+        // the code stream lives in rank[], which nothing uses before the sorted list is ranked
+        PackedSource ps;
+        u32* const stream = h->rank;
+        ps.stream = stream;
+        ps.sym_bits = pp.codes.bits;
+        ps.key_bits = pp.codes.key_syms * pp.codes.bits;
+        ps.words = ((u64)n * ps.sym_bits + 31) / 32 + 4;
+        u32* const gramhist = bytehist; // (read back already)
+        HIP_TRY(hipMemsetAsync(gramhist, 0, RADIX_BINS * sizeof(u32), s));
+        const u64 enc_blocks = (ps.words + ENCODE_BLOCK - 1) / ENCODE_BLOCK;
+        hipLaunchKernelGGL(encode_text_kernel, dim3((u32)(enc_blocks < 4096 ? enc_blocks : 4096)), dim3(ENCODE_BLOCK), 0, s, d_text, n,
+                           pp.codes, stream, ps.words, gramhist);
+        const PassPlan plan = make_plan(0, (int)ps.key_bits);
+        hipLaunchKernelGGL(packed_hist_expand_kernel, dim3(1), dim3(256), 0, s, ps.stream, n, ps.sym_bits, pp.codes.key_syms,
+                           plan.num_passes, gramhist, h->ghist);
+        HIP_TRY(hipGetLastError());
+        rc = radix_sort(L, SRC_PACKED, d_text, n, tail, 0, K[0], V[0], K[1], V[1], n, plan, &in_out, &p1, nullptr, 0, 0, &ps, 2);
+    } else {
+        rc = radix_sort(L, SRC_TEXT, d_text, n, tail, 0, K[0], V[0], K[1], V[1], n, make_plan(0, 64), &in_out, &p1, nullptr, 0, 0,
+                        nullptr, 1);
+    }
     if (rc)
         return rc;
     passes += p1;
@@ -908,6 +1024,16 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
                             reinterpret_cast<u32*>(bkey[1]) + h->cap};
     };
     u32 m = 0, groups = 0, big = 0;
+    // packed keys: what the generations that the first sort covers would have left (contexts 4 W, 8 W, ... symbols)
+    u32 level_active[8], level_groups[8];
+    for (u32 i = 0; i < pp.skipped; ++i) {
+        RerankArgs rl = ra;
+        rl.ell = (u32)wide_ell << i;
+        rl.key_drop = (ell - rl.ell) * pp.codes.bits;
+        rc = count_step(L, rl, &level_active[i], &level_groups[i]);
+        if (rc)
+            return rc;
+    }
     rc = rerank_step(L, ra, defer_buffers(), &m, &groups, &st->rank_update[0]);
     range_gen0.close();
     if (rc)
@@ -1222,6 +1348,40 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
             st->ms[g] = 0.0f;
         }
         st->generations = gen - merged;
+    }
+    // packed keys: the first sort stands for generations 0 .. skipped of the reference; those after the first are reported
+    // with the lists they would have had and no time or passes of their own
+    st->key_symbols = ell;
+    st->first_sort_generations = 1 + pp.skipped;
+    if (pp.skipped > 0) {
+        const int sk = (int)pp.skipped;
+        if (gen + sk > CSA_MAX_GENERATIONS)
+            return fail(CSA_ERR_INTERNAL, "%d generations do not fit the statistics", gen + sk);
+        for (int g = gen - 1; g >= 1; --g) {
+            st->active[g + sk] = st->active[g];
+            st->groups[g + sk] = st->groups[g];
+            st->big[g + sk] = st->big[g];
+            st->presorted[g + sk] = st->presorted[g];
+            st->passes[g + sk] = st->passes[g];
+            st->rank_update[g + sk] = st->rank_update[g];
+            st->small_only[g + sk] = st->small_only[g];
+            st->dense[g + sk] = st->dense[g];
+            st->ms[g + sk] = st->ms[g];
+        }
+        for (int g = 1; g <= sk; ++g) {
+            st->active[g] = level_active[g - 1];
+            st->groups[g] = level_groups[g - 1];
+            st->big[g] = st->presorted[g] = 0;
+            st->passes[g] = st->rank_update[g] = st->small_only[g] = st->dense[g] = 0;
+            st->ms[g] = 0.0f;
+        }
+        st->generations = gen + sk;
+        // the reference stops at the first generation that leaves nothing active
+        for (int g = 1; g <= sk; ++g)
+            if (st->active[g] == 0) {
+                st->generations = g;
+                break;
+            }
     }
     return CSA_OK;
 }
@@ -1736,6 +1896,7 @@ int csa_set_tuning(csa_handle* h, int knob, uint32_t value)
     switch (knob) {
     case CSA_TUNE_DEFER_MIN: h->defer_min = value; break;
     case CSA_TUNE_WINDOW_MIN_CHANGED: h->window_min_changed = value; break;
+    case CSA_TUNE_PACK_SYMBOLS: h->pack_symbols = value ? 1u : 0u; break;
     case CSA_TUNE_XCD_CHUNK:
         // the chunked order waits for workgroups that are dispatched later: 8 * chunk workgroups of a pass must be able
         // to be resident together, and the device must have room for twice that many (the condition csa_create applies)

@@ -61,6 +61,7 @@ struct RerankArgs {
     int key_words; // 1..4 (the words after the first are re-read from the text where the first words tie)
     u32 n;         // partition size
     u32 ell;       // symbols in the generation-0 key
+    u32 key_drop;  // low bits of the keys that do not count (0: whole keys): the counting pass on a shorter prefix of packed keys
     const u16* text;
     u32* rank;     // [n] by text position
     // Deferred rank update: instead of the scattered write rank[x] = r, the suffix at sorted index c leaves the record
@@ -148,7 +149,7 @@ __global__ __launch_bounds__(BLOCK) void rerank_count_kernel(RerankArgs a)
 #pragma unroll
     for (int k = 0; k < ITEMS + 1; ++k) {
         const u64 c = base + k; // right element of the pair (c - 1, c)
-        bool e = c >= 1 && c < m && key[k] == key[k + 1];
+        bool e = c >= 1 && c < m && ((key[k] ^ key[k + 1]) >> a.key_drop) == 0;
         for (int word = 1; e && word < a.key_words; ++word)
             e = load_kgram(a.text, a.n, suf[k], (u32)word) == load_kgram(a.text, a.n, suf[k + 1], (u32)word);
         // a suffix that runs off the text inside its key ties with nobody (include/bit-layout.hpp:99-100)
@@ -225,7 +226,7 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
 #pragma unroll
     for (int k = 0; k < ITEMS + 1; ++k) {
         const u64 c = base + k; // right element of the pair
-        bool e = c >= 1 && c < m && key[k] == key[k + 1];
+        bool e = c >= 1 && c < m && ((key[k] ^ key[k + 1]) >> a.key_drop) == 0;
         for (int word = 1; e && word < a.key_words; ++word)
             e = load_kgram(a.text, a.n, suf[k], (u32)word) == load_kgram(a.text, a.n, suf[k + 1], (u32)word);
         // a suffix that runs off the text inside its key ties with nobody (include/bit-layout.hpp:99-100)
@@ -827,6 +828,7 @@ __global__ __launch_bounds__(BLOCK) void apply_small_kernel(ApplySmallArgs a)
     constexpr int TILE = BLOCK * ITEMS;
     constexpr int WAVES = BLOCK / WAVE;
     __shared__ u32 s_w[WAVES][2];
+    __shared__ u32 s_suf[TILE], s_gid[TILE], s_head_rank[TILE], s_head_start[TILE];
     const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
     const u32 tile = blockIdx.x;
     const u64 tile_base = (u64)tile * TILE;
@@ -901,33 +903,72 @@ __global__ __launch_bounds__(BLOCK) void apply_small_kernel(ApplySmallArgs a)
     tile_rh += sp.sum3;
     if (t == 0 && tile_base + TILE >= m)
         a.gstart_out[tile_rh + tot_h] = tile_rc + tot_s; // gstart[groups] = survivors
+    // The survivors of a tile and its new groups land in one contiguous stretch each of the next list and of the next
+    // group table: they are compacted in LDS first, so that the stores below go out lane after lane (a thread owns
+    // ITEMS consecutive places, and its own stores would each touch a line that three more stores touch again).
+    const bool full = ITEMS % 4 == 0 && base + ITEMS <= m;
+    u32 rv[ITEMS];
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         const u64 c = base + k;
+        rv[k] = NO_RANK;
         if (c >= m)
             continue;
         const u32 word = nrw[k + 1], nr = word & 0x7FFFFFFFu, x = xs[k];
         const u32 f = (flags >> (2 * k)) & 3u;
         if (nr >= a.n || x >= a.n) {
             atomicExch(a.err, DEV_ERR_RERANK_RANGE);
+            // (a survivor still takes its slot below, so that every slot of the stretch is written: with a value in range)
+            if (f & 2u) {
+                s_head_rank[rh] = 0;
+                s_head_start[rh] = rc;
+                rh++;
+            }
+            if (f & 1u) {
+                s_suf[rc] = 0;
+                s_gid[rc] = rh - 1;
+                rc++;
+            }
             continue;
         }
         if (a.rank_vals)
-            a.rank_vals[c] = (word >> 31) ? nr : NO_RANK;
+            rv[k] = (word >> 31) ? nr : NO_RANK;
         else if (word >> 31)
             a.rank[x] = nr;
         if (!(f & 1u))
             a.sa32[nr] = x; // alone with its key: the rank is final
         if (f & 2u) {
-            a.gprim_out[tile_rh + rh] = nr;
-            a.gstart_out[tile_rh + rh] = tile_rc + rc;
+            s_head_rank[rh] = nr;
+            s_head_start[rh] = rc;
             rh++;
         }
         if (f & 1u) {
-            a.sufs_out[tile_rc + rc] = x;
-            a.gids_out[tile_rc + rc] = tile_rh + rh - 1;
+            s_suf[rc] = x;
+            s_gid[rc] = rh - 1; // (-1 wraps for members of a group that began in an earlier tile: added to tile_rh below)
             rc++;
         }
+    }
+    if (a.rank_vals) {
+        if (full && (reinterpret_cast<uintptr_t>(a.rank_vals) & 15u) == 0) {
+            uint4* out4 = reinterpret_cast<uint4*>(a.rank_vals + base);
+#pragma unroll
+            for (int k = 0; k < ITEMS; k += 4)
+                out4[k / 4] = make_uint4(rv[k], rv[k + 1], rv[k + 2], rv[k + 3]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k)
+                if (base + k < m)
+                    a.rank_vals[base + k] = rv[k];
+        }
+    }
+    __syncthreads();
+    for (u32 i = t; i < tot_s; i += BLOCK) {
+        a.sufs_out[tile_rc + i] = s_suf[i];
+        a.gids_out[tile_rc + i] = tile_rh + s_gid[i];
+    }
+    for (u32 i = t; i < tot_h; i += BLOCK) {
+        a.gprim_out[tile_rh + i] = s_head_rank[i];
+        a.gstart_out[tile_rh + i] = tile_rc + s_head_start[i];
     }
 }
 

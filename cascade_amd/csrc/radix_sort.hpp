@@ -10,6 +10,7 @@
 #pragma once
 
 #include "device_utils.hpp"
+#include "packed_text.hpp"
 
 namespace csa {
 
@@ -27,7 +28,8 @@ struct PassPlan {
 enum : int {
     SRC_PAIRS = 0, // keys_in[i], vals_in[i]
     SRC_TEXT = 1,  // generation 0, first pass: the pair of virtual position i is built from the text
-    SRC_RANKS = 2  // a dense later generation, first pass: pair i = ((rank[i], rank[i + hop]), i), built from rank[]
+    SRC_RANKS = 2, // a dense later generation, first pass: pair i = ((rank[i], rank[i + hop]), i), built from rank[]
+    SRC_PACKED = 3 // generation 0 over a small alphabet, first pass: the key of virtual position i is cut from the code stream
 };
 
 // Key of text position i in a dense generation: its rank, then the rank of the suffix `hop` symbols on (0 past the
@@ -294,6 +296,10 @@ struct OnesweepArgs {
     const u32* rank = nullptr; // SRC_RANKS: rank[] by text position ...
     u32 hop = 0;               // ... the distance to the second rank of a key ...
     u32 radix = 0;             // ... and how the two make the key (rank_pair_key)
+    const u32* stream = nullptr; // SRC_PACKED: the code stream of the text (packed_text.hpp), stream_words words of it ...
+    u64 stream_words = 0;
+    u32 sym_bits = 0;            // ... with sym_bits bits per symbol ...
+    u32 key_bits = 0;            // ... and keys of key_bits bits
 };
 
 // How the workgroups of a radix pass come by their tiles (one each). Whatever the order, a tile waits for the tiles
@@ -402,7 +408,25 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
         sym_off = stage_text(a.text, a.text_n, (u64)j0 + 4ull * a.word, count, reinterpret_cast<u64*>(s_keys), t, BLOCK);
         __syncthreads();
     }
-    auto text_key = [&](u32 i) -> u64 { // key of virtual position i of this tile (SRC_TEXT)
+    // the same over a small alphabet: the tile's stretch of the code stream (TILE * sym_bits bits and a key's worth more)
+    u64 stream_bit0 = 0;
+    if constexpr (SRC == SRC_PACKED) {
+        const u32 first_virtual = (u32)base > a.tail ? (u32)base : a.tail;
+        const u64 first_word = ((u64)(first_virtual - a.tail) * a.sym_bits) >> 5;
+        stream_bit0 = first_word << 5;
+        const u32 count = (u32)((((u64)TILE * a.sym_bits + a.key_bits) >> 5) + 3u);
+        static_assert(sizeof(KeyT) * TILE >= 4 * (TILE * 8 / 32 + 6), "the staged codes must fit the reorder buffer");
+        u32* s_codes = reinterpret_cast<u32*>(s_keys);
+        for (u32 i = t; i < count; i += BLOCK)
+            s_codes[i] = first_word + i < a.stream_words ? a.stream[first_word + i] : 0u;
+        __syncthreads();
+    }
+    auto text_key = [&](u32 i) -> u64 { // key of virtual position i of this tile (SRC_TEXT, SRC_PACKED)
+        if constexpr (SRC == SRC_PACKED) {
+            if (i < a.tail)
+                return packed_window(a.stream, (u64)(a.text_n - 1u - i) * a.sym_bits, a.key_bits);
+            return packed_window(reinterpret_cast<const u32*>(s_keys), (u64)(i - a.tail) * a.sym_bits - stream_bit0, a.key_bits);
+        }
         if (i < a.tail)
             return load_kgram(a.text, a.text_n, a.text_n - 1u - i, a.word);
         return staged_kgram(reinterpret_cast<const u32*>(s_keys), (i - a.tail) - j0 + sym_off);
@@ -524,9 +548,9 @@ __global__ __launch_bounds__(BLOCK, CSA_SORT_MIN_WAVES) void onesweep_kernel(One
         const u32 local = first_local + k * WAVE;
         val[k] = 0;
         if (VALS && local < valid)
-            val[k] = SRC == SRC_TEXT    ? virtual_to_suffix((u32)(base + local), a.text_n, a.tail)
-                     : SRC == SRC_RANKS ? (u32)(base + local)
-                                        : a.vals_in[base + local];
+            val[k] = (SRC == SRC_TEXT || SRC == SRC_PACKED) ? virtual_to_suffix((u32)(base + local), a.text_n, a.tail)
+                     : SRC == SRC_RANKS                     ? (u32)(base + local)
+                                                            : a.vals_in[base + local];
     }
     // ---- write runs of equal digits to their global places ----
     u32 dst[ITEMS];

@@ -34,6 +34,8 @@ def stats_to_dict(st):
         "radix_launches": int(st.radix_launches),
         "radix_pairs": int(st.radix_pairs),
         "radix_ms": float(st.radix_ms),
+        "key_symbols": int(st.key_symbols),
+        "first_sort_generations": int(st.first_sort_generations),
     }
 
 

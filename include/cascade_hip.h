@@ -68,6 +68,11 @@ typedef struct csa_stats {
     uint64_t presorted[CSA_MAX_GENERATIONS]; /* of big[g], members that skipped the radix sort: every large group of the
                                                 list was in order of rank[x + h] already (rising or falling along the
                                                 list, as in runs of one token and periodic stretches) */
+    uint32_t key_symbols;            /* symbols the first sort resolved: 4 (one K-gram word), or up to 64 when the text's
+                                        alphabet is small enough for packed codes of 1, 2, 4 or 8 bits */
+    uint32_t first_sort_generations; /* generations of the reference that sort stands for: 1, or 1 + j when its keys held
+                                        4 * key_words * 2^j symbols. Generations 1 .. j are then reported with the lists
+                                        they would have had (active[], groups[]) and with no time or passes of their own */
 } csa_stats;
 
 typedef struct csa_handle csa_handle;
@@ -136,8 +141,12 @@ int csa_set_device_exclusive(csa_handle* h, int exclusive);
  *                                (default 16; 0: the exclusive order is the default order); call before
  *                                csa_set_device_exclusive. 8 chunks of that many workgroups must be resident
  *                                together with room to spare: values above compute units / 16 fail with CSA_ERR_ARG
+ *   CSA_TUNE_PACK_SYMBOLS        1 (default): a text whose symbols take at most 256 values (by the values its low and its
+ *                                high bytes take) is sorted first on keys of as many packed symbols as 64 bits hold, which
+ *                                covers the first generations of the doubling (csa_stats.first_sort_generations); 0: the
+ *                                first sort always takes one K-gram word
  * No counterpart in the reference. */
-enum { CSA_TUNE_DEFER_MIN = 0, CSA_TUNE_WINDOW_MIN_CHANGED = 1, CSA_TUNE_XCD_CHUNK = 2 };
+enum { CSA_TUNE_DEFER_MIN = 0, CSA_TUNE_WINDOW_MIN_CHANGED = 1, CSA_TUNE_XCD_CHUNK = 2, CSA_TUNE_PACK_SYMBOLS = 3 };
 int csa_set_tuning(csa_handle* h, int knob, uint32_t value);
 
 /* Frees everything the handle owns (reference: the destructor, src/GPU_SACA.cu:103-120). */

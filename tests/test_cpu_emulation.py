@@ -48,6 +48,7 @@ def emu():
     lib.csa_scratch_high_water.restype = u64
     lib.csa_scratch_high_water.argtypes = [vp]
     lib.csa_last_step_result.argtypes = [vp, C.POINTER(_native.CsaStepResult)]
+    lib.csa_set_tuning.argtypes = [vp, i32, u32]
     return lib
 
 
@@ -60,11 +61,15 @@ def steps_handle(lib, key_words):
     return make
 
 
-def emu_sort(lib, T, key_words):
+def emu_sort(lib, T, key_words, pack=True):
+    """pack=False: the first sort takes one K-gram word even when the alphabet is small (CSA_TUNE_PACK_SYMBOLS 0), for the
+    tests that aim at what the generations after it do on such texts."""
     T = np.ascontiguousarray(T, dtype=np.uint16)
     n = T.size
     h = C.c_void_p()
     assert lib.csa_create(max(n, 1), key_words, C.byref(h)) == 0
+    if not pack:
+        assert lib.csa_set_tuning(h, _native.CSA_TUNE_PACK_SYMBOLS, 0) == 0
     out = np.zeros(5 * n + 8, dtype=np.uint8)
     st = _native.CsaStats()
     rc = lib.csa_sort_partition_u16_dev(h, T.ctypes.data, n, 0, out.ctypes.data, None, 0, C.byref(st))
@@ -74,6 +79,8 @@ def emu_sort(lib, T, key_words):
     emu_sort.small_only = [int(st.small_only[i]) for i in range(st.generations)]
     emu_sort.dense = [int(st.dense[i]) for i in range(st.generations)]
     emu_sort.presorted = [int(st.presorted[i]) for i in range(st.generations)]
+    emu_sort.key_symbols, emu_sort.first_sort_generations = int(st.key_symbols), int(st.first_sort_generations)
+    emu_sort.passes = [int(st.passes[i]) for i in range(st.generations)]
     return out[:5 * n], [int(st.active[i]) for i in range(st.generations)], [int(st.big[i]) for i in range(st.generations)]
 
 
@@ -133,7 +140,7 @@ def test_large_groups_that_are_in_order_already_skip_the_sort(emu, after_run):
     T = np.concatenate([texts.random_text(1300, 2, 21, sep_every=0) + 6, np.full(700, 5, dtype=np.uint16),
                         np.array([after_run], dtype=np.uint16), np.tile(np.array([3, 1, 4, 1, 5, 9, 2], dtype=np.uint16), 150),
                         texts.random_text(400, 3, 22, sep_every=0)])
-    got, active, big = emu_sort(emu, T, 1)
+    got, active, big = emu_sort(emu, T, 1, pack=False)
     assert np.array_equal(got, oracle_lib.build_sa40(T))
     _, counts = oracle_lib.prefix_doubling(T, 1)
     assert active == counts
@@ -146,7 +153,7 @@ def test_large_groups_that_are_in_order_already_skip_the_sort(emu, after_run):
 def test_small_and_large_groups_take_both_paths(emu):
     # 2 symbols, no separators: generation 1 has a few huge groups (radix path), later ones small groups (in-tile path)
     T = texts.random_text(6000, 2, 5, sep_every=0)
-    got, active, big = emu_sort(emu, T, 1)
+    got, active, big = emu_sort(emu, T, 1, pack=False)
     assert np.array_equal(got, oracle_lib.build_sa40(T))
     assert big[1] > 0 and any(b == 0 and a > 0 for a, b in zip(active[2:], big[2:]))
     # generation 0 takes the bucketed rank update here (records through one value-less radix pass on 4 position bits,
@@ -164,11 +171,49 @@ def test_dense_generations_sort_the_whole_partition_again(emu, name, key_words):
     the dense form (keys (rank[x], rank[x + h]) read in text order, every suffix sorted again, ranks back through the
     bucketed update). Same suffix array and the same active counts as the oracle's doubling, for plain and folded wide keys."""
     T = {"one_symbol": np.full(1700, 7, dtype=np.uint16), "period_3": np.tile(np.array([3, 1, 4], dtype=np.uint16), 560)}[name]
-    got, active, _ = emu_sort(emu, T, key_words)
+    got, active, _ = emu_sort(emu, T, key_words, pack=False)
     sa, counts = oracle_lib.prefix_doubling(T, key_words)
     assert np.array_equal(got, oracle_lib.u64_to_sa40(sa)) and active == counts
     assert emu_sort.dense[0] == 0 and sum(emu_sort.dense) >= 5 and emu_sort.dense[-1] == 0
     assert all(u == 1 for u, d in zip(emu_sort.rank_update, emu_sort.dense) if d)
+
+
+PACKED_CASES = {
+    "four_letters": (np.arange(4), 1, 32, 4),                    # codes of 2 bits
+    "one_letter": (np.array([7]), 1, 64, 5),                     # with the padding's zero: 2 codes, 1 bit
+    "acgt_ascii": (np.array([65, 67, 71, 84]), 1, 16, 3),        # 5 low-byte values with zero: 4 bits
+    "bytes": (np.arange(256), 1, 8, 2),
+    "bytes_two_words": (np.arange(256), 2, 8, 1),                # the caller's own key width, in one word
+    "high_bytes": (np.array([0x0101, 0x0102, 0x0201]), 1, 16, 3),  # 3 x 3 byte ranks: 9 codes
+    "three_words": (np.array([1, 2, 3]), 3, 24, 2),              # 12 -> 24 symbols of 2 bits; 48 would not fit
+    "four_words": (np.arange(4), 4, 32, 2),
+    "bytes_three_words": (np.arange(256), 3, 4, 1),              # 12 bytes do not fit a key: one K-gram word, as ever
+    "large_alphabet": (np.arange(1000, 1300), 1, 4, 1),
+}
+
+
+@pytest.mark.parametrize("name", sorted(PACKED_CASES))
+def test_small_alphabets_start_from_keys_of_many_symbols(emu, name):
+    """A text of at most 256 different symbols (by the values its low and high bytes take, zero, the key padding,
+    counted in) is sorted first on keys of as many packed symbols as 64 bits hold: codes of 1, 2, 4 or 8 bits, 4 W 2^j
+    symbols. That sort stands for the first 1 + j generations of the oracle's doubling: the suffix array is the oracle's, and
+    so is every generation's active count, those of the covered generations included (counted on prefixes of the sorted
+    keys). The texts hold a long repeat that keeps suffixes tied past the key, and zeros at the end, which tie with the
+    padding of the last keys."""
+    alphabet, key_words, key_symbols, first = PACKED_CASES[name]
+    rng = np.random.default_rng(len(name))
+    body = alphabet[rng.integers(0, alphabet.size, 2500)].astype(np.uint16)
+    T = np.concatenate([body, body[300:900], body[:50], np.zeros(3, dtype=np.uint16)]).astype(np.uint16)
+    got, active, _ = emu_sort(emu, T, key_words)
+    sa, counts = oracle_lib.prefix_doubling(T, key_words)
+    assert np.array_equal(got, oracle_lib.u64_to_sa40(sa))
+    assert active == counts
+    assert (emu_sort.key_symbols, emu_sort.first_sort_generations) == (key_symbols, first)
+    assert all(p == 0 for p in emu_sort.passes[1:first])
+    if first > 1 or name == "bytes_two_words":
+        # the same text without the packed keys: the same array, the same counts
+        got2, active2, _ = emu_sort(emu, T, key_words, pack=False)
+        assert np.array_equal(got2, got) and active2 == counts and emu_sort.first_sort_generations == 1
 
 
 def test_emulated_radix_sort_matches_stable_sort(emu):

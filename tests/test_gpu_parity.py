@@ -263,13 +263,16 @@ def test_many_small_partitions_of_low_entropy(torch_mod):
 @pytest.mark.parametrize("config", [2, 3, 4, 5])
 def test_sixteen_million_symbols_pass_the_oracle_verifier(torch_mod, config, exclusive):
     """Large enough for the bucketed rank update and many radix tiles; checked with the O(n) verifier of the
-    oracle (pass = byte-equal to the reference's suffix array, which is unique) and with the device verifier."""
-    from cascade_amd import PartitionSorter, workloads
+    oracle (pass = byte-equal to the reference's suffix array, which is unique) and with the device verifier.
+    (One K-gram word in the first sort, also for the four letters of config 4: the generations after it are what is
+    looked at here; test_four_letters_start_from_keys_of_32_symbols sorts the same text the default way.)"""
+    from cascade_amd import PartitionSorter, workloads, _native
     n = 1 << 24
     T = workloads.generate(config, n)
     d = to_dev(torch_mod, T)
     with PartitionSorter(n, key_words=1, device_exclusive=exclusive) as s:
         print(f"  sort config={config} n={n} exclusive={exclusive}", flush=True)
+        s.set_tuning(_native.CSA_TUNE_PACK_SYMBOLS, 0)
         out = s.sort(d)
         torch_mod.cuda.synchronize()
         assert s.verify(d, out)
@@ -304,12 +307,13 @@ def test_two_dense_generations_in_a_row_on_a_four_letter_text(torch_mod, exclusi
     whole partition again from the ranks read in text order; the suffix array passes the oracle's verifier and the
     generation sizes are the ones the oracle's doubling reports on a prefix-compatible smaller text (every suffix stays
     active through generation 2)."""
-    from cascade_amd import PartitionSorter, workloads
+    from cascade_amd import PartitionSorter, workloads, _native
     n = 20_000_000
     T = workloads.generate(4, n)
     d = to_dev(torch_mod, T)
     with PartitionSorter(n, key_words=1, device_exclusive=exclusive) as s:
         print(f"  sort config=4 n={n} exclusive={exclusive}", flush=True)
+        s.set_tuning(_native.CSA_TUNE_PACK_SYMBOLS, 0)
         out = s.sort(d)
         torch_mod.cuda.synchronize()
         assert s.verify(d, out)
@@ -318,6 +322,60 @@ def test_two_dense_generations_in_a_row_on_a_four_letter_text(torch_mod, exclusi
     assert oracle_lib.is_correct_sa40(got, T)
     assert stats["dense"][:4] == [0, 1, 1, 0] and stats["rank_update"][1] == 1 and stats["rank_update"][2] == 1
     assert stats["groups"][1] == 256 and stats["groups"][2] == 65536 and stats["active"][2] >= n - 16
+
+
+@TILE_ORDERS
+@pytest.mark.parametrize("key_words", [1, 4])
+def test_four_letters_start_from_keys_of_32_symbols(torch_mod, key_words, exclusive):
+    """The four-letter workload the default way: codes of 2 bits, 32 symbols in the key of the first sort, which stands for
+    generations 0-3 of the reference's doubling with one-word keys (0-1 with four-word keys). The suffix array passes the
+    oracle's verifier; the generation sizes, the covered generations' included, are those of the same text sorted from
+    one K-gram word, which the oracle's doubling confirms on a text small enough for it."""
+    from cascade_amd import PartitionSorter, workloads, _native
+    n = 1 << 24
+    T = workloads.generate(4, n)
+    d = to_dev(torch_mod, T)
+    with PartitionSorter(n, key_words=key_words, device_exclusive=exclusive) as s:
+        print(f"  packed sort config=4 n={n} key_words={key_words} exclusive={exclusive}", flush=True)
+        out = s.sort(d)
+        torch_mod.cuda.synchronize()
+        assert s.verify(d, out)
+        got = out.cpu().numpy()
+        packed = s.last_stats
+        s.set_tuning(_native.CSA_TUNE_PACK_SYMBOLS, 0)
+        out2 = s.sort(d)
+        plain = s.last_stats
+        assert torch_mod.equal(out, out2)
+        small = workloads.generate(4, 1 << 17)
+        s.set_tuning(_native.CSA_TUNE_PACK_SYMBOLS, 1)
+        got_small = s.sort(to_dev(torch_mod, small)).cpu().numpy()
+        small_stats = s.last_stats
+    assert oracle_lib.is_correct_sa40(got, T)
+    first = {1: 4, 4: 2}[key_words]
+    assert (packed["key_symbols"], packed["first_sort_generations"]) == (32, first) and plain["first_sort_generations"] == 1
+    assert packed["active"] == plain["active"] and packed["groups"][1:] == plain["groups"][1:]
+    assert packed["passes"][0] == 8 and all(p == 0 for p in packed["passes"][1:first]) and not any(packed["dense"])
+    sa, counts = oracle_lib.prefix_doubling(small, key_words)
+    assert np.array_equal(got_small, oracle_lib.u64_to_sa40(sa)) and small_stats["active"] == counts
+    assert small_stats["first_sort_generations"] == first
+
+
+def test_byte_texts_start_from_keys_of_8_symbols(torch_mod):
+    """A text of byte values (every value 0..255 occurs): codes of 8 bits, 8 symbols in the first key, which covers
+    generations 0-1 of one-word keys. A million symbols with long repeats and a tail of zeros, against the oracle."""
+    from cascade_amd import PartitionSorter
+    rng = np.random.default_rng(5)
+    n = 1 << 20
+    T = rng.integers(0, 256, n).astype(np.uint16)
+    T[n // 2:n // 2 + 50000] = T[1000:51000]
+    T[n // 3:n // 3 + 3000] = 65
+    T[-5:] = 0
+    with PartitionSorter(n, key_words=1) as s:
+        got = s.sort(to_dev(torch_mod, T)).cpu().numpy()
+        stats = s.last_stats
+    sa, counts = oracle_lib.prefix_doubling(T, 1)
+    assert np.array_equal(got, oracle_lib.u64_to_sa40(sa)) and stats["active"] == counts
+    assert (stats["key_symbols"], stats["first_sort_generations"]) == (8, 2)
 
 
 def test_random_small_texts_against_the_oracle(torch_mod):
