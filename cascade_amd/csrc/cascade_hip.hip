@@ -876,7 +876,8 @@ PackedPlan plan_packed_text(const u32* bytehist, u32 n, int key_words, u64 room_
 
 // Generation 0: ranks the sorted list described by `ra`: counts per tile, scans the counts, reads the totals back, then
 // applies them and brings rank[] up to date, directly from the kernel or through the two-pass bucketed update.
-int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivors, u32* groups, int* rank_update)
+int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivors, u32* groups, int* rank_update,
+                u32* level_counts = nullptr)
 {
     csa_handle* h = L.h;
     hipStream_t s = L.stream;
@@ -888,10 +889,27 @@ int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivo
     ra.slab = r.slab;
     ra.err = h->counts + 2;
     ra.rank_recs = nullptr;
+    // the level counts of packed keys ride along: accumulated in the (idle) digit histograms, read back with the totals
+    unsigned long long* const h_levels = reinterpret_cast<unsigned long long*>(h->h_pinned + PINNED_HIST + 512);
+    if (ra.levels) {
+        ra.level_totals = reinterpret_cast<unsigned long long*>(h->ghist);
+        HIP_TRY(hipMemsetAsync(ra.level_totals, 0, LEVEL_SLOTS * 8 * sizeof(unsigned long long), s));
+    }
     hipLaunchKernelGGL((rerank_count_kernel<RANK_BLOCK, RANK_ITEMS>), dim3(r.tiles), dim3(RANK_BLOCK), 0, s, ra);
+    if (ra.levels)
+        HIP_TRY(hipMemcpyAsync(h_levels, ra.level_totals, LEVEL_SLOTS * 8 * sizeof(unsigned long long), hipMemcpyDeviceToHost, s));
     int rc = rank_totals(L, r, true, ra.m, ra.n, false, survivors, groups, rank_update);
     if (rc)
         return rc;
+    for (u32 i = 0; i < ra.levels && level_counts; ++i) {
+        u64 sv = 0, hd = 0;
+        for (u32 slot = 0; slot < LEVEL_SLOTS; ++slot) {
+            sv += h_levels[slot * 8 + 2 * i];
+            hd += h_levels[slot * 8 + 2 * i + 1];
+        }
+        level_counts[2 * i] = (u32)sv;
+        level_counts[2 * i + 1] = (u32)hd;
+    }
     // what the list becomes decides what rank[] is to hold: ordinals for a dense generation, ranks otherwise
     ra.ordinals = dense_generation(*survivors, *groups, ra.n) ? 1u : 0u;
     if (*rank_update != 0)
@@ -901,23 +919,6 @@ int rerank_step(Launch& L, RerankArgs& ra, const DeferBuffers& buf, u32* survivo
     if (*rank_update == 1)
         return deferred_rank_update(L, buf, ra.n);
     return CSA_OK;
-}
-
-// Survivors and groups of the sorted list of `ra` when only the key bits above ra.key_drop and a context of ra.ell symbols
-// count: what a generation that had stopped at that context would have left.
-int count_step(Launch& L, RerankArgs ra, u32* survivors, u32* groups)
-{
-    csa_handle* h = L.h;
-    const RankTables r = rank_tables(h, ra.m, RANK_TILE);
-    ra.tile_agg = r.tile_agg;
-    ra.tile_prefix = r.tile_prefix;
-    ra.tile_splits = r.tile_splits;
-    ra.slab_total = r.slab_total;
-    ra.slab = r.slab;
-    ra.err = h->counts + 2;
-    hipLaunchKernelGGL((rerank_count_kernel<RANK_BLOCK, RANK_ITEMS>), dim3(r.tiles), dim3(RANK_BLOCK), 0, L.stream, ra);
-    int how = 0;
-    return rank_totals(L, r, true, ra.m, ra.n, false, survivors, groups, &how);
 }
 
 int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_sa40)
@@ -1025,16 +1026,15 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     };
     u32 m = 0, groups = 0, big = 0;
     // packed keys: what the generations that the first sort covers would have left (contexts 4 W, 8 W, ... symbols)
-    u32 level_active[8], level_groups[8];
+    u32 level_counts[2 * MAX_LEVELS]; // (survivors, groups) of each
+    if (pp.skipped > MAX_LEVELS)
+        return fail(CSA_ERR_INTERNAL, "the first sort covers %u generations", pp.skipped);
+    ra.levels = pp.skipped;
     for (u32 i = 0; i < pp.skipped; ++i) {
-        RerankArgs rl = ra;
-        rl.ell = (u32)wide_ell << i;
-        rl.key_drop = (ell - rl.ell) * pp.codes.bits;
-        rc = count_step(L, rl, &level_active[i], &level_groups[i]);
-        if (rc)
-            return rc;
+        ra.level_ell[i] = (u32)wide_ell << i;
+        ra.level_drop[i] = (ell - ra.level_ell[i]) * pp.codes.bits;
     }
-    rc = rerank_step(L, ra, defer_buffers(), &m, &groups, &st->rank_update[0]);
+    rc = rerank_step(L, ra, defer_buffers(), &m, &groups, &st->rank_update[0], level_counts);
     range_gen0.close();
     if (rc)
         return rc;
@@ -1369,8 +1369,8 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
             st->ms[g + sk] = st->ms[g];
         }
         for (int g = 1; g <= sk; ++g) {
-            st->active[g] = level_active[g - 1];
-            st->groups[g] = level_groups[g - 1];
+            st->active[g] = level_counts[2 * (g - 1)];
+            st->groups[g] = level_counts[2 * (g - 1) + 1];
             st->big[g] = st->presorted[g] = 0;
             st->passes[g] = st->rank_update[g] = st->small_only[g] = st->dense[g] = 0;
             st->ms[g] = 0.0f;

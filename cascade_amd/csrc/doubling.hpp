@@ -54,6 +54,8 @@ __device__ __forceinline__ SlabPrefix slabs_before(const u32* __restrict__ slab_
     return p;
 }
 
+constexpr u32 MAX_LEVELS = 4, LEVEL_SLOTS = 64;
+
 struct RerankArgs {
     const u64* keys;
     const u32* sufs;
@@ -61,7 +63,14 @@ struct RerankArgs {
     int key_words; // 1..4 (the words after the first are re-read from the text where the first words tie)
     u32 n;         // partition size
     u32 ell;       // symbols in the generation-0 key
-    u32 key_drop;  // low bits of the keys that do not count (0: whole keys): the counting pass on a shorter prefix of packed keys
+    // Packed keys of many symbols (packed_text.hpp): the counting pass also counts what the list would leave at shorter
+    // contexts. Level i looks at the key bits above level_drop[i] and sets apart the suffixes that run off the text inside
+    // level_ell[i] symbols; its survivors and groups are added to level_totals[slot * 8 + 2 i] and [.. + 1], slot = tile
+    // % LEVEL_SLOTS (spread so that the additions of neighbouring tiles do not queue on one address; zeroed by the caller).
+    u32 levels; // <= MAX_LEVELS
+    u32 level_drop[4];
+    u32 level_ell[4];
+    unsigned long long* level_totals;
     const u16* text;
     u32* rank;     // [n] by text position
     // Deferred rank update: instead of the scattered write rank[x] = r, the suffix at sorted index c leaves the record
@@ -149,7 +158,7 @@ __global__ __launch_bounds__(BLOCK) void rerank_count_kernel(RerankArgs a)
 #pragma unroll
     for (int k = 0; k < ITEMS + 1; ++k) {
         const u64 c = base + k; // right element of the pair (c - 1, c)
-        bool e = c >= 1 && c < m && ((key[k] ^ key[k + 1]) >> a.key_drop) == 0;
+        bool e = c >= 1 && c < m && key[k] == key[k + 1];
         for (int word = 1; e && word < a.key_words; ++word)
             e = load_kgram(a.text, a.n, suf[k], (u32)word) == load_kgram(a.text, a.n, suf[k + 1], (u32)word);
         // a suffix that runs off the text inside its key ties with nobody (include/bit-layout.hpp:99-100)
@@ -164,6 +173,29 @@ __global__ __launch_bounds__(BLOCK) void rerank_count_kernel(RerankArgs a)
             lheads += (ka && !single) ? 1u : 0u;
         }
         prev_eq = e;
+    }
+    // the same counts at the shorter contexts of packed keys (one-word keys: nothing is read from the text)
+    __shared__ u32 s_level[WAVES][MAX_LEVELS];
+    for (u32 i = 0; i < a.levels; ++i) {
+        const u32 drop = a.level_drop[i];
+        const u64 lell = a.level_ell[i];
+        u32 cs = 0, ch = 0;
+        bool pe = false;
+#pragma unroll
+        for (int k = 0; k < ITEMS + 1; ++k) {
+            const u64 c = base + k;
+            const bool e = c >= 1 && c < m && ((key[k] ^ key[k + 1]) >> drop) == 0 && (u64)suf[k] + lell < a.n && (u64)suf[k + 1] + lell < a.n;
+            if (k >= 1 && c - 1 < m) {
+                const bool ka = !pe;
+                const bool single = ka && !e;
+                cs += single ? 0u : 1u;
+                ch += (ka && !single) ? 1u : 0u;
+            }
+            pe = e;
+        }
+        const u32 packed = wave_reduce_sum(cs | (ch << 16)); // at most 64 * ITEMS each
+        if (lane == 0)
+            s_level[w][i] = packed;
     }
     u32 ra = la, rc = lcnt, rh = lheads;
 #pragma unroll
@@ -191,6 +223,18 @@ __global__ __launch_bounds__(BLOCK) void rerank_count_kernel(RerankArgs a)
         a.tile_agg[(u64)tile * 4 + 2] = tc;
         a.tile_agg[(u64)tile * 4 + 3] = th;
         a.tile_splits[tile] = 0;
+    }
+    if (t < a.levels) {
+        u32 sv = 0, hd = 0;
+        for (int ww = 0; ww < WAVES; ++ww) {
+            sv += s_level[ww][t] & 0xFFFFu;
+            hd += s_level[ww][t] >> 16;
+        }
+        unsigned long long* slot = a.level_totals + (u64)(tile % LEVEL_SLOTS) * 8 + 2 * t;
+        if (sv)
+            atomicAdd(slot, (unsigned long long)sv);
+        if (hd)
+            atomicAdd(slot + 1, (unsigned long long)hd);
     }
 }
 
@@ -226,7 +270,7 @@ __global__ __launch_bounds__(BLOCK) void rerank_kernel(RerankArgs a)
 #pragma unroll
     for (int k = 0; k < ITEMS + 1; ++k) {
         const u64 c = base + k; // right element of the pair
-        bool e = c >= 1 && c < m && ((key[k] ^ key[k + 1]) >> a.key_drop) == 0;
+        bool e = c >= 1 && c < m && key[k] == key[k + 1];
         for (int word = 1; e && word < a.key_words; ++word)
             e = load_kgram(a.text, a.n, suf[k], (u32)word) == load_kgram(a.text, a.n, suf[k + 1], (u32)word);
         // a suffix that runs off the text inside its key ties with nobody (include/bit-layout.hpp:99-100)
