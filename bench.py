@@ -591,8 +591,9 @@ def main():
     # generations; a share of the peak above 1 is no measurement either. In both cases the per-generation figures of
     # the profile are dropped (not printed), and the line says why.
     moved_gen_dropped = None
-    if moved_gen and sorted(moved_gen) != list(range(st["generations"])):
-        moved_gen_dropped = f"the profile holds {len(moved_gen)} generations, the run had {st['generations']}"
+    ran = [g for g in range(st["generations"]) if not 1 <= g < st["first_sort_generations"]]  # (the others have no launches)
+    if moved_gen and sorted(moved_gen) != ran:
+        moved_gen_dropped = f"the profile holds generations {sorted(moved_gen)}, the run had {ran}"
     elif any(st["ms"][g] > 0 and moved_gen[g] / (st["ms"][g] * 1e-3) / 1e9 > HBM_PEAK_GBS for g in moved_gen):
         moved_gen_dropped = "a generation's bytes over this run's time exceed the HBM peak"
     if moved_gen_dropped:
