@@ -1519,14 +1519,20 @@ extern "C++" {
 namespace {
 // Builds the join directory of the suffix-ordered cohort d_sa[0, n) in `dir` (room for `room` entries) and returns the
 // log2 of its bucket count through *dir_log2; leaves *dir_log2 = 0 and builds nothing when the cohort is small.
-int build_join_directory(const u64* d_sa, u64 n, u32* dir, u64 room, hipStream_t s, u32* dir_log2)
+int build_join_directory(const u64* d_sa, u64 n, u32* dir, u64 room, hipStream_t s, u32* dir_log2, bool sorted_probes)
 {
     *dir_log2 = 0;
     if (n < CSA_JOIN_DIR_MIN || room < 3)
         return CSA_OK;
-    u32 lg = (u32)bit_length(n) - 2u; // two to four cohort entries per bucket
-    if (lg > 22u)
-        lg = 22u;
+    // Probes in arrival order: one to two cohort entries per bucket, so that a probe costs the directory's line and one
+    // line of the cohort (with at most 2^22 buckets a cohort of 44 M suffixes had 10 per bucket and the join of 268 M
+    // messages took 14.5 ms instead of 9.5). Probes sorted by target walk the cohort and the directory in order and find
+    // their lines in cache: a coarse directory (two to four entries per bucket, at most 2^22 buckets) is built four
+    // times faster and serves them as well.
+    u32 lg = (u32)bit_length(n) - (sorted_probes ? 2u : 1u);
+    const u32 cap = sorted_probes ? 22u : 26u;
+    if (lg > cap)
+        lg = cap;
     while (lg && (1ull << lg) + 1 > room)
         --lg;
     if (lg == 0)
@@ -1602,7 +1608,7 @@ int csa_join_messages_sorted_dev(csa_handle* h, const uint8_t* d_msg_target, con
     if (rc)
         return rc;
     u32 dir_log2 = 0;
-    rc = build_join_directory(d_sa, n, dir, dir_room, s, &dir_log2);
+    rc = build_join_directory(d_sa, n, dir, dir_room, s, &dir_log2, true);
     if (rc)
         return rc;
     hipLaunchKernelGGL(join_messages_kernel, dim3((msg_c + 255u) / 256u), dim3(256), 0, s, (const u8*)nullptr,

@@ -369,7 +369,7 @@ int step_rerank(Launch& L, const char* who, StepColumns& c, const StepPlan& pl, 
     hipLaunchKernelGGL(fill_u64_kernel, dim3(blocks), dim3(256), 0, s, keys, m, ~0ull);
     if (c.inbox_sz) {
         u32 dir_log2 = 0;
-        rc = build_join_directory(words_by_suffix, m, dir, m, s, &dir_log2);
+        rc = build_join_directory(words_by_suffix, m, dir, m, s, &dir_log2, false);
         if (rc)
             return rc;
         hipLaunchKernelGGL(join_messages_kernel, dim3((c.inbox_sz + 255u) / 256u), dim3(256), 0, s, c.inbox_target, (const u64*)nullptr,

@@ -387,6 +387,12 @@ def test_random_small_texts_against_the_oracle(torch_mod):
         n = int(rng.integers(1, 6000))
         sigma = int(rng.integers(1, 5))
         T = rng.integers(0, sigma, n).astype(np.uint16)
+        if case % 5 == 2:  # other alphabets that still pack: scattered byte values, two high bytes, up to 200 symbols
+            sigma = int(rng.choice([3, 7, 16, 40, 200]))
+            alphabet = rng.choice(np.arange(1, 256), size=min(sigma, 120), replace=False).astype(np.uint16)
+            if case % 10 == 2:
+                alphabet = np.concatenate([alphabet[:sigma // 2 + 1], alphabet[:sigma // 2 + 1] + 0x0700]).astype(np.uint16)
+            T = alphabet[rng.integers(0, alphabet.size, n)]
         if case % 3 == 0:
             T[-int(rng.integers(1, min(n, 40) + 1)):] = 0
         if case % 4 == 1 and n > 600:
