@@ -148,7 +148,9 @@ constexpr int RANK_TILE = RANK_BLOCK * RANK_ITEMS;
 // the radix sort. A list of mostly short groups (at most SMALL_AVG_LIMIT members per group on average: token corpora)
 // takes the higher limit SMALL_MAXG_HI, which leaves fewer members to the radix passes (1B-token workload: 117.5 ->
 // 115.4 ms per sort). A list of long groups (small alphabets, runs) keeps the lower one: the tile's halo of SMALL_MAXG
-// elements on either side and the longer member loops only cost there (4-letter workload: +6 % with the higher limit).
+// elements on either side and the longer member loops only cost there (4-letter workload sorted from one K-gram word:
+// +6 % with the higher limit). The adversarial workload's generation 1 averages 16.5 members per group, most of them in
+// groups of 65 to 256: the higher limit takes 37 M members off its radix passes (31.1 -> 29.0 ms), hence 32.
 #ifndef CSA_SMALL_MAXG
 #define CSA_SMALL_MAXG 64
 #endif
@@ -156,7 +158,7 @@ constexpr int RANK_TILE = RANK_BLOCK * RANK_ITEMS;
 #define CSA_SMALL_MAXG_HI 256
 #endif
 #ifndef CSA_SMALL_AVG_LIMIT
-#define CSA_SMALL_AVG_LIMIT 16
+#define CSA_SMALL_AVG_LIMIT 32
 #endif
 // tile of the small-group kernel and of the counting / applying kernels behind it (measured per sort of the 1B-token
 // workload with 16-byte loads in the applying kernel: 256 x 8 109.4 ms, 256 x 4 106.5, 512 x 4 106.2, 1024 x 4 106.7,
@@ -1424,8 +1426,9 @@ int csa_partition_ids_u16_dev(const uint16_t* d_text, uint64_t n, uint64_t text_
     a.tiles = (u32)tiles64;
     const u32 grid = a.tiles < 8192u ? a.tiles : 8192u;
     hipStream_t s = (hipStream_t)stream;
-    const bool piv_lds = (u64)(p - 1) * (u64)pivot_words <= PID_LDS_PIVOT_WORDS;
-    const u32 lds = partition_ids_lds_bytes(pivot_words, p, piv_lds, d_psz != nullptr, &a.hist_copies_log2);
+    // (the table in LDS is filled up to 2^bits(p - 1) - 1 entries)
+    const bool piv_lds = (((u64)1 << bit_length((u64)(p - 1))) - 1) * (u64)pivot_words <= PID_LDS_PIVOT_WORDS;
+    const u32 lds = partition_ids_lds_bytes(pivot_words, p, piv_lds, d_psz != nullptr, d_packed != nullptr, a.bits, &a.hist_copies_log2);
 #define CSA_LAUNCH_PID(W)                                                                                  \
     do {                                                                                                   \
         if (piv_lds)                                                                                       \

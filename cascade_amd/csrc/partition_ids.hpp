@@ -30,7 +30,10 @@ constexpr u32 PID_LDS_BINS = 4096;        // partition sizes are counted in LDS 
 
 // LDS bytes of a workgroup, and the histogram replication that goes with them: at most 16 counters per partition and
 // at most 16 KB of histogram.
-inline u32 partition_ids_lds_bytes(int W, u32 p, bool piv_lds, bool want_sizes, u32* copies_log2)
+// words of the packed map that one tile fills: PID_TILE / 64 groups of `bits` 64-bit words
+__host__ __device__ inline u32 partition_ids_pack_words(u32 bits) { return (u32)(PID_TILE / 64) * bits; }
+
+inline u32 partition_ids_lds_bytes(int W, u32 p, bool piv_lds, bool want_sizes, bool want_packed, u32 bits, u32* copies_log2)
 {
     u32 c = 0;
     const bool hist_lds = want_sizes && p <= PID_LDS_BINS;
@@ -38,12 +41,19 @@ inline u32 partition_ids_lds_bytes(int W, u32 p, bool piv_lds, bool want_sizes, 
         ++c;
     *copies_log2 = c;
     const u32 text_words = (PID_TILE + 4 * W + 6) / 4 + 2;
-    return text_words * 8u + (piv_lds ? (p - 1u) * (u32)W * 8u : 0u) + (hist_lds ? (p << c) * 4u : 0u);
+    u32 steps = 0;
+    while (((p - 1u) >> steps) != 0)
+        ++steps;
+    return text_words * 8u + (piv_lds ? ((1u << steps) - 1u) * (u32)W * 8u : 0u) + (want_packed ? partition_ids_pack_words(bits) * 8u : 0u) +
+           (hist_lds ? (p << c) * 4u : 0u);
 }
 
 // W: 64-bit words per pivot (the reference's K_WORDS, include/Packed_Prefix.hpp:26-34). PIV_LDS: the pivots fit in LDS.
-// A wave handles 64 consecutive suffixes at a time: exactly one group of the packed map, whose `bits` words the
-// wave assembles with one shuffle and one ballot per word. The searches of a thread's PID_ITEMS suffixes advance
+// A wave handles 64 consecutive suffixes at a time: exactly one group of the packed map. The map is a bit stream (entry e
+// of a group takes bits [e * bits, (e + 1) * bits) of the group's `bits` words, least significant first): every lane ORs
+// its entry into an image of the tile's stretch of the map in LDS (one or two 32-bit LDS atomics), and after a barrier
+// the workgroup stores the image as one contiguous run of words. (One shuffle and one ballot per word and group, the
+// first form, was 45 % of the kernel's instructions at 9 bits per entry.) The searches of a thread's PID_ITEMS suffixes advance
 // together, one pivot probe each per step, so that their LDS (or cache) latencies overlap. Workgroups stride over
 // the tiles so that the LDS histogram is flushed once per workgroup, not once per tile; it is replicated so that
 // the lanes of a wave that meet in one hot partition spread over several counters.
@@ -57,29 +67,30 @@ __global__ __launch_bounds__(PID_BLOCK) void partition_ids_kernel(PartitionIdArg
     constexpr u32 TEXT_WORDS = (PID_TILE + 4 * W + 6) / 4 + 2;
     u64* s_text = s_dyn;
     const u32 np = a.p - 1u; // pivots
-    u64* s_piv = s_dyn + TEXT_WORDS;
-    u32* s_hist = reinterpret_cast<u32*>(s_piv + (PIV_LDS ? np * (u32)W : 0u));
-    const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
-    const bool hist_lds = a.psz != nullptr && a.p <= PID_LDS_BINS;
-    const u32 copies_log2 = a.hist_copies_log2; // counters per partition in the LDS histogram
-    if (PIV_LDS)
-        for (u32 i = t; i < np * (u32)W; i += PID_BLOCK)
-            s_piv[i] = a.pivots[i];
-    if (hist_lds)
-        for (u32 i = t; i < (a.p << copies_log2); i += PID_BLOCK)
-            s_hist[i] = 0;
     int steps = 0; // bits of the pivot count: probes per search
     while ((np >> steps) != 0)
         ++steps;
-    // entry and bit inside the entry that this lane contributes to word 0 of a group; +64 bits per further word
-    const u32 ent0 = lane / a.bits, sh0 = lane % a.bits;
-    const u32 dq = 64u / a.bits, dr = 64u % a.bits;
+    const u32 piv_slots = PIV_LDS ? ((1u << steps) - 1u) * (u32)W : 0u; // the table, filled up with all-ones keys
+    u64* s_piv = s_dyn + TEXT_WORDS;
+    u64* s_pack = s_piv + piv_slots;
+    const u32 pack_words = a.packed ? partition_ids_pack_words(a.bits) : 0u;
+    u32* s_hist = reinterpret_cast<u32*>(s_pack + pack_words);
+    const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
+    const bool hist_lds = a.psz != nullptr && a.p <= PID_LDS_BINS;
+    const u32 copies_log2 = a.hist_copies_log2; // counters per partition in the LDS histogram
+    for (u32 i = t; i < piv_slots; i += PID_BLOCK)
+        s_piv[i] = i < np * (u32)W ? a.pivots[i] : ~0ull;
+    if (hist_lds)
+        for (u32 i = t; i < (a.p << copies_log2); i += PID_BLOCK)
+            s_hist[i] = 0;
     __syncthreads();
 
     for (u32 tile = blockIdx.x; tile < a.tiles; tile += gridDim.x) {
         const u64 tile_base = (u64)tile * PID_TILE;
         const u32 count = (u32)(a.n - tile_base < (u64)PID_TILE ? a.n - tile_base : (u64)PID_TILE);
         const u32 sym_off = stage_text(a.text, a.text_len, tile_base, count + 4u * W - 1u, s_text, t, PID_BLOCK);
+        for (u32 i = t; i < pack_words; i += PID_BLOCK)
+            s_pack[i] = 0;
         __syncthreads();
         const u32* s_dw = reinterpret_cast<const u32*>(s_text);
 
@@ -95,14 +106,26 @@ __global__ __launch_bounds__(PID_BLOCK) void partition_ids_kernel(PartitionIdArg
                 key[k][j] = local < count ? staged_kgram(s_dw, sym_off + local + 4u * j) : 0ull;
         }
         // id = number of pivots below the key = the smallest id with key <= pivots[id], p - 1 if there is none
-        // (test/partitioning.cpp:21-31), found by fixing the bits of the answer from the top
+        // (test/partitioning.cpp:21-31), found by fixing the bits of the answer from the top. In LDS the table is filled up
+        // to 2^steps - 1 entries with all-ones keys, which are below no key: no probe needs a bounds check, and every
+        // probe reads all W words and decides without a branch.
         for (int b = steps - 1; b >= 0; --b) {
 #pragma unroll
             for (int k = 0; k < PID_ITEMS; ++k) {
                 const u32 cand = id[k] + (1u << b);
-                if (cand <= np) {
-                    const u64* pv = (PIV_LDS ? s_piv : a.pivots) + (u64)(cand - 1u) * W;
-                    bool below = false; // pivot < key
+                if (PIV_LDS) {
+                    const u64* pv = s_piv + (u64)(cand - 1u) * W;
+                    bool below = false, decided = false; // pivot < key, by the first word that differs
+#pragma unroll
+                    for (int j = 0; j < W; ++j) {
+                        const u64 x = pv[j];
+                        below = decided ? below : x < key[k][j];
+                        decided = decided || x != key[k][j];
+                    }
+                    id[k] = below ? cand : id[k];
+                } else if (cand <= np) {
+                    const u64* pv = a.pivots + (u64)(cand - 1u) * W;
+                    bool below = false;
 #pragma unroll
                     for (int j = 0; j < W; ++j) {
                         const u64 x = pv[j];
@@ -134,29 +157,26 @@ __global__ __launch_bounds__(PID_BLOCK) void partition_ids_kernel(PartitionIdArg
             } else {
                 id[k] = 0;
             }
-            if (a.packed) {
-                // Entries fill the words least significant bits first (include/Partition_ID_Map.hpp:158-177): bit b of
-                // word ww of the group is bit (64 ww + b) % bits of entry (64 ww + b) / bits. Lanes past the end of
-                // the text hold id 0, which is what the reference's partial last word carries there.
-                u32 ent = ent0, sh = sh0;
-                u64 mine = 0;
-                for (u32 ww = 0; ww < a.bits; ++ww) {
-                    const u32 v = __shfl(id[k], ent & 63u);
-                    const u64 m = __ballot(((v >> sh) & 1u) != 0);
-                    if (lane == ww)
-                        mine = m;
-                    ent += dq;
-                    sh += dr;
-                    if (sh >= a.bits) {
-                        sh -= a.bits;
-                        ent++;
-                    }
-                }
-                const u32 sz = count - group_local < 64u ? count - group_local : 64u;
-                const u32 nwords = (sz * a.bits + 63u) / 64u; // the reference writes no more for a partial last group
-                if (lane < nwords)
-                    a.packed[((tile_base + group_local) / 64u) * a.bits + lane] = mine;
+            if (a.packed && id[k] != 0) {
+                // Entries fill the words least significant bits first (include/Partition_ID_Map.hpp:158-177): entry e of the
+                // group is bits [e * bits, (e + 1) * bits) of its words. Lanes past the end of the text hold id 0 and add
+                // nothing, which is what the reference's partial last word carries there.
+                u32* image = reinterpret_cast<u32*>(s_pack + (u64)(w * PID_ITEMS + (u32)k) * a.bits);
+                const u32 bit = lane * a.bits;
+                const u64 v = (u64)id[k] << (bit & 31u); // at most 17 bits, shifted by at most 31
+                atomicOr(&image[bit >> 5], (u32)v);
+                if ((u32)(v >> 32))
+                    atomicOr(&image[(bit >> 5) + 1u], (u32)(v >> 32));
             }
+        }
+        if (a.packed) {
+            __syncthreads();
+            // whole groups take `bits` words each; a partial last group only the words its entries reach
+            const u32 full = count / 64u, rest = count % 64u;
+            const u32 words = full * a.bits + (rest * a.bits + 63u) / 64u;
+            u64* out = a.packed + (tile_base / 64u) * a.bits;
+            for (u32 i = t; i < words; i += PID_BLOCK)
+                out[i] = s_pack[i];
         }
         __syncthreads(); // the staged text is replaced in the next round
     }

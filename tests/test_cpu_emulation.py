@@ -202,7 +202,7 @@ def test_small_alphabets_start_from_keys_of_many_symbols(emu, name):
     padding of the last keys."""
     alphabet, key_words, key_symbols, first = PACKED_CASES[name]
     rng = np.random.default_rng(len(name))
-    body = alphabet[rng.integers(0, alphabet.size, 2500)].astype(np.uint16)
+    body = alphabet[rng.integers(0, alphabet.size, 900 if name == "one_letter" else 2500)].astype(np.uint16)  # (one letter: every generation is dense)
     T = np.concatenate([body, body[300:900], body[:50], np.zeros(3, dtype=np.uint16)]).astype(np.uint16)
     got, active, _ = emu_sort(emu, T, key_words)
     sa, counts = oracle_lib.prefix_doubling(T, key_words)
