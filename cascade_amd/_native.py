@@ -13,7 +13,7 @@ CSA_MAX_PART_SZ = 2147483647
 CSA_MAX_INDEX = 1 << 40
 CSA_OK, CSA_ERR_ARG, CSA_ERR_TOO_LARGE, CSA_ERR_HIP, CSA_ERR_INTERNAL = 0, -1, -2, -3, -4
 CSA_FLAG_KERNEL_TIMING = 1
-CSA_TUNE_DEFER_MIN, CSA_TUNE_WINDOW_MIN_CHANGED, CSA_TUNE_XCD_CHUNK, CSA_TUNE_PACK_SYMBOLS = 0, 1, 2, 3
+CSA_TUNE_DEFER_MIN, CSA_TUNE_WINDOW_MIN_CHANGED, CSA_TUNE_XCD_CHUNK, CSA_TUNE_PACK_SYMBOLS, CSA_TUNE_EXPECT_PRESORTED = 0, 1, 2, 3, 4
 
 # every symbol include/cascade_hip.h declares
 EXPORTS = (

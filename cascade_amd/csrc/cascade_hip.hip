@@ -310,6 +310,7 @@ struct csa_handle {
     u32 xcd_chunk = XCD_CHUNK;                   // tiles of a radix pass that one XCD takes in a row under TILES_STATIC_CHUNKS
     u32 defer_min = DEFER_MIN; // lists at least this long use the bucketed rank update (csa_set_tuning)
     u32 window_min_changed = WINDOW_MIN_CHANGED; // csa_set_tuning (0xFFFFFFFF: never)
+    u32 expect_presorted = 0; // csa_set_tuning: 1 = every generation first runs as if its large groups were in order already
     u32 pack_symbols = 1; // csa_set_tuning: texts over small alphabets start from keys of many symbols (packed_text.hpp)
     csa_step_result last_step = {};              // counters of the last partition step (csa_last_step_result)
     std::vector<hipEvent_t> events;
@@ -390,15 +391,10 @@ void launch_onesweep_shape(const TileOrder& o, OnesweepArgs& a, hipStream_t s)
         hipLaunchKernelGGL((onesweep_kernel<u64, BLOCK, SORT_ITEMS, SRC, 0, VALS>), dim3(a.tiles), dim3(BLOCK), 0, s, a);
 }
 
-// the first pass of generation 0 (keys built from the text) may take the other shape
-#ifndef CSA_TEXT_WIDE
-#define CSA_TEXT_WIDE 1
-#endif
-
 template <int SRC, bool VALS = true>
 void launch_onesweep(const csa_handle* h, OnesweepArgs& a, hipStream_t s)
 {
-    if (wide_workgroups(a) && (SRC != SRC_TEXT || CSA_TEXT_WIDE))
+    if (wide_workgroups(a))
         launch_onesweep_shape<SRC, SORT_WIDE_BLOCK, VALS>(tile_order_of(h), a, s);
     else
         launch_onesweep_shape<SRC, SORT_BLOCK, VALS>(tile_order_of(h), a, s);
@@ -1050,6 +1046,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
     int gen = 1;
     int gp = 0; // gprim[gp] / gstart[gp] describe the current groups
     bool all_small = false; // no group of the current list exceeds the limit of the generation that found it so
+    bool presorted_before = false; // every large group of the generation before was in order as it stood
     bool high_limit = false; // that generation's limit was SMALL_MAXG_HI (groups only split: the limit stays from there on)
     const int sec_bits = bit_length(n > 1 ? n - 1 : 1);
     u64 ctx = ell; // symbols resolved so far; the next generation looks hop symbols ahead
@@ -1113,6 +1110,7 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
             st->passes[gen] = passes;
             st->dense[gen] = 1;
             all_small = false;
+            presorted_before = false;
             gp ^= 1;
             HIP_TRY(hipEventRecord(h->ev_gen[gen + 1], s));
             gen++;
@@ -1184,12 +1182,20 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
                                    gr.tile_agg, gr.tile_splits, (const u32*)gr.tile_prefix, (const u32*)gr.slab_total, gr.slab, gr.slabs,
                                    h->counts + 4);
             }
-            if (high_limit)
-                hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG_HI, false>), dim3(r.tiles), dim3(SMALL_BLOCK), 0,
-                                   s, sa);
-            else
-                hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG, false>), dim3(r.tiles), dim3(SMALL_BLOCK), 0, s,
-                                   sa);
+            auto gather_and_sort_small = [&]() {
+                if (high_limit)
+                    hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG_HI, false>), dim3(r.tiles), dim3(SMALL_BLOCK),
+                                       0, s, sa);
+                else
+                    hipLaunchKernelGGL((smallsort_kernel<SMALL_BLOCK, SMALL_ITEMS, SMALL_MAXG, false>), dim3(r.tiles), dim3(SMALL_BLOCK), 0,
+                                       s, sa);
+            };
+            // A list whose large groups were all in order in the generation before (a run, a period: they stay so until
+            // they dissolve) is expected to be so again: the (key, suffix) pairs for the radix sort, 12 of the 16 bytes the
+            // kernel writes per member of a large group, are then left out, and the kernel runs once more with them in
+            // the rare generation in which the marks say otherwise.
+            sa.side_list = (presorted_before || h->expect_presorted) ? 0u : 1u;
+            gather_and_sort_small();
             hipLaunchKernelGGL(group_order_kernel, dim3((marks + 255u) / 256u), dim3(256), 0, s, (const u32*)sa.not_asc, (const u32*)sa.not_desc,
                                marks, h->counts + 5);
             HIP_TRY(hipGetLastError());
@@ -1198,6 +1204,12 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
                 return rc;
             all_small = big == 0;
             const u32 unordered = h->h_pinned[5];
+            if (big > 0 && unordered != 0 && !sa.side_list) {
+                sa.side_list = 1u;
+                gather_and_sort_small();
+                HIP_TRY(hipGetLastError());
+            }
+            presorted_before = big > 0 && unordered == 0;
             if (big > 0 && unordered == 0) {
                 // 2a. every large group is in order as it stands (runs of one token, periodic stretches: the gathered ranks
                 //     rise or fall along the list): no sort, the members are ranked by their runs of equal gathered ranks
@@ -1906,6 +1918,7 @@ int csa_set_tuning(csa_handle* h, int knob, uint32_t value)
     case CSA_TUNE_DEFER_MIN: h->defer_min = value; break;
     case CSA_TUNE_WINDOW_MIN_CHANGED: h->window_min_changed = value; break;
     case CSA_TUNE_PACK_SYMBOLS: h->pack_symbols = value ? 1u : 0u; break;
+    case CSA_TUNE_EXPECT_PRESORTED: h->expect_presorted = value ? 1u : 0u; break;
     case CSA_TUNE_XCD_CHUNK:
         // the chunked order waits for workgroups that are dispatched later: 8 * chunk workgroups of a pass must be able
         // to be resident together, and the device must have room for twice that many (the condition csa_create applies)

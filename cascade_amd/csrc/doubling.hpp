@@ -593,6 +593,8 @@ struct SmallSortArgs {
     u32* nr_out;   // ... and its refined rank, bit 31 set if it differs from the old rank
     u64* big_keys; // elements of groups larger than MAXG: (group id << sec_bits) | rank[x + h], in list order:
     u32* big_sufs; // the member at list place e of large group g goes to big_first[g] + (e - gstart[g])
+    u32 side_list; // 0: the two arrays above are not written (the caller expects every large group to be in order already, as
+                   //    in the generation before, and runs the kernel again if the marks say otherwise)
     const u32* big_first; // [groups]: members of large groups before group g (big_prefix_kernel)
     u32* tile_agg;    // COUNT: [tiles][4], zero before the launch: [2] survivors, [3] new groups per tile of the sorted list
     u32* tile_splits; // COUNT: [tiles], zero before the launch: changed ranks
@@ -703,8 +705,10 @@ __global__ __launch_bounds__(BLOCK) void smallsort_kernel(SmallSortArgs a)
             } else {
                 const u32 first = a.big_first[g[k]];
                 const u32 slot = first + ((u32)e - gs[k]);
-                a.big_keys[slot] = ((u64)g[k] << a.sec_bits) | (u64)sec[k];
-                a.big_sufs[slot] = x[k];
+                if (a.side_list) {
+                    a.big_keys[slot] = ((u64)g[k] << a.sec_bits) | (u64)sec[k];
+                    a.big_sufs[slot] = x[k];
+                }
                 a.big_sec[e] = sec[k];
                 if (e > (long long)gs[k]) { // the member before it in the list belongs to the same group
                     const u32 before = s_sec[MAXG + (e - 1 - t0)]; // an own element, or the last one of the left halo

@@ -145,8 +145,18 @@ int csa_set_device_exclusive(csa_handle* h, int exclusive);
  *                                high bytes take) is sorted first on keys of as many packed symbols as 64 bits hold, which
  *                                covers the first generations of the doubling (csa_stats.first_sort_generations); 0: the
  *                                first sort always takes one K-gram word
+ *   CSA_TUNE_EXPECT_PRESORTED    0 (default): a generation leaves out the (key, suffix) pairs of its large groups' radix sort
+ *                                when every large group of the generation before was in order as it stood (csa_stats.presorted),
+ *                                and gathers again with them if this one's are not; 1: every generation starts that way
+ *                                (tests of the second gather)
  * No counterpart in the reference. */
-enum { CSA_TUNE_DEFER_MIN = 0, CSA_TUNE_WINDOW_MIN_CHANGED = 1, CSA_TUNE_XCD_CHUNK = 2, CSA_TUNE_PACK_SYMBOLS = 3 };
+enum {
+    CSA_TUNE_DEFER_MIN = 0,
+    CSA_TUNE_WINDOW_MIN_CHANGED = 1,
+    CSA_TUNE_XCD_CHUNK = 2,
+    CSA_TUNE_PACK_SYMBOLS = 3,
+    CSA_TUNE_EXPECT_PRESORTED = 4
+};
 int csa_set_tuning(csa_handle* h, int knob, uint32_t value);
 
 /* Frees everything the handle owns (reference: the destructor, src/GPU_SACA.cu:103-120). */

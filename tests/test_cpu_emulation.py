@@ -61,15 +61,17 @@ def steps_handle(lib, key_words):
     return make
 
 
-def emu_sort(lib, T, key_words, pack=True):
+def emu_sort(lib, T, key_words, pack=True, expect_presorted=False):
     """pack=False: the first sort takes one K-gram word even when the alphabet is small (CSA_TUNE_PACK_SYMBOLS 0), for the
-    tests that aim at what the generations after it do on such texts."""
+    tests that aim at what the generations after it do on such texts. expect_presorted: CSA_TUNE_EXPECT_PRESORTED 1."""
     T = np.ascontiguousarray(T, dtype=np.uint16)
     n = T.size
     h = C.c_void_p()
     assert lib.csa_create(max(n, 1), key_words, C.byref(h)) == 0
     if not pack:
         assert lib.csa_set_tuning(h, _native.CSA_TUNE_PACK_SYMBOLS, 0) == 0
+    if expect_presorted:
+        assert lib.csa_set_tuning(h, _native.CSA_TUNE_EXPECT_PRESORTED, 1) == 0
     out = np.zeros(5 * n + 8, dtype=np.uint8)
     st = _native.CsaStats()
     rc = lib.csa_sort_partition_u16_dev(h, T.ctypes.data, n, 0, out.ctypes.data, None, 0, C.byref(st))
@@ -148,6 +150,11 @@ def test_large_groups_that_are_in_order_already_skip_the_sort(emu, after_run):
     assert any(p > 0 for p in presorted), (big, presorted)
     assert all(p in (0, b) for p, b in zip(presorted, big))        # all of a generation's large groups, or none
     assert any(b > 0 and p == 0 for p, b in zip(presorted, big))   # and some generation did sort its large groups
+    # A generation that follows one whose large groups were all in order gathers without the pairs of the radix sort, and
+    # once more with them if its own large groups are not in order: with every generation starting that way, the ones that
+    # do sort take the second gather, and nothing else changes
+    got2, active2, big2 = emu_sort(emu, T, 1, pack=False, expect_presorted=True)
+    assert np.array_equal(got2, got) and (active2, big2, emu_sort.presorted) == (active, big, presorted)
 
 
 def test_small_and_large_groups_take_both_paths(emu):

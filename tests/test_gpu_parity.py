@@ -360,6 +360,34 @@ def test_four_letters_start_from_keys_of_32_symbols(torch_mod, key_words, exclus
     assert small_stats["first_sort_generations"] == first
 
 
+def test_generations_that_expect_their_large_groups_in_order(torch_mod):
+    """A generation that follows one whose large groups were all in order leaves out the pairs of the radix sort when it
+    gathers, and gathers once more with them if its own large groups turn out not to be in order. With
+    CSA_TUNE_EXPECT_PRESORTED every generation starts that way: on the adversarial workload (runs and periods, whose late
+    generations are in order, after early ones that are not) and on the token workload (never in order) the suffix arrays
+    and the statistics must be those of the default."""
+    from cascade_amd import PartitionSorter, workloads, _native
+    n = 1 << 22
+    for config in (5, 3):
+        T = workloads.generate(config, n)
+        d = to_dev(torch_mod, T)
+        with PartitionSorter(n, key_words=1) as s:
+            print(f"  expect-presorted config={config} n={n}", flush=True)
+            out = s.sort(d)
+            plain = s.last_stats
+            s.set_tuning(_native.CSA_TUNE_EXPECT_PRESORTED, 1)
+            out2 = s.sort(d)
+            forced = s.last_stats
+            assert torch_mod.equal(out, out2)
+            got = out.cpu().numpy()
+        assert oracle_lib.is_correct_sa40(got, T)
+        for key in ("active", "groups", "big", "presorted", "passes"):
+            assert plain[key] == forced[key], (config, key)
+        assert any(b > 0 and p == 0 for b, p in zip(plain["big"], plain["presorted"]))  # some generation sorted its large groups
+        if config == 5:
+            assert any(p > 0 for p in plain["presorted"])
+
+
 def test_byte_texts_start_from_keys_of_8_symbols(torch_mod):
     """A text of byte values (every value 0..255 occurs): codes of 8 bits, 8 symbols in the first key, which covers
     generations 0-1 of one-word keys. A million symbols with long repeats and a tail of zeros, against the oracle."""
