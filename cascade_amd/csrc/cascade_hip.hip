@@ -1066,18 +1066,31 @@ int sort_partition(Launch& L, const u16* d_text, u64 n64, u64 index_base, u8* d_
         // retired are alone with their rank: they sort to the place they hold already and keep their rank.
         const bool dense = dense_generation(m_in, groups, n);
         if (dense) {
-            // The generation before knew this one would be dense (the same test on the same numbers) and left ordinals in
-            // rank[]: the key runs of its sorted list numbered 0, 1, 2, ...; there are as many as it had groups and
-            // singletons. Two ordinals make a key of 2 log2(runs) bits: 17 bits after generation 0 of a four-letter
-            // text (256 groups and the last four suffixes), three passes where two 31-bit ranks take eight.
-            if (!ordinals_in_rank)
-                return fail(CSA_ERR_INTERNAL, "generation %d is dense but the one before it left ranks, not ordinals", gen);
-            const u64 runs = (u64)groups + ((u64)n - m_in);
-            const u32 radix = (u32)runs;
-            const PassPlan plan = make_plan(0, runs > 1 ? bit_length(runs * runs - 1) : 1);
+            // A generation that runs in this form itself, or generation 0, knew that this one would be dense (the same test on
+            // the same numbers) and left ordinals in rank[]: the key runs of its sorted list numbered 0, 1, 2, ...; there
+            // are as many as it had groups and singletons. Two ordinals make a key of 2 log2(runs) bits: 17 bits after
+            // generation 0 of a four-letter text (256 groups and the last four suffixes), three passes where two 31-bit ranks
+            // take eight. A generation of the other form leaves ranks, and the list it leaves can still qualify (its many
+            // short groups dissolved, a few long ones are left): the key is then the two ranks side by side.
             passes = 0;
-            rc = radix_sort(L, SRC_RANKS, nullptr, n, 0, 0, bkey[0], bx[0], bkey[1], bx[1], n, plan, &in_out, &passes, h->rank, (u32)hop,
-                            radix);
+            if (ordinals_in_rank) {
+                const u64 runs = (u64)groups + ((u64)n - m_in);
+                const u32 radix = (u32)runs;
+                const PassPlan plan = make_plan(0, runs > 1 ? bit_length(runs * runs - 1) : 1);
+                rc = radix_sort(L, SRC_RANKS, nullptr, n, 0, 0, bkey[0], bx[0], bkey[1], bx[1], n, plan, &in_out, &passes, h->rank,
+                                (u32)hop, radix);
+            } else {
+                PassPlan plan; // the digits of the two ranks of a key: bits [0, sec_bits) and [32, 32 + sec_bits)
+                plan.num_passes = 0;
+                for (int half = 0; half < 2; ++half)
+                    for (int b = 0; b < sec_bits; b += RADIX_BITS) {
+                        plan.shift[plan.num_passes] = 32 * half + b;
+                        plan.bits[plan.num_passes] = sec_bits - b < RADIX_BITS ? sec_bits - b : RADIX_BITS;
+                        plan.num_passes++;
+                    }
+                rc = radix_sort(L, SRC_RANKS, nullptr, n, 0, 0, bkey[0], bx[0], bkey[1], bx[1], n, plan, &in_out, &passes, h->rank,
+                                (u32)hop, 0u);
+            }
             if (rc)
                 return rc;
             RerankArgs rd;

@@ -185,6 +185,19 @@ def test_dense_generations_sort_the_whole_partition_again(emu, name, key_words):
     assert all(u == 1 for u, d in zip(emu_sort.rank_update, emu_sort.dense) if d)
 
 
+def test_a_dense_generation_after_one_that_was_not(emu):
+    """A long run of one token and a stretch whose K-grams collide in pairs: generation 1 holds the run's one long group and
+    a couple of hundred pairs (short groups on average: the gather form, which leaves ranks in rank[]); the pairs dissolve
+    there, and generation 2 is left with the long group alone and takes the dense form, on keys of two ranks side by side
+    (a generation 0 or a dense generation before it would have left run ordinals instead)."""
+    rng = np.random.default_rng(3)
+    T = np.concatenate([rng.integers(1, 7, 350), np.full(1400, 9), rng.integers(1, 7, 350)]).astype(np.uint16)
+    got, active, _ = emu_sort(emu, T, 1, pack=False)
+    sa, counts = oracle_lib.prefix_doubling(T, 1)
+    assert np.array_equal(got, oracle_lib.u64_to_sa40(sa)) and active == counts
+    assert emu_sort.dense[:3] == [0, 0, 1], emu_sort.dense
+
+
 PACKED_CASES = {
     "four_letters": (np.arange(4), 1, 32, 4),                    # codes of 2 bits
     "one_letter": (np.array([7]), 1, 64, 5),                     # with the padding's zero: 2 codes, 1 bit

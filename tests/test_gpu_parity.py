@@ -360,6 +360,23 @@ def test_four_letters_start_from_keys_of_32_symbols(torch_mod, key_words, exclus
     assert small_stats["first_sort_generations"] == first
 
 
+def test_a_dense_generation_after_one_that_was_not(torch_mod):
+    """A run of 110 000 equal tokens between two stretches whose K-grams collide in some 1500 pairs: generation 1 (one long
+    group, many pairs: short groups on average) gathers and leaves ranks in rank[]; the pairs dissolve, generation 2 holds
+    the long group alone and sorts the whole partition again from keys of two ranks side by side (after a generation 0 or a
+    dense generation it would find run ordinals there). Against the oracle, generation sizes included."""
+    from cascade_amd import PartitionSorter, _native
+    rng = np.random.default_rng(12)
+    T = np.concatenate([rng.integers(1, 31, 25000), np.full(110000, 77), rng.integers(1, 31, 25000)]).astype(np.uint16)
+    with PartitionSorter(T.size, key_words=1) as s:
+        s.set_tuning(_native.CSA_TUNE_PACK_SYMBOLS, 0)
+        got = s.sort(to_dev(torch_mod, T)).cpu().numpy()
+        stats = s.last_stats
+    sa, counts = oracle_lib.prefix_doubling(T, 1)
+    assert np.array_equal(got, oracle_lib.u64_to_sa40(sa)) and stats["active"] == counts
+    assert stats["dense"][:3] == [0, 0, 1], stats["dense"]
+
+
 def test_generations_that_expect_their_large_groups_in_order(torch_mod):
     """A generation that follows one whose large groups were all in order leaves out the pairs of the radix sort when it
     gathers, and gathers once more with them if its own large groups turn out not to be in order. With
