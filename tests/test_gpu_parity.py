@@ -449,6 +449,68 @@ def test_random_small_texts_against_the_oracle(torch_mod):
         assert np.array_equal(got, oracle_lib.build_sa40(T)), (case, n, sigma, kw)
 
 
+def test_random_alphabets_structures_and_paths_against_the_oracle(torch_mod):
+    """600 random texts: alphabets that pack into 1, 2, 4 or 8 bits, that pack through their byte ranks, that do not pack;
+    repeats, runs, periodic stretches and zero tails laid over them; all four key widths; and, at random, the knobs that
+    force the other paths (one K-gram word in the first sort, every generation expecting its large groups in order, the
+    bucketed rank updates). Suffix array and generation sizes against the oracle's doubling. (A run of this generator over
+    some 350 000 texts found the one dense-after-gather case that test_a_dense_generation_after_one_that_was_not pins.)"""
+    from cascade_amd import PartitionSorter, _native
+    rng = np.random.default_rng(31)
+    for case in range(600):
+        n = max(1, int(rng.choice([1, 2, 3, 5, 17, 63, 64, 65, 255, 1000, 4097, 20000])) + int(rng.integers(-3, 4)))
+        kind = int(rng.integers(0, 7))
+        if kind == 0:
+            alphabet = np.arange(int(rng.integers(1, 5)))
+        elif kind == 1:
+            alphabet = rng.choice(np.arange(0, 256), size=int(rng.integers(1, 200)), replace=False)
+        elif kind == 2:
+            lo = rng.choice(np.arange(0, 256), size=int(rng.integers(1, 12)), replace=False)
+            hi = rng.choice(np.arange(0, 256), size=int(rng.integers(1, 12)), replace=False)
+            alphabet = (hi[:, None] * 256 + lo[None, :]).ravel()
+        elif kind == 3:
+            alphabet = rng.choice(np.arange(0, 65536), size=int(rng.integers(2, 3000)), replace=False)
+        elif kind == 4:
+            alphabet = np.array([65, 67, 71, 84])
+        elif kind == 5:
+            alphabet = np.array([int(rng.integers(0, 65536))])
+        else:
+            alphabet = np.arange(256)
+        T = alphabet.astype(np.uint16)[rng.integers(0, alphabet.size, n)]
+        for _ in range(int(rng.integers(0, 4))):
+            if n < 8:
+                break
+            a, length = int(rng.integers(0, n - 4)), int(rng.integers(1, max(2, n // 3)))
+            what = int(rng.integers(0, 4))
+            if what == 0:
+                b = int(rng.integers(0, n - 4))
+                length = min(length, n - max(a, b))
+                T[b:b + length] = T[a:a + length].copy()
+            elif what == 1:
+                T[a:a + length] = T[a]
+            elif what == 2:
+                length = min(length, n - a)
+                T[a:a + length] = np.resize(T[a:a + int(rng.integers(2, 9))].copy(), length)
+            else:
+                T[-min(n, int(rng.integers(1, 70))):] = 0
+        kw = int(rng.integers(1, 5))
+        knobs = [int(rng.integers(0, 3)) == 0 for _ in range(3)]
+        with PartitionSorter(n, key_words=kw) as s:
+            if knobs[0]:
+                s.set_tuning(_native.CSA_TUNE_PACK_SYMBOLS, 0)
+            if knobs[1]:
+                s.set_tuning(_native.CSA_TUNE_EXPECT_PRESORTED, 1)
+            if knobs[2]:
+                s.set_tuning(_native.CSA_TUNE_DEFER_MIN, 1)
+                s.set_tuning(_native.CSA_TUNE_WINDOW_MIN_CHANGED, 1)
+            if case % 100 == 0:
+                print(f"  random text case={case} n={n} alphabet kind={kind} key_words={kw} knobs={knobs}", flush=True)
+            got = s.sort(to_dev(torch_mod, T)).cpu().numpy()
+            stats = s.last_stats
+        sa, counts = oracle_lib.prefix_doubling(T, kw)
+        assert np.array_equal(got, oracle_lib.u64_to_sa40(sa)) and stats["active"] == counts, (case, n, kind, kw, knobs)
+
+
 def test_bucketed_rank_updates_at_small_and_ragged_sizes(torch_mod):
     """The bucketed rank updates normally serve lists of millions of suffixes: generation 0 sends (position, rank)
     records through value-less radix passes and a window placement, later generations (position, rank) pairs through one
