@@ -593,6 +593,31 @@ def test_three_dispatcher_threads_with_their_own_handles_and_streams(torch_mod):
     assert not errors, errors
 
 
+def test_the_references_own_tool_accepts_the_command_line_builders_file(tmp_path):
+    """tools/sa_convert.cpp of the reference, compiled from its one source file into oracle/_ref (oracle/Makefile), is
+    what the reference runs on a finished 40-bit suffix array: the file cascade_sa writes passes its size checks and
+    its spot check of the order (100 000 adjacent pairs, the reference's comparator), gets an index.meta, and widens,
+    through the reference's own sa40 loader, to the oracle's 64-bit array."""
+    import os
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    tool, exe = os.path.join(root, "oracle", "_ref", "sa_convert"), os.path.join(root, "cascade_amd", "cascade_sa")
+    if not os.path.exists(tool):
+        pytest.skip("oracle/_ref/sa_convert is not built (make -C oracle where the reference tree is present)")
+    T = texts.random_text(300000, 50257, 8, sep_every=900)
+    T[200000:260000] = T[1000:61000]
+    ip, op = tmp_path / "t.u16", tmp_path / "t.sa40"
+    T.astype("<u2").tofile(ip)
+    r = subprocess.run([exe, str(ip), str(op)], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0, r.stderr
+    r = subprocess.run([tool, "--meta-only", "--sa", str(op), "--text", str(ip), "--sym-bytes", "2", "--index-dir", str(tmp_path / "index")],
+                       capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0 and "spot-check passed" in r.stderr and (tmp_path / "index" / "index.meta").exists(), r.stderr
+    r = subprocess.run([tool, "--widen", "--in", str(op), "--out", str(tmp_path / "t.u64")], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0, r.stderr
+    assert np.array_equal(np.fromfile(tmp_path / "t.u64", dtype="<u8"), oracle_lib.sa40_to_u64(oracle_lib.build_sa40(T)))
+
+
 def test_command_line_builder_writes_the_oracles_suffix_array(tmp_path):
     """cascade_amd/cascade_sa <text-file> <suffix-array-file>: the reference's program (src/main.cu:12-46) through the
     C++ mirror of its builder class; the file it writes is the oracle's, byte for byte; a missing input ends it with
@@ -611,3 +636,4 @@ def test_command_line_builder_writes_the_oracles_suffix_array(tmp_path):
             assert np.array_equal(np.fromfile(op, dtype=np.uint8), oracle_lib.build_sa40(T)), (name, key_words)
     r = subprocess.run([exe, str(tmp_path / "missing.u16"), str(tmp_path / "x.sa40")], capture_output=True, text=True, timeout=100)
     assert r.returncode == 1 and "cannot open" in r.stderr
+

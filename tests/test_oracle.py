@@ -223,3 +223,40 @@ def test_stable_sort_pairs_contract():
     k, v = oracle_lib.stable_sort_pairs(keys, vals, 7, 15)  # a sub-range of the bits only
     order = np.argsort((keys >> np.uint64(7)) & np.uint64(0xFF), kind="stable")
     assert np.array_equal(k, keys[order]) and np.array_equal(v, vals[order])
+
+
+SA_CONVERT = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle", "_ref", "sa_convert")
+
+
+@pytest.mark.skipif(not os.path.exists(SA_CONVERT), reason="oracle/_ref/sa_convert is not built (make -C oracle, with the reference tree present)")
+def test_the_references_own_tool_accepts_and_widens_the_oracles_suffix_array_file(tmp_path):
+    """The reference's tools/sa_convert.cpp, compiled from its one source file (oracle/Makefile): `--meta-only` is what the
+    reference runs on a finished 40-bit suffix array (file of 5 n bytes beside a text of n symbols, a spot check of the
+    order of adjacent entries with its own comparator, index.meta), `--widen` reads the 5-byte entries with its own
+    sa40 loader. The oracle's file must pass the first and widen to the oracle's 64-bit array; a file with two entries
+    swapped, and one that is an entry short, must be refused. Pins the on-disk layout of the output row."""
+    import subprocess
+    for name, T in (("tokens", texts.random_text(30000, 50257, 3, sep_every=700)), ("ties", texts.random_text(5000, 2, 4, sep_every=0))):
+        text, sa = tmp_path / f"{name}.u16", tmp_path / f"{name}.u40"
+        T.astype("<u2").tofile(text)
+        sa40 = oracle_lib.build_sa40(T)
+        sa40.tofile(sa)
+        idx = tmp_path / f"{name}.index"
+        r = subprocess.run([SA_CONVERT, "--meta-only", "--sa", str(sa), "--text", str(text), "--sym-bytes", "2", "--index-dir", str(idx)],
+                           capture_output=True, text=True, timeout=120)
+        assert r.returncode == 0 and "spot-check passed" in r.stderr, r.stderr
+        assert (idx / "index.meta").exists()
+        wide = tmp_path / f"{name}.u64"
+        r = subprocess.run([SA_CONVERT, "--widen", "--in", str(sa), "--out", str(wide)], capture_output=True, text=True, timeout=120)
+        assert r.returncode == 0, r.stderr
+        assert np.array_equal(np.fromfile(wide, dtype="<u8"), oracle_lib.sa40_to_u64(sa40))
+        bad = sa40.copy()
+        bad[5 * 100:5 * 101], bad[5 * 101:5 * 102] = sa40[5 * 101:5 * 102].copy(), sa40[5 * 100:5 * 101].copy()
+        bad.tofile(sa)
+        r = subprocess.run([SA_CONVERT, "--meta-only", "--sa", str(sa), "--text", str(text), "--sym-bytes", "2", "--index-dir", str(idx)],
+                           capture_output=True, text=True, timeout=120)
+        assert r.returncode != 0, "two swapped entries passed the order check"
+        sa40[:-5].tofile(sa)
+        r = subprocess.run([SA_CONVERT, "--meta-only", "--sa", str(sa), "--text", str(text), "--sym-bytes", "2", "--index-dir", str(idx)],
+                           capture_output=True, text=True, timeout=120)
+        assert r.returncode != 0, "a file one entry short passed"
