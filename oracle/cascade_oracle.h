@@ -20,8 +20,14 @@
  *   orc_fwd_tag : closed form, and the tail-order property it exists for.
  *   orc_prefix_doubling_u16 : final order equals orc_build_sa40_u16 on every fixture;
  *       per-generation active counts equal orc_retire_generations (an independent
- *       closed form over SA + LCP, src/sa_structure.cpp:295-306,375).
- *   orc_sa40_store / orc_sa40_load : round trip (src/test_query.cu:78-96) and explicit bytes.
+ *       closed form over SA + LCP, src/sa_structure.cpp:295-306,375) and, where the
+ *       reference tree is present, the retirements that the reference's own
+ *       src/sa_structure.cpp, compiled into _ref/sa_structure, predicts from the finished
+ *       array, for key widths of 1 to 4 words.
+ *   orc_sa40_store / orc_sa40_load : round trip (src/test_query.cu:78-96) and explicit bytes;
+ *       the file of orc_build_sa40_u16 passes the reference's own tools/sa_convert.cpp
+ *       (compiled into _ref/sa_convert: sizes, order spot check, index.meta) and widens
+ *       through it to the 64-bit array.
  */
 #ifndef CASCADE_ORACLE_H
 #define CASCADE_ORACLE_H

@@ -140,7 +140,8 @@ def build_sa(lib, to_dev, to_host, T, p, key_words=1, pivot_words=2, seed=0, max
     permutation goes through csa_scatter_slabs with the output cut into disk blocks.
     step_handle / slab_handle may also be a function: it is called with the largest partition's size once that is known
     and returns the handle (a handle of exactly that capacity is the tightest the floor plan allows); build_sa destroys it.
-    build_sa.high_water then holds the most bytes any step of the run kept alive in the handle's block."""
+    build_sa.high_water then holds the most bytes any step of the run kept alive in the handle's block, and
+    build_sa.pill_receipts the pill receipts the library counted in every step (csa_step_result.pills)."""
     T = np.ascontiguousarray(T, dtype=np.uint16)
     n, ell = T.size, 4 * key_words
     rng = np.random.default_rng(seed)
@@ -166,6 +167,7 @@ def build_sa(lib, to_dev, to_host, T, p, key_words=1, pivot_words=2, seed=0, max
         slab_handle = slab_handle(max(int(psz.max()), 1))
         own_handles.append(slab_handle)
     build_sa.high_water = 0
+    build_sa.pill_receipts = []  # (generation, partition, cohort members that a poison pill joined) of the library's steps
     try:
         return _build_sa(lib, to_dev, to_host, T, p, key_words, seed, max_generations, log, join_handle, step_handle, slab_handle,
                          host_buf, chunk_cap, n, ell, rng, d_T, pid, words, psz, P_off, bits)
@@ -245,6 +247,7 @@ def _build_sa(lib, to_dev, to_host, T, p, key_words, seed, max_generations, log,
                 sr = _native.CsaStepResult()
                 assert lib.csa_last_step_result(slab_handle, C.byref(sr)) == 0
                 assert sr.unserved == 0 and sr.incoherent_pills == 0, (gen, q, int(sr.unserved), int(sr.incoherent_pills))
+                build_sa.pill_receipts.append((gen, q, int(sr.pills)))
                 a_new, total = int(active_slot.value), int(end[p - 1])
                 assert (int(sr.active), int(sr.messages)) == (a_new, total)
                 new_suf, new_rank = np.zeros(a, dtype=np.uint64), np.zeros(a, dtype=np.uint32)
@@ -292,6 +295,7 @@ def _build_sa(lib, to_dev, to_host, T, p, key_words, seed, max_generations, log,
                 _note_high_water(lib, step_handle)
                 # what the reference checks under -DTESTS (src/GPU_SACA.cu:2055-2063, include/GPU_SACA.cuh:246-249)
                 assert res.unserved == 0 and res.incoherent_pills == 0, (gen, q, int(res.unserved), int(res.incoherent_pills))
+                build_sa.pill_receipts.append((gen, q, int(res.pills)))
                 a_new, total = int(res.active), int(res.messages)
                 end = to_host(d_off)
                 assert total == int(end[p - 1])
@@ -436,3 +440,23 @@ def lib_handle(lib):
     h = C.c_void_p()
     assert lib.csa_create(16, 1, C.byref(h)) == 0
     return h
+
+
+def structure_of_a_pipeline_run(T, p, key_words, pivot_words, seed, log, receipts, workdir):
+    """Per generation, summed over the partitions: what a multi_partition.build_sa run through the library's steps had
+    (cohort members, messages emitted, pill receipts) beside what the reference's own predictor (src/sa_structure.cpp
+    compiled into oracle/_ref) gives for that text, key width, pivot width and partition sizes: active-set sizes, the
+    messages before any is withheld from a retired recipient (payloads + forwarded pills), and the queries whose target had
+    retired before (look-back of one generation or more: the answer is a pill). Returns two dicts of lists."""
+    pivots = oracle_lib.sample_pivots(T, p, pivot_words, np.random.default_rng(seed))  # as build_sa draws them
+    _, psz = oracle_lib.partition_ids(T, pivots, p, pivot_words)
+    # (the tool refuses empty partitions, which a run of the reference never has; they neither hold nor receive anything)
+    got = oracle_lib.reference_structure(T, oracle_lib.build_sa40(T), 4 * key_words, 4 * pivot_words, psz[psz > 0], workdir)
+    gens = 1 + max(step[0] for step in log)
+    ours = {"cohorts": [sum(step[2] for step in log if step[0] == g) for g in range(gens)],
+            "messages": [sum(step[4] for step in log if step[0] == g) for g in range(gens)],
+            "pill_receipts": [sum(r[2] for r in receipts if r[0] == g) for g in range(gens)]}
+    cohorts = oracle_lib.active_sizes_from_retirements(T.size, got["retire_hist"])
+    theirs = {"cohorts": cohorts, "messages": [a + b for a, b in zip(got["payloads"], got["forwards"])][:len(cohorts)],
+              "pill_receipts": [sum(row[1:]) for row in got["lookback"]][:len(cohorts)]}
+    return ours, theirs

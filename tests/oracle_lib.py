@@ -323,3 +323,40 @@ def join_messages(msg_target, msg_rank, sa, primary, keys):
     keys = np.array(keys, dtype=np.uint64, copy=True)
     oracle().orc_join_messages(_ptr(lanes), _ptr(msg_rank), msg_rank.size, _ptr(sa), _ptr(primary), _ptr(keys), sa.size)
     return keys
+
+
+SA_STRUCTURE = os.path.join(ORACLE_DIR, "_ref", "sa_structure")
+
+
+def reference_structure(T, sa40, ell, K, partition_sizes, workdir):
+    """What the reference's own src/sa_structure.cpp (compiled from its source into oracle/_ref/sa_structure) predicts for a
+    run over the text T with the finished suffix array sa40 (5-byte entries), generation-0 keys of ell symbols, pivots of K
+    symbols (0 < K <= ell) and the given partition sizes: a dict with retire_hist[d] (suffixes that retire at generation d),
+    payloads[t] and forwards[t] (messages and forwarded pills emitted at generation t) and the rest of its JSON. The tool
+    also checks that the array is a permutation in suffix order. None if the tool is not built."""
+    import json
+    if not os.path.exists(SA_STRUCTURE):
+        return None
+    workdir = str(workdir)
+    text, sa, log, out = (os.path.join(workdir, f) for f in ("structure_text.u16", "structure_sa.u40", "structure_run.log", "structure.json"))
+    _text(T).astype("<u2").tofile(text)
+    np.ascontiguousarray(sa40, dtype=np.uint8)[:5 * _text(T).size].tofile(sa)
+    with open(log, "w") as f:  # the two lines of a STATS build that the tool reads (src/sa_structure.cpp:78-112)
+        f.write(f"Pivots selection: {len(partition_sizes)} partitions from 0 samples of {int(K)}-symbol prefixes; initial sort-keys of {int(ell)} symbols.\n")
+        f.write("Partition sizes: " + " ".join(str(int(x)) for x in partition_sizes) + "\n")
+    run = subprocess.run([SA_STRUCTURE, text, sa, log, out], capture_output=True, text=True, timeout=600)
+    assert run.returncode == 0, run.stderr[-2000:]
+    with open(out) as f:
+        return json.load(f)
+
+
+def active_sizes_from_retirements(n, retire_hist):
+    """Active-set size entering every generation 0, 1, ... from the retirements per generation, trailing empty ones cut."""
+    sizes, left = [], int(n)
+    for r in retire_hist:
+        sizes.append(left)
+        left -= int(r)
+    assert left == 0
+    while sizes and sizes[-1] == 0:
+        sizes.pop()
+    return sizes

@@ -402,6 +402,30 @@ def test_multi_partition_pipeline_with_the_emulated_step_entries(emu, p, key_wor
     assert log == glue_log
 
 
+@pytest.mark.skipif(not os.path.exists(oracle_lib.SA_STRUCTURE), reason="oracle/_ref/sa_structure is not built (make -C oracle, with the reference tree present)")
+@pytest.mark.parametrize("p,key_words,pivot_words", [(4, 1, 1), (5, 2, 2), (3, 4, 2)])
+def test_the_references_own_predictor_gives_the_cohorts_and_pill_receipts_of_the_steps(emu, tmp_path, p, key_words, pivot_words):
+    """The reference's src/sa_structure.cpp predicts a run from the finished suffix array, the key and pivot widths and the
+    partition sizes: every generation's active-set size, every query's look-back (how long ago its target retired), and the
+    messages emitted before any is withheld from a recipient that is flagged retired. The partition steps of the library
+    (one csa_sort_init_dev / csa_sort_rerank_dev call each, on the emulated kernels) must have had exactly those cohorts
+    and exactly that many members joined by a pill (csa_step_result.pills, counted on the device), summed over the
+    partitions; they emit that many messages in generation 0, when nothing is flagged yet, and never more later."""
+    import multi_partition
+    T = texts.random_text(800, 2, 17 * p, sep_every=0)
+    T[300:520] = T[20:240]
+    T[-6:] = 0
+    log = []
+    sa, _ = multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, p, key_words=key_words,
+                                     pivot_words=pivot_words, seed=p, log=log, step_handle=steps_handle(emu, key_words))
+    assert np.array_equal(sa, oracle_lib.sa40_to_u64(oracle_lib.build_sa40(T)))
+    ours, theirs = multi_partition.structure_of_a_pipeline_run(T, p, key_words, pivot_words, p, log, multi_partition.build_sa.pill_receipts, tmp_path)
+    assert ours["cohorts"] == theirs["cohorts"], (ours, theirs)
+    assert ours["pill_receipts"] == theirs["pill_receipts"], (ours, theirs)
+    assert ours["messages"][0] == theirs["messages"][0] and all(a <= b for a, b in zip(ours["messages"], theirs["messages"])), (ours, theirs)
+    assert len(ours["cohorts"]) >= 4 and sum(ours["pill_receipts"]) > 0
+
+
 @pytest.mark.parametrize("p,key_words,sigma,n,chunk_cap", [(3, 1, 3, 900, 4096)])
 def test_multi_partition_pipeline_through_the_emulated_slab_entries(emu, p, key_words, sigma, n, chunk_cap):
     """csa_sort_init_slabs / csa_sort_rerank_slabs / csa_scatter_slabs: every partition step takes and returns host slabs of

@@ -175,6 +175,38 @@ def test_step_entries_on_hard_shapes(gpu, shape, p):
         assert np.array_equal(sa, np.arange(n - 1, -1, -1, dtype=np.uint64))
 
 
+@pytest.mark.parametrize("p,key_words,pivot_words,slabs", [(16, 1, 1, False), (7, 2, 2, True), (40, 4, 2, False)])
+def test_the_references_own_predictor_gives_the_cohorts_and_pill_receipts_of_the_steps(gpu, tmp_path, p, key_words, pivot_words, slabs):
+    """The reference's src/sa_structure.cpp (compiled from its one source file into oracle/_ref) predicts a run from the
+    finished suffix array, the key and pivot widths and the partition sizes: every generation's active-set size, every
+    query's look-back, the messages before any is withheld from a retired recipient. 150 000 symbols with long repeats in
+    7 to 40 partitions through the device and the slab entries: the steps must have had exactly those cohorts and exactly
+    that many members joined by a pill (csa_step_result.pills), summed over the partitions, and emit that many messages in
+    generation 0 and never more later."""
+    import os
+    if not os.path.exists(oracle_lib.SA_STRUCTURE):
+        pytest.skip("oracle/_ref/sa_structure is not built (make -C oracle where the reference tree is present)")
+    lib, to_dev, to_host = gpu
+    rng = np.random.default_rng(p)
+    T = rng.integers(0, 5, 150000).astype(np.uint16)
+    T[90000:130000] = T[10000:50000]
+    T[140000:141000] = T[0]
+    T[-11:] = 0
+    log = []
+    kw = {"slab_handle": steps_handle(lib, key_words), "host_buf": pinned_host_buf, "chunk_cap": 8192} if slabs else {
+        "step_handle": steps_handle(lib, key_words)}
+    print(f"  pipeline against sa_structure p={p} key_words={key_words} pivot_words={pivot_words} slabs={slabs}", flush=True)
+    sa, _ = multi_partition.build_sa(lib, to_dev, to_host, T, p, key_words=key_words, pivot_words=pivot_words, seed=p, log=log, **kw)
+    want, _ = oracle_lib.prefix_doubling(T, 1)
+    assert np.array_equal(sa, want)
+    ours, theirs = multi_partition.structure_of_a_pipeline_run(T, p, key_words, pivot_words, p, log, multi_partition.build_sa.pill_receipts,
+                                                               tmp_path)
+    assert ours["cohorts"] == theirs["cohorts"], (ours, theirs)
+    assert ours["pill_receipts"] == theirs["pill_receipts"], (ours, theirs)
+    assert ours["messages"][0] == theirs["messages"][0] and all(a <= b for a, b in zip(ours["messages"], theirs["messages"]))
+    assert len(ours["cohorts"]) >= 10 and sum(ours["pill_receipts"]) > 0
+
+
 def test_random_pipelines_through_the_step_entries(gpu):
     """Random texts (tiny alphabets, long repeats, zero tails), 1 to 200 partitions, all four key widths: every step
     passes the reference's validators inside the harness and the suffix array is the oracle's."""

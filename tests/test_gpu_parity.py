@@ -593,6 +593,27 @@ def test_three_dispatcher_threads_with_their_own_handles_and_streams(torch_mod):
     assert not errors, errors
 
 
+@pytest.mark.parametrize("config,key_words", [(3, 1), (3, 4), (2, 2), (4, 1)])
+def test_generation_sizes_are_those_the_references_own_predictor_gives(torch_mod, tmp_path, config, key_words):
+    """src/sa_structure.cpp of the reference (compiled from its one source file into oracle/_ref) predicts, from a finished
+    suffix array, how many suffixes retire at every generation of a run, and verifies the array while it reads it. Two
+    million symbols of the token workloads and of the four-letter workload (whose first sort takes keys of 32 packed
+    symbols and stands for several generations): the sizes the library reports for every generation, the covered ones
+    included, must be the predictor's, and its file must pass the tool's own order and permutation checks."""
+    from cascade_amd import PartitionSorter, workloads
+    if not os.path.exists(oracle_lib.SA_STRUCTURE):
+        pytest.skip("oracle/_ref/sa_structure is not built (make -C oracle where the reference tree is present)")
+    n = 1 << 21
+    T = workloads.generate(config, n)
+    with PartitionSorter(n, key_words=key_words) as s:
+        print(f"  sort against sa_structure config={config} key_words={key_words}", flush=True)
+        got = s.sort(to_dev(torch_mod, T)).cpu().numpy()
+        stats = s.last_stats
+    ell = 4 * key_words
+    theirs = oracle_lib.reference_structure(T, got, ell, ell, [n], tmp_path)
+    assert oracle_lib.active_sizes_from_retirements(n, theirs["retire_hist"]) == stats["active"], (stats["active"], theirs["retire_hist"])
+
+
 def test_the_references_own_tool_accepts_the_command_line_builders_file(tmp_path):
     """tools/sa_convert.cpp of the reference, compiled from its one source file into oracle/_ref (oracle/Makefile), is
     what the reference runs on a finished 40-bit suffix array: the file cascade_sa writes passes its size checks and

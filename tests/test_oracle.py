@@ -260,3 +260,26 @@ def test_the_references_own_tool_accepts_and_widens_the_oracles_suffix_array_fil
         r = subprocess.run([SA_CONVERT, "--meta-only", "--sa", str(sa), "--text", str(text), "--sym-bytes", "2", "--index-dir", str(idx)],
                            capture_output=True, text=True, timeout=120)
         assert r.returncode != 0, "a file one entry short passed"
+
+
+@pytest.mark.skipif(not os.path.exists(oracle_lib.SA_STRUCTURE), reason="oracle/_ref/sa_structure is not built (make -C oracle, with the reference tree present)")
+@pytest.mark.parametrize("key_words", [1, 2, 3, 4])
+def test_generation_sizes_are_those_the_references_own_predictor_gives(tmp_path, key_words):
+    """The reference's src/sa_structure.cpp, compiled from its one source file (oracle/Makefile), predicts from a finished
+    suffix array how many suffixes retire at every generation of a run (and checks the array on the way). The oracle's
+    prefix doubling must report exactly those active-set sizes, for every key width, on texts with deep repeats, runs and
+    a tail of zeros. Pins orc_prefix_doubling's per-generation counts on the reference's code instead of on the
+    restatement of its rule (orc_retire_generations)."""
+    ell = 4 * key_words
+    rng = np.random.default_rng(key_words)
+    cases = {"tokens": texts.random_text(20000, 50257, 3, sep_every=500), "ties": texts.random_text(20000, 3, 5, sep_every=0),
+             "run": np.concatenate([texts.random_text(3000, 4, 6, sep_every=0), np.full(5000, 2, dtype=np.uint16),
+                                    texts.random_text(3000, 4, 7, sep_every=0)]).astype(np.uint16)}
+    cases["tokens"][12000:18000] = cases["tokens"][1000:7000]
+    cases["ties"][15000:19000] = cases["ties"][2000:6000]
+    cases["ties"][-9:] = 0
+    for name, T in cases.items():
+        sa, counts = oracle_lib.prefix_doubling(T, key_words)
+        got = oracle_lib.reference_structure(T, oracle_lib.u64_to_sa40(sa), ell, ell, [T.size], tmp_path)
+        assert got["n"] == T.size and got["ell"] == ell
+        assert oracle_lib.active_sizes_from_retirements(T.size, got["retire_hist"]) == counts, name
