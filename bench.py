@@ -435,9 +435,9 @@ def bench_next_rows(args):
                                                                  C.byref(res)))
             ms, _ = _timed(torch, rer, args.steps, args.warmup)
             ok = int(res.active) <= a
-            alg = a * (5 * 2 * 24 + 29 + 8 * 2 * 24 + 90 + 9)  # suffix-order sort, join, key sort, re-rank, narrow (src/GPU_SACA.cu:1769-1995)
+            alg = a * (5 * 2 * 24 + 29 + 8 * 2 * 24 + 90 + 9)  # the reference's plan: suffix-order sort, join, key sort, re-rank, narrow (src/GPU_SACA.cu:1769-1995)
             res_row = _row_result("active suffixes through a later partition step/sec at 1 GPU", workloads.NAMES[args.config], a, ms,
-                                  "csa_sort_rerank_dev (13 radix passes + join + glue)", alg,
+                                  "csa_sort_rerank_dev (the reference: 13 radix passes + join + glue; here 8 passes and a hash join)", alg,
                                   {"partitions": p, "inbox": total, "active_after": int(res.active)}, args.steps, args.warmup, ok)
         sorter.close()
         res = res_row

@@ -617,9 +617,10 @@ int read_counts(Launch& L, u32* big)
                                            "an active suffix lies outside its group's range (small-group sort)",
                                            "a large-group member was sent outside the active list (place)",
                                            "a rank or suffix index out of range in the sorted active list (rerank)",
-                                           "a large group appeared in a list whose groups were all small"};
+                                           "a large group appeared in a list whose groups were all small",
+                                           "the join table of a partition step has more members than slots"};
         const u32 code = h->h_pinned[2];
-        return fail(CSA_ERR_INTERNAL, "device invariant %u failed: %s", code, code < 6 ? what[code] : "unknown");
+        return fail(CSA_ERR_INTERNAL, "device invariant %u failed: %s", code, code < 7 ? what[code] : "unknown");
     }
     if (big)
         *big = h->h_pinned[4];

@@ -21,6 +21,7 @@ constexpr unsigned DEV_ERR_SMALLSORT_TABLES = 2;
 constexpr unsigned DEV_ERR_PLACE_RANGE = 3;
 constexpr unsigned DEV_ERR_RERANK_RANGE = 4;
 constexpr unsigned DEV_ERR_UNEXPECTED_LARGE_GROUP = 5;
+constexpr unsigned DEV_ERR_JOIN_TABLE_FULL = 6;
 
 __device__ __forceinline__ u32 lane_id() { return __lane_id(); }
 

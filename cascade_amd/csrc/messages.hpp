@@ -255,6 +255,102 @@ __global__ __launch_bounds__(256) void join_messages_kernel(const u8* __restrict
     keys[low] = key;
 }
 
+// ---- the join through a hash table over the cohort's suffixes (the per-generation step) ----
+//
+// The step receives its cohort in rank order and needs it in suffix order for nothing but the join. Instead of sorting
+// it by suffix (five radix passes and two gathers, src/GPU_SACA.cu:1769-1800) and searching, the cohort's suffixes go into
+// an open-addressed table (linear probing; a slot holds the 40-bit suffix, a parallel array the member's list place), and
+// every message probes it: a message whose recipient has retired, which most are, ends at an empty slot of the line it
+// read first, instead of a directory line and a line of the sorted cohort. What a message delivers is the 32-bit rank
+// word as it came (pill bit included) at the recipient's list place; the composite keys are put together afterwards in
+// one streaming pass. Same outcome as join_messages_kernel (include/GPU_SACA.cuh:362-389).
+constexpr u64 JOIN_EMPTY = ~0ull;      // no suffix is all ones (suffixes are below 2^40)
+constexpr u32 JOIN_NOTHING = ~0u;      // no rank word is all ones (ranks are below 2^31 - 1)
+
+__device__ __forceinline__ u64 join_home(u64 suffix, u64 slots)
+{
+    return __umul64hi(suffix * 0x9E3779B97F4A7C15ull, slots); // the high word of a 128-bit product: in [0, slots)
+}
+
+__device__ __forceinline__ u64 lane_value(const u8* __restrict__ lanes, u64 i)
+{
+    u64 v = 0;
+#pragma unroll
+    for (int b = 0; b < 5; ++b)
+        v |= (u64)lanes[5 * i + b] << (8 * b);
+    return v;
+}
+
+// table[s] = suffix of list place place_of[s]; `slots` >= m entries, all JOIN_EMPTY before the launch
+__global__ __launch_bounds__(256) void join_table_insert_kernel(const u8* __restrict__ suf40, u64 m, unsigned long long* table,
+                                                                u32* __restrict__ place_of, u64 slots, u32* err)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= m)
+        return;
+    const u64 suffix = lane_value(suf40, i);
+    u64 s = join_home(suffix, slots);
+    for (u64 step = 0; step < slots; ++step) {
+        // an atomic costs several times a load: only a slot that reads empty is tried
+        if (*(volatile unsigned long long*)&table[s] == JOIN_EMPTY &&
+            atomicCAS(&table[s], (unsigned long long)JOIN_EMPTY, (unsigned long long)suffix) == JOIN_EMPTY) {
+            place_of[s] = (u32)i;
+            return;
+        }
+        s = s + 1 == slots ? 0 : s + 1;
+    }
+    atomicExch(err, DEV_ERR_JOIN_TABLE_FULL); // more members than slots: the caller sized the table wrongly
+}
+
+// sec[place] = rank word of the message whose target is the member at that list place (sec is JOIN_NOTHING-filled)
+__global__ __launch_bounds__(256) void join_table_probe_kernel(const u8* __restrict__ msg_target, const u32* __restrict__ msg_rank, u32 msg_c,
+                                                               const unsigned long long* __restrict__ table, const u32* __restrict__ place_of,
+                                                               u64 slots, u32* __restrict__ sec)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= msg_c)
+        return;
+    const u64 target = lane_value(msg_target, i);
+    u64 s = join_home(target, slots);
+    for (u64 step = 0; step < slots; ++step) {
+        const u64 v = table[s];
+        if (v == JOIN_EMPTY)
+            return; // the recipient is not in the cohort: it has retired, the message is dropped
+        if (v == target) {
+            sec[place_of[s]] = msg_rank[i];
+            return;
+        }
+        s = s + 1 == slots ? 0 : s + 1;
+    }
+}
+
+// keys[i] = primary[i] << 31 | received rank, marked if the message was a pill; all ones where nothing arrived
+// (src/GPU_SACA.cu:1826, include/GPU_SACA.cuh:383-387)
+__global__ __launch_bounds__(256) void compose_join_keys_kernel(const u32* __restrict__ primary, const u32* __restrict__ sec, u64 m,
+                                                                u64* __restrict__ keys)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= m)
+        return;
+    const u32 r = sec[i];
+    u64 key = ~0ull;
+    if (r != JOIN_NOTHING) {
+        key = ((u64)primary[i] << 31) | (u64)(r & ~MSG_PILL_BIT);
+        if (r & MSG_PILL_BIT)
+            key |= MSG_PILL_RECEIPT;
+    }
+    keys[i] = key;
+}
+
+// words[i] = suffix of list place perm[i] (5-byte lanes gathered through a permutation)
+__global__ __launch_bounds__(256) void gather_lanes_kernel(const u8* __restrict__ lanes, const u32* __restrict__ perm, u64 count,
+                                                           u64* __restrict__ words)
+{
+    const u64 i = (u64)blockIdx.x * 256 + threadIdx.x;
+    if (i < count)
+        words[i] = lane_value(lanes, perm[i]);
+}
+
 // 5-byte lanes -> 64-bit words (the keys of the inbox sort)
 __global__ __launch_bounds__(256) void unpack_lanes_kernel(const u8* __restrict__ lanes, u64 count, u64* __restrict__ words)
 {

@@ -28,12 +28,12 @@
 //           words 0 and 1 from the sorted columns) or [48,52) (W >= 3: it reads words 2 and 3 through the permutation)
 //   [ 0, 5) outbox targets, [ 5, 9) outbox ranks, [ 9,13) ranks out, [40,45) lanes out
 // Generation t >= 1 (47 bytes per unit, the unit being the larger of the cohort and its inbox):
-//   [ 0,24) K0 K1 P0 P1 (the sort by suffix); lanes in at [ 8,13) until they are unpacked into K0, before that sort
-//   [24,28) ranks in, [28,32) routing tags in, [32,37) inbox targets, [37,41) inbox ranks
-//   ranks and tags in suffix order -> the two halves of the spare K; the join directory is the spare P
-//   [24,32) composite keys (ranks and tags in are dead); the join ends the inbox's life
-//   the second sort: keys [24,32) <-> [32,40), permutations in P0 P1
-//   sorted suffix words -> the other of [24,32) / [32,40); sorted tags -> the spare P
+//   [ 0, 4) routing tags in, [ 4, 8) ranks in, [12,17) inbox targets, [17,21) inbox ranks, [42,47) lanes in
+//   [21,35) the join table (8-byte slots, up to 1.75 per unit), [35,42) the list places of its slots
+//   [ 8,12) what the messages deliver: the rank word received at every list place
+//   [24,32) composite keys (the table and the inbox are dead)
+//   the sort: keys [24,32) <-> [32,40), permutations in P0 [16,20) and P1 [20,24)
+//   sorted suffix words (gathered from the lanes in) -> the other of [24,32) / [32,40); sorted tags -> the spare P
 //   [ 0, 8) ranked keys, [ 8,16) ranked suffix words, ranked tags -> the permutation's place
 //   [24,34) outbox targets, [34,42) outbox ranks (two messages per suffix), [16,20) ranks out, [42,47) lanes out
 // With the caller's own buffers for inputs and outputs (csa_sort_init_dev, csa_sort_rerank_dev) the same plans hold
@@ -103,7 +103,7 @@ struct RerankInputs {
     u8* inbox_target;
     u32* inbox_rank;
 };
-RerankInputs rerank_input_places(const StepPlan& pl) { return {pl.at<u32>(24), pl.at<u8>(8), pl.at<u32>(28), pl.at<u8>(32), pl.at<u32>(37)}; }
+RerankInputs rerank_input_places(const StepPlan& pl) { return {pl.at<u32>(4), pl.at<u8>(42), pl.at<u32>(0), pl.at<u8>(12), pl.at<u32>(17)}; }
 
 // Where the tail of a step (ranking, messages, narrowing) puts its columns.
 struct TailPlaces {
@@ -346,40 +346,31 @@ int step_rerank(Launch& L, const char* who, StepColumns& c, const StepPlan& pl, 
     hipStream_t s = L.stream;
     const u32 blocks = (u32)((m + 255) / 256);
     HIP_TRY(hipMemsetAsync(h->counts, 0, 8 * sizeof(u32), s));
-    u64* K[2] = {pl.at<u64>(0), pl.at<u64>(8)};
     u32* P[2] = {pl.at<u32>(16), pl.at<u32>(20)};
-    // 1. the cohort in suffix order, so that messages can be joined by search (src/GPU_SACA.cu:1769-1800)
-    hipLaunchKernelGGL(unpack_words_kernel, dim3(blocks), dim3(256), 0, s, c.suf40, (const u32*)nullptr, (const u32*)nullptr, m, 0, K[0],
-                       (u32*)nullptr);
-    hipLaunchKernelGGL(iota_kernel, dim3(blocks), dim3(256), 0, s, P[0], m);
-    int in_out = 0, passes = 0;
-    int rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, K[0], P[0], K[1], P[1], (u32)m, make_plan(0, 40), &in_out, &passes);
-    if (rc)
-        return rc;
-    const u64* words_by_suffix = K[in_out];
-    u32* spare_k = reinterpret_cast<u32*>(K[in_out ^ 1]);
-    u32* primary_by_suffix = spare_k;
-    u32* beta_by_suffix = spare_k + pl.unit; // the second half of the spare key array
-    u32* dir = P[in_out ^ 1];                // the spare permutation array holds the join directory
-    hipLaunchKernelGGL(gather_u32_kernel, dim3(blocks), dim3(256), 0, s, c.rank_in, (const u32*)P[in_out], m, primary_by_suffix);
-    hipLaunchKernelGGL(gather_u32_kernel, dim3(blocks), dim3(256), 0, s, c.beta, (const u32*)P[in_out], m, beta_by_suffix);
-    // 2. composite keys from the inbox: primary << 31 | received rank, all ones where nothing arrives
-    //    (src/GPU_SACA.cu:1803-1835)
+    // 1. the join (src/GPU_SACA.cu:1769-1835): the cohort stays in the order it came in; its suffixes go into a hash
+    //    table, the messages probe it and leave their rank words at the recipients' list places
+    u32* sec = pl.at<u32>(8);
     u64* keys = pl.at<u64>(24);
-    hipLaunchKernelGGL(fill_u64_kernel, dim3(blocks), dim3(256), 0, s, keys, m, ~0ull);
+    HIP_TRY(hipMemsetAsync(sec, 0xFF, m * sizeof(u32), s));
+    int rc;
     if (c.inbox_sz) {
-        u32 dir_log2 = 0;
-        rc = build_join_directory(words_by_suffix, m, dir, m, s, &dir_log2, false);
-        if (rc)
-            return rc;
-        hipLaunchKernelGGL(join_messages_kernel, dim3((c.inbox_sz + 255u) / 256u), dim3(256), 0, s, c.inbox_target, (const u64*)nullptr,
-                           c.inbox_rank, c.inbox_sz, words_by_suffix, (const u32*)primary_by_suffix, keys, m,
-                           (const u32*)(dir_log2 ? dir : nullptr), dir_log2);
+        unsigned long long* table = pl.at<unsigned long long>(21);
+        u32* place_of = pl.at<u32>(35);
+        u64 slots = pl.unit + pl.unit / 2 + pl.unit / 4; // 14 bytes per unit of slots, 7 of places
+        if (slots > 2 * m + 64)
+            slots = 2 * m + 64;
+        HIP_TRY(hipMemsetAsync(table, 0xFF, slots * sizeof(unsigned long long), s));
+        hipLaunchKernelGGL(join_table_insert_kernel, dim3(blocks), dim3(256), 0, s, c.suf40, m, table, place_of, slots, h->counts + 2);
+        hipLaunchKernelGGL(join_table_probe_kernel, dim3((c.inbox_sz + 255u) / 256u), dim3(256), 0, s, c.inbox_target, c.inbox_rank,
+                           c.inbox_sz, (const unsigned long long*)table, (const u32*)place_of, slots, sec);
     }
+    // 2. composite keys: primary << 31 | received rank, all ones where nothing arrived (src/GPU_SACA.cu:1803-1835)
+    hipLaunchKernelGGL(compose_join_keys_kernel, dim3(blocks), dim3(256), 0, s, c.rank_in, (const u32*)sec, m, keys);
     HIP_TRY(hipGetLastError());
     // 3. sort by (primary, secondary): key bits [0, 62) (src/GPU_SACA.cu:1841-1871)
     u64* keys_partner = pl.at<u64>(32);
     hipLaunchKernelGGL(iota_kernel, dim3(blocks), dim3(256), 0, s, P[0], m);
+    int in_out = 0, passes = 0;
     rc = radix_sort(L, SRC_PAIRS, nullptr, 0, 0, 0, keys, P[0], keys_partner, P[1], (u32)m, make_plan(0, 62), &in_out, &passes);
     if (rc)
         return rc;
@@ -387,8 +378,8 @@ int step_rerank(Launch& L, const char* who, StepColumns& c, const StepPlan& pl, 
     u64* sorted_words = in_out ? keys : keys_partner;
     const u32* perm = P[in_out];
     u32* sorted_beta = P[in_out ^ 1];
-    hipLaunchKernelGGL(gather_u64_kernel, dim3(blocks), dim3(256), 0, s, words_by_suffix, perm, m, 1u, 0u, sorted_words);
-    hipLaunchKernelGGL(gather_u32_kernel, dim3(blocks), dim3(256), 0, s, (const u32*)beta_by_suffix, perm, m, sorted_beta);
+    hipLaunchKernelGGL(gather_lanes_kernel, dim3(blocks), dim3(256), 0, s, c.suf40, perm, m, sorted_words);
+    hipLaunchKernelGGL(gather_u32_kernel, dim3(blocks), dim3(256), 0, s, c.beta, perm, m, sorted_beta);
     HIP_TRY(hipGetLastError());
     // 4. refine, split, messages, narrow
     TailPlaces tp;
