@@ -78,8 +78,12 @@ __global__ __launch_bounds__(PID_BLOCK) void partition_ids_kernel(PartitionIdArg
     const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
     const bool hist_lds = a.psz != nullptr && a.p <= PID_LDS_BINS;
     const u32 copies_log2 = a.hist_copies_log2; // counters per partition in the LDS histogram
-    for (u32 i = t; i < piv_slots; i += PID_BLOCK)
-        s_piv[i] = i < np * (u32)W ? a.pivots[i] : ~0ull;
+    // word j of pivot i at s_piv[j * slots + i]: the first words of all pivots lie together
+    const u32 slots = PIV_LDS ? (1u << steps) - 1u : 1u;
+    for (u32 i = t; i < piv_slots; i += PID_BLOCK) {
+        const u32 j = i / slots, pv = i - j * slots;
+        s_piv[i] = pv < np ? a.pivots[(u64)pv * W + j] : ~0ull;
+    }
     if (hist_lds)
         for (u32 i = t; i < (a.p << copies_log2); i += PID_BLOCK)
             s_hist[i] = 0;
@@ -95,47 +99,75 @@ __global__ __launch_bounds__(PID_BLOCK) void partition_ids_kernel(PartitionIdArg
         const u32* s_dw = reinterpret_cast<const u32*>(s_text);
 
         // keys of this thread's suffixes (zero for lanes past the end: never used)
-        u64 key[PID_ITEMS][W];
+        // (with the pivots in LDS the words after the first are taken from the staged text only where they are needed)
+        u64 key[PID_ITEMS][PIV_LDS ? 1 : W];
         u32 id[PID_ITEMS];
 #pragma unroll
         for (int k = 0; k < PID_ITEMS; ++k) {
             const u32 local = (w * PID_ITEMS + (u32)k) * 64u + lane;
             id[k] = 0;
 #pragma unroll
-            for (int j = 0; j < W; ++j)
+            for (int j = 0; j < (PIV_LDS ? 1 : W); ++j)
                 key[k][j] = local < count ? staged_kgram(s_dw, sym_off + local + 4u * j) : 0ull;
         }
         // id = number of pivots below the key = the smallest id with key <= pivots[id], p - 1 if there is none
         // (test/partitioning.cpp:21-31), found by fixing the bits of the answer from the top. In LDS the table is filled up
-        // to 2^steps - 1 entries with all-ones keys, which are below no key: no probe needs a bounds check, and every
-        // probe reads all W words and decides without a branch.
-        for (int b = steps - 1; b >= 0; --b) {
+        // to 2^steps - 1 entries with all-ones keys, which are below no key: no probe needs a bounds check.
+        if (PIV_LDS) {
+            // First by the first word alone (one LDS word and one compare per probe): the number of pivots whose first
+            // word is below the key's. Only a key whose first word equals that of the pivot it stopped at (a K-gram that
+            // some pivot starts with: few suffixes of a text) is placed again, by all W words.
+            for (int b = steps - 1; b >= 0; --b) {
 #pragma unroll
-            for (int k = 0; k < PID_ITEMS; ++k) {
-                const u32 cand = id[k] + (1u << b);
-                if (PIV_LDS) {
-                    const u64* pv = s_piv + (u64)(cand - 1u) * W;
-                    bool below = false, decided = false; // pivot < key, by the first word that differs
+                for (int k = 0; k < PID_ITEMS; ++k) {
+                    const u32 cand = id[k] + (1u << b);
+                    id[k] = s_piv[cand - 1u] < key[k][0] ? cand : id[k];
+                }
+            }
+            if (W > 1) {
 #pragma unroll
-                    for (int j = 0; j < W; ++j) {
-                        const u64 x = pv[j];
-                        below = decided ? below : x < key[k][j];
-                        decided = decided || x != key[k][j];
-                    }
-                    id[k] = below ? cand : id[k];
-                } else if (cand <= np) {
-                    const u64* pv = a.pivots + (u64)(cand - 1u) * W;
-                    bool below = false;
+                for (int k = 0; k < PID_ITEMS; ++k) {
+                    const u32 local = (w * PID_ITEMS + (u32)k) * 64u + lane;
+                    if (local < count && id[k] < np && s_piv[id[k]] == key[k][0]) {
+                        u64 whole[W];
 #pragma unroll
-                    for (int j = 0; j < W; ++j) {
-                        const u64 x = pv[j];
-                        if (x != key[k][j]) {
-                            below = x < key[k][j];
-                            break;
+                        for (int j = 0; j < W; ++j)
+                            whole[j] = staged_kgram(s_dw, sym_off + local + 4u * j);
+                        u32 again = 0;
+                        for (int b = steps - 1; b >= 0; --b) {
+                            const u32 cand = again + (1u << b);
+                            bool below = false, decided = false; // pivot < key, by the first word that differs
+#pragma unroll
+                            for (int j = 0; j < W; ++j) {
+                                const u64 x = s_piv[(u32)j * slots + cand - 1u];
+                                below = decided ? below : x < whole[j];
+                                decided = decided || x != whole[j];
+                            }
+                            again = below ? cand : again;
                         }
+                        id[k] = again;
                     }
-                    if (below)
-                        id[k] = cand;
+                }
+            }
+        } else {
+            for (int b = steps - 1; b >= 0; --b) {
+#pragma unroll
+                for (int k = 0; k < PID_ITEMS; ++k) {
+                    const u32 cand = id[k] + (1u << b);
+                    if (cand <= np) {
+                        const u64* pv = a.pivots + (u64)(cand - 1u) * W;
+                        bool below = false;
+#pragma unroll
+                        for (int j = 0; j < W; ++j) {
+                            const u64 x = pv[j];
+                            if (x != key[k][j]) {
+                                below = x < key[k][j];
+                                break;
+                            }
+                        }
+                        if (below)
+                            id[k] = cand;
+                    }
                 }
             }
         }
