@@ -1541,7 +1541,11 @@ int csa_emit_messages_dev(const uint64_t* d_sa, const uint64_t* d_keys, const ui
     a.msg_target = d_msg_target;
     a.msg_rank = d_msg_rank;
     a.msg_off = d_msg_off;
-    hipLaunchKernelGGL(emit_messages_kernel, dim3(a.tiles < 4096u ? a.tiles : 4096u), dim3(MSG_BLOCK), 0, (hipStream_t)stream, a);
+    const u64 emit_tiles = (n + EMIT_TILE - 1) / EMIT_TILE;
+    if (a.p <= EMIT_FEW_PARTS)
+        hipLaunchKernelGGL((emit_messages_kernel<EMIT_FEW_PARTS>), dim3((u32)(emit_tiles < 2048u ? emit_tiles : 2048u)), dim3(EMIT_BLOCK), 0, (hipStream_t)stream, a);
+    else
+        hipLaunchKernelGGL((emit_messages_kernel<MSG_LDS_PARTS>), dim3((u32)(emit_tiles < 2048u ? emit_tiles : 2048u)), dim3(EMIT_BLOCK), 0, (hipStream_t)stream, a);
     HIP_TRY(hipGetLastError());
     return CSA_OK;
 }

@@ -99,25 +99,44 @@ __global__ __launch_bounds__(MSG_BLOCK) void count_messages_kernel(MessageArgs a
     }
 }
 
-// Writes the messages: a tile counts its messages per destination in LDS, reserves one range per destination with
-// a single global atomic, and its messages take consecutive slots of that range.
-__global__ __launch_bounds__(MSG_BLOCK) void emit_messages_kernel(MessageArgs a)
+// Writes the messages: a tile of EMIT_TILE list elements counts its messages per destination in LDS, reserves one range
+// per destination with a single global atomic, orders its messages by destination in LDS and stores them as runs: the
+// messages of one destination leave together, lane after lane, instead of as single 5-byte and 4-byte stores all over
+// the outbox. With more than MSG_LDS_PARTS destinations every message takes its slot with a global atomic and is
+// stored where it falls, as the reference does.
+constexpr u32 EMIT_FEW_PARTS = 256;
+constexpr int EMIT_BLOCK = 512;
+constexpr int EMIT_ITEMS = 4;
+constexpr int EMIT_TILE = EMIT_BLOCK * EMIT_ITEMS;
+constexpr int EMIT_CAP = 2 * EMIT_TILE; // a payload and a forwarded pill per element
+
+// PARTS: the destinations the LDS tables hold (fewer: more workgroups per CU).
+template <u32 PARTS>
+__global__ __launch_bounds__(EMIT_BLOCK) void emit_messages_kernel(MessageArgs a)
 {
-    __shared__ u32 s_cnt[MSG_LDS_PARTS];
-    __shared__ u32 s_base[MSG_LDS_PARTS];
-    const u32 t = threadIdx.x;
-    const bool lds = a.p <= MSG_LDS_PARTS;
+    __shared__ u32 s_cnt[PARTS];  // the tile's messages per destination
+    __shared__ u32 s_excl[PARTS]; // where they start in the ordered tile
+    __shared__ u32 s_base[PARTS]; // where they go in the outbox
+    __shared__ u32 s_low[EMIT_CAP];
+    __shared__ u32 s_rank[EMIT_CAP];
+    __shared__ u16 s_dest[EMIT_CAP];
+    __shared__ u8 s_high[EMIT_CAP];
+    __shared__ u32 s_wave[EMIT_BLOCK / 64 + 1];
+    const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
+    const bool lds = a.p <= PARTS;
     const u64 active_sz = *a.active_sz;
-    for (u32 tile = blockIdx.x; tile < a.tiles; tile += gridDim.x) {
+    const u64 tiles = (a.n + EMIT_TILE - 1) / EMIT_TILE;
+    const u32 per = (a.p + EMIT_BLOCK - 1) / EMIT_BLOCK; // destinations per thread in the scan
+    for (u64 tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
         if (lds)
-            for (u32 q = t; q < a.p; q += MSG_BLOCK)
+            for (u32 q = t; q < a.p; q += EMIT_BLOCK)
                 s_cnt[q] = 0;
-        __syncthreads();
-        Message m[2 * MSG_ITEMS];
-        u32 slot[2 * MSG_ITEMS];
+        __syncthreads(); // also: the ordered tile of the round before has been stored
+        Message m[2 * EMIT_ITEMS];
+        u32 slot[2 * EMIT_ITEMS];
 #pragma unroll
-        for (int k = 0; k < MSG_ITEMS; ++k) {
-            const u64 i = (u64)tile * MSG_TILE + (u64)k * MSG_BLOCK + t;
+        for (int k = 0; k < EMIT_ITEMS; ++k) {
+            const u64 i = tile * EMIT_TILE + (u64)k * EMIT_BLOCK + t;
             m[2 * k].dest = m[2 * k + 1].dest = 0xFFFFFFFFu;
             if (i < a.n)
                 messages_of(a, i, active_sz, m[2 * k], m[2 * k + 1]);
@@ -130,24 +149,65 @@ __global__ __launch_bounds__(MSG_BLOCK) void emit_messages_kernel(MessageArgs a)
                     slot[2 * k + e] = atomicAdd(lds ? &s_cnt[mm.dest] : &a.msg_off[mm.dest], 1u);
             }
         }
-        if (lds) {
-            __syncthreads();
-            for (u32 q = t; q < a.p; q += MSG_BLOCK)
-                if (s_cnt[q])
-                    s_base[q] = atomicAdd(&a.msg_off[q], s_cnt[q]);
-            __syncthreads();
-        }
+        if (!lds) {
 #pragma unroll
-        for (int e = 0; e < 2 * MSG_ITEMS; ++e) {
+            for (int e = 0; e < 2 * EMIT_ITEMS; ++e) {
+                if (m[e].dest == 0xFFFFFFFFu)
+                    continue;
+                const u64 s = slot[e];
+#pragma unroll
+                for (int b = 0; b < 5; ++b)
+                    a.msg_target[5 * s + b] = (u8)(m[e].target >> (8 * b));
+                a.msg_rank[s] = m[e].rank;
+            }
+            continue;
+        }
+        __syncthreads();
+        // exclusive prefix sums of the counts over the destinations; one range of the outbox per destination
+        const u32 first = t * per < a.p ? t * per : a.p;
+        const u32 last = first + per < a.p ? first + per : a.p;
+        u32 sum = 0;
+        for (u32 q = first; q < last; ++q)
+            sum += s_cnt[q];
+        const u32 incl = wave_incl_sum(sum);
+        if (lane == 63u)
+            s_wave[w] = incl;
+        __syncthreads();
+        u32 run = incl - sum;
+        for (u32 ww = 0; ww < w; ++ww)
+            run += s_wave[ww];
+        if (t == EMIT_BLOCK - 1)
+            s_wave[EMIT_BLOCK / 64] = run + sum; // the tile's messages
+        for (u32 q = first; q < last; ++q) {
+            const u32 c = s_cnt[q];
+            s_excl[q] = run;
+            if (c)
+                s_base[q] = atomicAdd(&a.msg_off[q], c);
+            run += c;
+        }
+        __syncthreads();
+        const u32 total = s_wave[EMIT_BLOCK / 64];
+#pragma unroll
+        for (int e = 0; e < 2 * EMIT_ITEMS; ++e) {
             if (m[e].dest == 0xFFFFFFFFu)
                 continue;
-            const u64 s = (u64)slot[e] + (lds ? s_base[m[e].dest] : 0u);
-#pragma unroll
-            for (int b = 0; b < 5; ++b)
-                a.msg_target[5 * s + b] = (u8)(m[e].target >> (8 * b));
-            a.msg_rank[s] = m[e].rank;
+            const u32 at = s_excl[m[e].dest] + slot[e];
+            s_low[at] = (u32)m[e].target;
+            s_high[at] = (u8)(m[e].target >> 32);
+            s_rank[at] = m[e].rank;
+            s_dest[at] = (u16)m[e].dest;
         }
-        __syncthreads(); // the counters are cleared for the next tile
+        __syncthreads();
+        for (u32 j = t; j < total; j += EMIT_BLOCK) {
+            const u32 d = s_dest[j];
+            const u64 s = (u64)s_base[d] + (j - s_excl[d]);
+            const u32 low = s_low[j];
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+                a.msg_target[5 * s + b] = (u8)(low >> (8 * b));
+            a.msg_target[5 * s + 4] = s_high[j];
+            a.msg_rank[s] = s_rank[j];
+        }
     }
 }
 

@@ -173,7 +173,11 @@ int finish_partition_step(Launch& L, const char* who, StepColumns& c, const Tail
     ma.active_sz = d_active;
     ma.msg_target = c.msg_target;
     ma.msg_rank = c.msg_rank;
-    hipLaunchKernelGGL(emit_messages_kernel, dim3(grid), dim3(MSG_BLOCK), 0, s, ma);
+    const u64 emit_tiles = (m + EMIT_TILE - 1) / EMIT_TILE;
+    if (ma.p <= EMIT_FEW_PARTS)
+        hipLaunchKernelGGL((emit_messages_kernel<EMIT_FEW_PARTS>), dim3((u32)(emit_tiles < 2048u ? emit_tiles : 2048u)), dim3(EMIT_BLOCK), 0, s, ma);
+    else
+        hipLaunchKernelGGL((emit_messages_kernel<MSG_LDS_PARTS>), dim3((u32)(emit_tiles < 2048u ? emit_tiles : 2048u)), dim3(EMIT_BLOCK), 0, s, ma);
     HIP_TRY(hipGetLastError());
     // what the caller persists: narrowed ranks and lanes (src/GPU_SACA.cu:1289-1305)
     if (!c.rank_out)
