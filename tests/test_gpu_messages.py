@@ -67,7 +67,7 @@ def gpu():
 @pytest.mark.parametrize("packed,ctx", [(False, 4), (True, 8), (True, 1 << 20)])
 def test_count_offsets_and_emit_match_the_oracle(gpu, packed, ctx):
     lib, to_dev, to_host = gpu
-    for n, p in ((1, 3), (255, 3), (1025, 17), (100003, 64), (1 << 20, 2048), (50000, 2049), (50000, 32768)):
+    for n, p in ((1, 3), (255, 3), (1025, 17), (100003, 64), (70001, 256), (70001, 257), (1 << 20, 2048), (50000, 2049), (50000, 32768)):
         print(f"  messages n={n} p={p} ctx={ctx} packed={packed}", flush=True)
         check_messages(lib, to_dev, to_host, n, p, ctx, packed, seed=n + p)
 
