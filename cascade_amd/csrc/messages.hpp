@@ -325,7 +325,8 @@ __global__ __launch_bounds__(256) void join_messages_kernel(const u8* __restrict
 // word as it came (pill bit included) at the recipient's list place; the composite keys are put together afterwards in
 // one streaming pass. Same outcome as join_messages_kernel (include/GPU_SACA.cuh:362-389).
 constexpr u64 JOIN_EMPTY = ~0ull;      // no suffix is all ones (suffixes are below 2^40)
-constexpr u32 JOIN_NOTHING = ~0u;      // no rank word is all ones (ranks are below 2^31 - 1)
+constexpr u32 JOIN_NOTHING = ~0u;      // no rank word is all ones: ranks are below 2^31 - 1 (only the forwarded pill of a member that
+                                       // no message joined would be, which the exchange scheme excludes; it counts as nothing)
 
 __device__ __forceinline__ u64 join_home(u64 suffix, u64 slots)
 {
