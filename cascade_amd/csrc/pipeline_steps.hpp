@@ -366,6 +366,17 @@ __global__ __launch_bounds__(STEP_BLOCK) void step_rank_kernel(StepRankArgs a)
     }
     u32 ra = xa > pre_a ? xa : pre_a, rb = xb > pre_b ? xb : pre_b;
     u32 act_before = pre_c + xc; // active entries before this thread's first
+    // everything the thread moves is read before its first store: the outputs may alias the inputs as far as the
+    // compiler can tell, and loads behind a store would wait for it
+    u64 old_key[STEP_ITEMS], old_word[STEP_ITEMS];
+    u32 old_beta[STEP_ITEMS];
+#pragma unroll
+    for (int k = 0; k < STEP_ITEMS; ++k) {
+        const u64 i = base + k;
+        old_key[k] = i < a.m ? a.key0[i] : 0ull;
+        old_word[k] = i < a.m ? a.words[i] : 0ull;
+        old_beta[k] = i < a.m ? a.beta[i] : 0u;
+    }
 #pragma unroll
     for (int k = 0; k < STEP_ITEMS; ++k) {
         const u64 i = base + k;
@@ -376,7 +387,7 @@ __global__ __launch_bounds__(STEP_BLOCK) void step_rank_kernel(StepRankArgs a)
         if (ph[k])
             rb = (u32)i + 1u;
         const bool active = !(kh[k] && kh[k + 1]);
-        const u64 old = a.key0[i];
+        const u64 old = old_key[k];
         u64 key;
         if (GEN0) {
             key = (u64)(ra - 1u); // plain rank: offset of the run's head
@@ -386,8 +397,8 @@ __global__ __launch_bounds__(STEP_BLOCK) void step_rank_kernel(StepRankArgs a)
         }
         const u64 dest = active ? (u64)act_before : (u64)total_active + (i - act_before);
         a.key_out[dest] = key;
-        a.words_out[dest] = a.words[i];
-        a.beta_out[dest] = a.beta[i];
+        a.words_out[dest] = old_word[k];
+        a.beta_out[dest] = old_beta[k];
         act_before += active ? 1u : 0u;
     }
 }

@@ -4,21 +4,23 @@
 // product never loads a library built with this header.
 //
 // Execution model: a launch runs its workgroups one after another, in blockIdx order; the threads of
-// a workgroup are real host threads, __syncthreads() is a barrier over them, and every wave-level
-// operation (__ballot, __shfl*, wave barrier) is a barrier over the 64 threads of a wave followed by an
-// exchange through a per-wave buffer. Kernels must therefore call wave operations from all 64 lanes
-// (the kernels here do). "Device memory" is host memory.
+// a workgroup are fibers of the calling host thread (each with a stack of its own, switched by hand:
+// no scheduler, no system call, the same order every run), __syncthreads() is a barrier over them, and
+// every wave-level operation (__ballot, __shfl*, wave barrier) is a barrier over the 64 fibers of a wave
+// followed by an exchange through a per-wave buffer. A fiber runs until it reaches a barrier (or
+// s_sleep) that it cannot pass yet and then hands over to the next one. Kernels must therefore call
+// wave operations from all 64 lanes (the kernels here do), and a wait on another thread of the same
+// workgroup must go through a barrier or s_sleep (theirs do). One launch at a time per process (the
+// LDS arrays are static). "Device memory" is host memory.
 #pragma once
 
 #include <atomic>
-#include <barrier>
 #include <chrono>
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
 #include <functional>
 #include <memory>
-#include <thread>
 #include <vector>
 
 #define __global__
@@ -40,17 +42,54 @@ struct dim3 {
     dim3(unsigned x_ = 1, unsigned y_ = 1, unsigned z_ = 1) : x(x_), y(y_), z(z_) {}
 };
 
+#if !defined(__x86_64__)
+#error "the fiber switch of the CPU stand-in is written for x86-64"
+#endif
+
+// hipemu_switch(save, load): parks the running fiber (its callee-saved registers on its stack, the stack pointer in
+// *save) and resumes the one whose stack pointer is `load`.
+extern "C" void hipemu_switch(void** save, void* load);
+asm(".text\n"
+    ".globl hipemu_switch\n"
+    ".type hipemu_switch,@function\n"
+    "hipemu_switch:\n"
+    "    pushq %rbp\n"
+    "    pushq %rbx\n"
+    "    pushq %r12\n"
+    "    pushq %r13\n"
+    "    pushq %r14\n"
+    "    pushq %r15\n"
+    "    movq %rsp, (%rdi)\n"
+    "    movq %rsi, %rsp\n"
+    "    popq %r15\n"
+    "    popq %r14\n"
+    "    popq %r13\n"
+    "    popq %r12\n"
+    "    popq %rbx\n"
+    "    popq %rbp\n"
+    "    ret\n"
+    ".size hipemu_switch,.-hipemu_switch\n");
+
 namespace hipemu {
 struct Wave {
-    std::barrier<> bar{64};
+    unsigned arrived = 0, phase = 0;
     uint64_t buf[64];
 };
-struct Block {
-    std::unique_ptr<std::barrier<>> bar;
-    std::vector<std::unique_ptr<Wave>> waves;
+struct Fiber {
+    void* sp = nullptr;
+    unsigned t = 0;
+    bool done = false;
 };
+struct Run {
+    std::vector<Fiber> fibers;
+    std::vector<Wave> waves;
+    unsigned arrived = 0, phase = 0; // the workgroup's barrier
+    unsigned current = 0, live = 0;
+    void* main_sp = nullptr;
+    const std::function<void()>* body = nullptr;
+};
+inline thread_local Run* run = nullptr;
 inline thread_local Wave* wave = nullptr;
-inline thread_local Block* block = nullptr;
 inline thread_local unsigned lane = 0;
 
 inline void launch(dim3 grid, dim3 blk, size_t shmem, const std::function<void()>& body);
@@ -66,57 +105,141 @@ inline void* dynamic_lds() { return dynamic_lds_storage().data(); }
 
 inline thread_local dim3 threadIdx, blockIdx, blockDim, gridDim;
 
+namespace hipemu {
+constexpr size_t FIBER_STACK = 256 * 1024;
+// stacks are kept from launch to launch
+inline std::vector<std::unique_ptr<char[]>>& fiber_stacks()
+{
+    static thread_local std::vector<std::unique_ptr<char[]>> v;
+    return v;
+}
+
+inline void enter(Fiber& f)
+{
+    run->current = f.t;
+    threadIdx = dim3(f.t);
+    lane = f.t % 64;
+    wave = &run->waves[f.t / 64];
+}
+
+// hands over to the next fiber that has not finished; returns when this one is resumed
+inline void yield()
+{
+    Run& r = *run;
+    Fiber& me = r.fibers[r.current];
+    unsigned n = me.t;
+    do
+        n = n + 1 == r.fibers.size() ? 0 : n + 1;
+    while (r.fibers[n].done);
+    if (n == me.t)
+        return; // alone: whatever it waits for will not come from a switch
+    enter(r.fibers[n]);
+    hipemu_switch(&me.sp, r.fibers[n].sp);
+    enter(me);
+}
+
+inline void barrier(unsigned& arrived, unsigned& phase, unsigned count)
+{
+    const unsigned mine = phase;
+    if (++arrived == count) {
+        arrived = 0;
+        phase = mine + 1; // the last one to arrive goes on; the others find the new phase when they are resumed
+        return;
+    }
+    while (phase == mine)
+        yield();
+}
+
+inline thread_local dim3 launch_grid;
+inline void fiber_main()
+{
+    Run& r = *run;
+    Fiber& me = r.fibers[r.current];
+    // HIPEMU_REVERSE=1 runs the workgroups from the last blockIdx to the first: results must not depend on it
+    static const bool reverse = std::getenv("HIPEMU_REVERSE") != nullptr;
+    const unsigned blocks = launch_grid.x;
+    for (unsigned i = 0; i < blocks; ++i) {
+        blockIdx = dim3(reverse ? blocks - 1 - i : i);
+        (*r.body)();
+        barrier(r.arrived, r.phase, (unsigned)r.fibers.size()); // LDS ("static") is reused by the next workgroup
+    }
+    me.done = true;
+    void* unused;
+    if (--r.live == 0) {
+        hipemu_switch(&unused, r.main_sp);
+    } else {
+        unsigned n = me.t;
+        do
+            n = n + 1 == r.fibers.size() ? 0 : n + 1;
+        while (r.fibers[n].done);
+        enter(r.fibers[n]);
+        hipemu_switch(&unused, r.fibers[n].sp);
+    }
+    std::abort(); // a finished fiber is never resumed
+}
+} // namespace hipemu
+
 inline void hipemu::launch(dim3 grid, dim3 blk, size_t shmem, const std::function<void()>& body)
 {
     const unsigned B = blk.x;
     dynamic_lds_storage().assign(shmem / 8 + 2, 0ull);
-    if (B % 64 != 0)
-        std::abort();
-    // HIPEMU_REVERSE=1 runs the workgroups from the last blockIdx to the first: results must not depend on it
-    static const bool reverse = std::getenv("HIPEMU_REVERSE") != nullptr;
-    Block b;
-    b.bar = std::make_unique<std::barrier<>>(B);
-    for (unsigned w = 0; w < B / 64; ++w)
-        b.waves.push_back(std::make_unique<Wave>());
-    std::vector<std::thread> threads;
+    if (B % 64 != 0 || run != nullptr)
+        std::abort(); // whole waves only; no launch from inside a kernel
+    if (grid.x == 0)
+        return;
+    Run r;
+    r.fibers.resize(B);
+    r.waves.resize(B / 64);
+    r.live = B;
+    r.body = &body;
+    auto& stacks = fiber_stacks();
+    while (stacks.size() < B)
+        stacks.emplace_back(new char[FIBER_STACK]);
     for (unsigned t = 0; t < B; ++t) {
-        threads.emplace_back([&, t] {
-            hipemu::block = &b;
-            hipemu::wave = b.waves[t / 64].get();
-            hipemu::lane = t % 64;
-            threadIdx = dim3(t);
-            blockDim = blk;
-            gridDim = grid;
-            for (unsigned i = 0; i < grid.x; ++i) {
-                const unsigned g = reverse ? grid.x - 1 - i : i;
-                blockIdx = dim3(g);
-                body();
-                b.bar->arrive_and_wait(); // LDS ("static") is reused by the next workgroup
-            }
-        });
+        // a fresh fiber's stack: the six registers hipemu_switch pops, then fiber_main as its return address; the
+        // stack pointer is 8 below a 16-byte boundary when fiber_main starts, as after a call
+        uintptr_t top = (reinterpret_cast<uintptr_t>(stacks[t].get()) + FIBER_STACK) & ~(uintptr_t)15;
+        void** sp = reinterpret_cast<void**>(top);
+        *--sp = nullptr; // where fiber_main would return to: it never does
+        *--sp = reinterpret_cast<void*>(&fiber_main);
+        for (int k = 0; k < 6; ++k)
+            *--sp = nullptr;
+        r.fibers[t].sp = sp;
+        r.fibers[t].t = t;
     }
-    for (auto& th : threads)
-        th.join();
+    blockDim = blk;
+    gridDim = grid;
+    launch_grid = grid;
+    const dim3 saved_thread = threadIdx, saved_block = blockIdx;
+    run = &r;
+    enter(r.fibers[0]);
+    hipemu_switch(&r.main_sp, r.fibers[0].sp);
+    run = nullptr;
+    threadIdx = saved_thread;
+    blockIdx = saved_block;
 }
 
 #define hipLaunchKernelGGL(kernel, grid, blk, shmem, stream, ...) \
     hipemu::launch((grid), (blk), (shmem), [&] { kernel(__VA_ARGS__); })
 
 // ---- synchronisation and wave operations ----
-inline void __syncthreads() { hipemu::block->bar->arrive_and_wait(); }
+inline void __syncthreads() { hipemu::barrier(hipemu::run->arrived, hipemu::run->phase, (unsigned)hipemu::run->fibers.size()); }
 inline unsigned __lane_id() { return hipemu::lane; }
-inline void __builtin_amdgcn_wave_barrier() { hipemu::wave->bar.arrive_and_wait(); }
-inline void __builtin_amdgcn_s_sleep(int) { std::this_thread::yield(); }
+namespace hipemu {
+inline void wave_sync(Wave* w) { barrier(w->arrived, w->phase, 64u); }
+} // namespace hipemu
+inline void __builtin_amdgcn_wave_barrier() { hipemu::wave_sync(hipemu::wave); }
+inline void __builtin_amdgcn_s_sleep(int) { hipemu::yield(); }
 
 inline unsigned long long __ballot(int pred)
 {
     hipemu::Wave* w = hipemu::wave;
     w->buf[hipemu::lane] = pred ? 1 : 0;
-    w->bar.arrive_and_wait();
+    hipemu::wave_sync(w);
     unsigned long long m = 0;
     for (int l = 0; l < 64; ++l)
         m |= (unsigned long long)(w->buf[l] & 1) << l;
-    w->bar.arrive_and_wait();
+    hipemu::wave_sync(w);
     return m;
 }
 
@@ -125,9 +248,9 @@ inline T __shfl(T var, unsigned src)
 {
     hipemu::Wave* w = hipemu::wave;
     w->buf[hipemu::lane] = (uint64_t)var;
-    w->bar.arrive_and_wait();
+    hipemu::wave_sync(w);
     const T r = (T)w->buf[src & 63u];
-    w->bar.arrive_and_wait();
+    hipemu::wave_sync(w);
     return r;
 }
 
@@ -136,9 +259,9 @@ inline T __shfl_up(T var, unsigned delta)
 {
     hipemu::Wave* w = hipemu::wave;
     w->buf[hipemu::lane] = (uint64_t)var;
-    w->bar.arrive_and_wait();
+    hipemu::wave_sync(w);
     const T r = hipemu::lane >= delta ? (T)w->buf[hipemu::lane - delta] : var;
-    w->bar.arrive_and_wait();
+    hipemu::wave_sync(w);
     return r;
 }
 
@@ -147,9 +270,9 @@ inline T __shfl_xor(T var, unsigned mask)
 {
     hipemu::Wave* w = hipemu::wave;
     w->buf[hipemu::lane] = (uint64_t)var;
-    w->bar.arrive_and_wait();
+    hipemu::wave_sync(w);
     const T r = (T)w->buf[(hipemu::lane ^ mask) & 63u];
-    w->bar.arrive_and_wait();
+    hipemu::wave_sync(w);
     return r;
 }
 
