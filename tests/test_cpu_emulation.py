@@ -153,9 +153,8 @@ def test_large_groups_that_are_in_order_already_skip_the_sort(emu, after_run):
     # A generation that follows one whose large groups were all in order gathers without the pairs of the radix sort, and
     # once more with them if its own large groups are not in order: with every generation starting that way, the ones that
     # do sort take the second gather, and nothing else changes
-    if after_run == 2:
-        got2, active2, big2 = emu_sort(emu, T, 1, pack=False, expect_presorted=True)
-        assert np.array_equal(got2, got) and (active2, big2, emu_sort.presorted) == (active, big, presorted)
+    got2, active2, big2 = emu_sort(emu, T, 1, pack=False, expect_presorted=True)
+    assert np.array_equal(got2, got) and (active2, big2, emu_sort.presorted) == (active, big, presorted)
 
 
 def test_small_and_large_groups_take_both_paths(emu):
@@ -223,8 +222,8 @@ def test_small_alphabets_start_from_keys_of_many_symbols(emu, name):
     padding of the last keys."""
     alphabet, key_words, key_symbols, first = PACKED_CASES[name]
     rng = np.random.default_rng(len(name))
-    body = alphabet[rng.integers(0, alphabet.size, 900 if name == "one_letter" else 1600)].astype(np.uint16)  # (one letter: every generation is dense)
-    T = np.concatenate([body, body[300:800], body[:50], np.zeros(3, dtype=np.uint16)]).astype(np.uint16)
+    body = alphabet[rng.integers(0, alphabet.size, 900 if name == "one_letter" else 2500)].astype(np.uint16)  # (one letter: every generation is dense)
+    T = np.concatenate([body, body[300:900], body[:50], np.zeros(3, dtype=np.uint16)]).astype(np.uint16)
     got, active, _ = emu_sort(emu, T, key_words)
     sa, counts = oracle_lib.prefix_doubling(T, key_words)
     assert np.array_equal(got, oracle_lib.u64_to_sa40(sa))
@@ -404,7 +403,7 @@ def test_multi_partition_pipeline_with_the_emulated_step_entries(emu, p, key_wor
 
 
 @pytest.mark.skipif(not os.path.exists(oracle_lib.SA_STRUCTURE), reason="oracle/_ref/sa_structure is not built (make -C oracle, with the reference tree present)")
-@pytest.mark.parametrize("p,key_words,pivot_words", [(4, 1, 1), (3, 4, 2)])
+@pytest.mark.parametrize("p,key_words,pivot_words", [(4, 1, 1), (5, 2, 2), (3, 4, 2)])
 def test_the_references_own_predictor_gives_the_cohorts_and_pill_receipts_of_the_steps(emu, tmp_path, p, key_words, pivot_words):
     """The reference's src/sa_structure.cpp predicts a run from the finished suffix array, the key and pivot widths and the
     partition sizes: every generation's active-set size, every query's look-back (how long ago its target retired), and the
@@ -413,8 +412,8 @@ def test_the_references_own_predictor_gives_the_cohorts_and_pill_receipts_of_the
     and exactly that many members joined by a pill (csa_step_result.pills, counted on the device), summed over the
     partitions; they emit that many messages in generation 0, when nothing is flagged yet, and never more later."""
     import multi_partition
-    T = texts.random_text(600, 2, 17 * p, sep_every=0)
-    T[300:500] = T[20:220]
+    T = texts.random_text(800, 2, 17 * p, sep_every=0)
+    T[300:520] = T[20:240]
     T[-6:] = 0
     log = []
     sa, _ = multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, p, key_words=key_words,
