@@ -274,11 +274,20 @@ def test_emulated_radix_sort_without_allocation_matches_the_one_with_a_handle(em
     assert emu.csa_radix_sort_pairs_static_dev(big.ctypes.data, big.ctypes.data, 20001, 0, 64, None) == -2
 
 
-@pytest.mark.parametrize("words,p", [(1, 1), (1, 3), (2, 17), (3, 300), (4, 5)])
+@pytest.mark.parametrize("words,p", [(1, 1), (1, 3), (2, 2), (2, 16), (2, 17), (2, 256), (3, 300), (4, 5), (4, 64)])
 def test_emulated_partition_ids_match_the_oracle(emu, words, p):
+    """Pivot counts that fill the searched table exactly (p = 2^k) and that leave it padded; texts over three symbols, of one
+    symbol and of separators only (all-ones K-grams, the value the table's padding holds): most suffixes start like some
+    pivot there and are placed by the search over all key words."""
     rng = np.random.default_rng(words * 1000 + p)
-    for n in (1, 64, 65, 2049, 4500):
+    for n in (1, 64, 65, 2049, 4500, 3001, 3002):
         T = texts.random_text(n, 3, n + p, sep_every=0)
+        if n == 3001:
+            T[:] = 7
+            T[n // 2] = 8
+        if n == 3002:
+            T[:] = 0xFFFF
+            T[n // 3] = 5
         pivots = oracle_lib.sample_pivots(T, p, words, rng, duplicates=True)
         bits = oracle_lib.partition_id_bits(p)
         ids = np.zeros(n, dtype=np.uint16)

@@ -49,6 +49,21 @@ def test_ids_map_and_sizes_match_the_oracle(torch_mod, words):
             check(torch_mod, T, oracle_lib.sample_pivots(T, p, words, rng, duplicates=True), p, words, f"n={n}")
 
 
+@pytest.mark.parametrize("words", [2, 4])
+def test_texts_whose_suffixes_start_like_the_pivots(torch_mod, words):
+    """One symbol repeated, and separators only (K-grams of all ones, the value that pads the searched table): nearly every
+    suffix equals some pivot in its first key word and is placed by the search over all words; pivot counts that fill the
+    table exactly (p = 2^k) and that leave it padded."""
+    rng = np.random.default_rng(10 + words)
+    n = 70001
+    for fill in (7, 0xFFFF):
+        T = np.full(n, fill, dtype=np.uint16)
+        T[n // 3] = 5
+        T[n // 2:n // 2 + 40] = rng.integers(0, 3, 40)
+        for p in (2, 16, 17, 256):
+            check(torch_mod, T, oracle_lib.sample_pivots(T, p, words, rng, duplicates=True), p, words, f"fill={fill} p={p}")
+
+
 def test_many_partitions_take_the_global_tables(torch_mod):
     # more pivots than fit in LDS, and more partitions than the LDS histogram holds
     rng = np.random.default_rng(3)
