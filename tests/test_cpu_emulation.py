@@ -100,6 +100,37 @@ def test_fixtures_through_the_emulated_kernels(emu, key_words):
         assert active == counts, name
 
 
+def test_random_texts_through_the_emulated_sort(emu):
+    """Random alphabets (1 to 65536 symbols), structures (plain, a long repeat, a zero tail, a run of one symbol, a period),
+    key widths and tuning knobs (packed first sort on and off, the speculative gather): the suffix array and every
+    generation's active-set size are the oracle's."""
+    rng = np.random.default_rng(77)
+    for case in range(60):
+        n = int(rng.integers(1, 3000))
+        sigma = int(rng.choice([1, 2, 3, 4, 7, 16, 200, 300, 65536]))
+        T = rng.integers(0, sigma, n).astype(np.uint16)
+        shape = int(rng.integers(0, 5))
+        if shape == 1 and n > 100:
+            length = int(rng.integers(10, n // 2))
+            T[n - length:] = T[:length]
+        if shape == 2:
+            T[-int(rng.integers(1, 40)):] = 0
+        if shape == 3 and n > 100:
+            a = int(rng.integers(0, n // 2))
+            T[a:a + int(rng.integers(5, n // 2))] = T[a]
+        if shape == 4 and n > 100:
+            period = int(rng.integers(1, 9))
+            a = int(rng.integers(0, n // 2))
+            stretch = int(rng.integers(20, n // 2))
+            T[a:a + stretch] = np.resize(T[a:a + period], stretch)
+        key_words = int(rng.integers(1, 5))
+        pack, speculate = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        got, active, _ = emu_sort(emu, T, key_words, pack=pack, expect_presorted=speculate)
+        assert np.array_equal(got, oracle_lib.build_sa40(T)), (case, n, sigma, shape, key_words, pack, speculate)
+        _, counts = oracle_lib.prefix_doubling(T, key_words)
+        assert active == counts, (case, n, sigma, shape, key_words, pack, speculate)
+
+
 @pytest.mark.parametrize("key_words", [3, 4])
 def test_keys_of_three_and_four_words(emu, key_words):
     # wide keys (four words, 16 symbols, are the reference's default) run as one-word keys whose first generations stand
@@ -409,6 +440,34 @@ def test_multi_partition_pipeline_with_the_emulated_step_entries(emu, p, key_wor
     # the same run with numpy glue between the stages: the same cohorts, survivors and message counts at every step
     multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, p, key_words=key_words, log=glue_log)
     assert log == glue_log
+
+
+def test_random_pipelines_through_the_emulated_entries(emu):
+    """Random texts (tiny alphabets, long repeats, runs of one symbol, zero tails), 1 to 40 partitions, all four key widths,
+    through the device-buffer entries and the slab-shaped ones: every step passes the reference's validators inside the
+    harness and the suffix array is the oracle's."""
+    import multi_partition
+    rng = np.random.default_rng(2024)
+    for case in range(16):
+        n = int(rng.integers(40, 1400))
+        sigma = int(rng.choice([1, 2, 3, 5, 40, 65536]))
+        T = rng.integers(0, sigma, n).astype(np.uint16)
+        shape = case % 4
+        if shape == 1 and n > 200:
+            length = int(rng.integers(10, n // 2))
+            T[n - length:] = T[:length]
+        if shape == 2:
+            T[-int(rng.integers(1, 30)):] = 0
+        if shape == 3 and n > 300:
+            a = int(rng.integers(0, n // 2))
+            T[a:a + n // 3] = T[a]
+        p = int(rng.choice([1, 2, 3, 7, 16, 40]))
+        key_words = 1 + case % 4
+        kw = {"step_handle": steps_handle(emu, key_words)} if (case // 4) % 2 == 0 else {
+            "slab_handle": steps_handle(emu, key_words), "host_buf": lambda nbytes: np.zeros(nbytes, dtype=np.uint8), "chunk_cap": 4096}
+        sa, _ = multi_partition.build_sa(emu, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, p, key_words=key_words, seed=case, **kw)
+        want, _ = oracle_lib.prefix_doubling(T, 1)
+        assert np.array_equal(sa, want), (case, n, sigma, p, key_words)
 
 
 @pytest.mark.skipif(not os.path.exists(oracle_lib.SA_STRUCTURE), reason="oracle/_ref/sa_structure is not built (make -C oracle, with the reference tree present)")
