@@ -14,13 +14,11 @@ import texts
 from cascade_amd import _native
 
 EMU_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpu_emu")
-EMU_LIB = os.path.join(EMU_DIR, "libcascade_emu.so")
 
 
-@pytest.fixture(scope="module")
-def emu():
-    subprocess.run(["make", "-C", EMU_DIR, "libcascade_emu.so"], check=True, capture_output=True)
-    lib = C.CDLL(EMU_LIB)
+def load_emulation(target):
+    subprocess.run(["make", "-C", EMU_DIR, target], check=True, capture_output=True)
+    lib = C.CDLL(os.path.join(EMU_DIR, target))
     vp, u64, u32, i32 = C.c_void_p, C.c_uint64, C.c_uint32, C.c_int
     lib.csa_create.argtypes = [u64, i32, C.POINTER(vp)]
     lib.csa_destroy.argtypes = [vp]
@@ -50,6 +48,18 @@ def emu():
     lib.csa_last_step_result.argtypes = [vp, C.POINTER(_native.CsaStepResult)]
     lib.csa_set_tuning.argtypes = [vp, i32, u32]
     return lib
+
+
+@pytest.fixture(scope="module")
+def emu():
+    """The kernels with small tiles and low thresholds, so that texts of a few thousand symbols reach every path."""
+    return load_emulation("libcascade_emu.so")
+
+
+@pytest.fixture(scope="module")
+def emu_dev():
+    """The kernels with the tile sizes and thresholds of the device build."""
+    return load_emulation("libcascade_emu_dev.so")
 
 
 def steps_handle(lib, key_words):
@@ -98,6 +108,32 @@ def test_fixtures_through_the_emulated_kernels(emu, key_words):
         assert np.array_equal(got, oracle_lib.build_sa40(T)), name
         _, counts = oracle_lib.prefix_doubling(T, key_words)
         assert active == counts, name
+
+
+@pytest.mark.parametrize("n,sigma,key_words,pack", [(70000, 3, 1, True), (50000, 300, 1, False), (40000, 2, 2, False)])
+def test_the_device_builds_tile_sizes_in_the_emulation(emu_dev, n, sigma, key_words, pack):
+    """The same sources compiled with the device build's own constants (1024-thread workgroups, tiles of 16384 pairs, 2048
+    members per small-group tile): texts of several tiles with a long repeat and a zero tail."""
+    T = texts.random_text(n, sigma, n + sigma, sep_every=0)
+    T[n // 3:n // 3 + n // 5] = T[:n // 5]
+    T[-9:] = 0
+    got, active, _ = emu_sort(emu_dev, T, key_words, pack=pack)
+    assert np.array_equal(got, oracle_lib.build_sa40(T))
+    _, counts = oracle_lib.prefix_doubling(T, key_words)
+    assert active == counts
+
+
+def test_a_pipeline_at_the_device_builds_tile_sizes(emu_dev):
+    """Partition ids, slab staging, the two partition steps with their messages and the final scatter at the device build's
+    tile sizes: 30000 suffixes in 5 partitions."""
+    import multi_partition
+    T = texts.random_text(30000, 4, 5, sep_every=0)
+    T[12000:17000] = T[1000:6000]
+    T[-6:] = 0
+    sa, gens = multi_partition.build_sa(emu_dev, lambda a: HostArray(np.array(a, copy=True)), lambda d: d.a, T, 5, key_words=1,
+                                        step_handle=steps_handle(emu_dev, 1))
+    want, _ = oracle_lib.prefix_doubling(T, 1)
+    assert np.array_equal(sa, want) and gens >= 5
 
 
 def test_random_texts_through_the_emulated_sort(emu):
