@@ -136,6 +136,17 @@ def test_a_pipeline_at_the_device_builds_tile_sizes(emu_dev):
     assert np.array_equal(sa, want) and gens >= 5
 
 
+def test_results_do_not_depend_on_the_order_of_the_workgroups():
+    """The emulation runs the workgroups of a launch one after the other, by blockIdx; HIPEMU_REVERSE=1 runs them from the
+    last to the first (a process-wide switch, hence a process of its own): tiles numbered by arrival, look-back chains and
+    atomically reserved ranges must give the same results either way."""
+    import sys
+    env = dict(os.environ, HIPEMU_REVERSE="1")
+    chosen = "fixtures_through or random_texts_through or random_pipelines_through or emulated_message_kernels or partition_ids_match"
+    run = subprocess.run([sys.executable, "-m", "pytest", os.path.abspath(__file__), "-x", "-q", "-k", chosen], env=env, capture_output=True, text=True)
+    assert run.returncode == 0, run.stdout[-2000:] + run.stderr[-2000:]
+
+
 def test_random_texts_through_the_emulated_sort(emu):
     """Random alphabets (1 to 65536 symbols), structures (plain, a long repeat, a zero tail, a run of one symbol, a period),
     key widths and tuning knobs (packed first sort on and off, the speculative gather): the suffix array and every
