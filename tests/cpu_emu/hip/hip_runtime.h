@@ -122,15 +122,28 @@ inline void enter(Fiber& f)
     wave = &run->waves[f.t / 64];
 }
 
+// HIPEMU_LANES_REVERSE=1 hands over from a fiber to the one before it instead of the one after it (and starts with the
+// last): what one thread writes and another reads between two barriers without an order of their own shows up under one
+// of the two directions.
+inline bool lanes_reverse()
+{
+    static const bool reverse = std::getenv("HIPEMU_LANES_REVERSE") != nullptr;
+    return reverse;
+}
+inline unsigned next_fiber(const Run& r, unsigned n)
+{
+    do
+        n = lanes_reverse() ? (n == 0 ? (unsigned)r.fibers.size() - 1 : n - 1) : (n + 1 == r.fibers.size() ? 0 : n + 1);
+    while (r.fibers[n].done);
+    return n;
+}
+
 // hands over to the next fiber that has not finished; returns when this one is resumed
 inline void yield()
 {
     Run& r = *run;
     Fiber& me = r.fibers[r.current];
-    unsigned n = me.t;
-    do
-        n = n + 1 == r.fibers.size() ? 0 : n + 1;
-    while (r.fibers[n].done);
+    const unsigned n = next_fiber(r, me.t);
     if (n == me.t)
         return; // alone: whatever it waits for will not come from a switch
     enter(r.fibers[n]);
@@ -168,10 +181,7 @@ inline void fiber_main()
     if (--r.live == 0) {
         hipemu_switch(&unused, r.main_sp);
     } else {
-        unsigned n = me.t;
-        do
-            n = n + 1 == r.fibers.size() ? 0 : n + 1;
-        while (r.fibers[n].done);
+        const unsigned n = next_fiber(r, me.t);
         enter(r.fibers[n]);
         hipemu_switch(&unused, r.fibers[n].sp);
     }
@@ -212,8 +222,9 @@ inline void hipemu::launch(dim3 grid, dim3 blk, size_t shmem, const std::functio
     launch_grid = grid;
     const dim3 saved_thread = threadIdx, saved_block = blockIdx;
     run = &r;
-    enter(r.fibers[0]);
-    hipemu_switch(&r.main_sp, r.fibers[0].sp);
+    Fiber& first = r.fibers[lanes_reverse() ? B - 1 : 0];
+    enter(first);
+    hipemu_switch(&r.main_sp, first.sp);
     run = nullptr;
     threadIdx = saved_thread;
     blockIdx = saved_block;

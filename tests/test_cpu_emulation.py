@@ -136,13 +136,17 @@ def test_a_pipeline_at_the_device_builds_tile_sizes(emu_dev):
     assert np.array_equal(sa, want) and gens >= 5
 
 
-def test_results_do_not_depend_on_the_order_of_the_workgroups():
-    """The emulation runs the workgroups of a launch one after the other, by blockIdx; HIPEMU_REVERSE=1 runs them from the
-    last to the first (a process-wide switch, hence a process of its own): tiles numbered by arrival, look-back chains and
-    atomically reserved ranges must give the same results either way."""
+@pytest.mark.parametrize("switch", ["HIPEMU_REVERSE", "HIPEMU_LANES_REVERSE"])
+def test_results_do_not_depend_on_the_order_of_workgroups_and_lanes(switch):
+    """The emulation runs the workgroups of a launch one after the other, by blockIdx, and the lanes of a workgroup as fibers
+    that hand over to the next lane at a barrier. HIPEMU_REVERSE=1 runs the workgroups from the last to the first: tiles
+    numbered by arrival, look-back chains and atomically reserved ranges must give the same results. HIPEMU_LANES_REVERSE=1
+    hands over to the lane before instead: a value that one lane writes and another reads between two barriers, without an
+    order of their own, would show under one of the two directions. (Process-wide switches, hence a process of its own.)"""
     import sys
-    env = dict(os.environ, HIPEMU_REVERSE="1")
-    chosen = "fixtures_through or random_texts_through or random_pipelines_through or emulated_message_kernels or partition_ids_match"
+    env = dict(os.environ, **{switch: "1"})
+    chosen = ("fixtures_through or random_texts_through or random_pipelines_through or emulated_message_kernels or partition_ids_match "
+              "or slab_staging or three_and_four_words")
     run = subprocess.run([sys.executable, "-m", "pytest", os.path.abspath(__file__), "-x", "-q", "-k", chosen], env=env, capture_output=True, text=True)
     assert run.returncode == 0, run.stdout[-2000:] + run.stderr[-2000:]
 
