@@ -1,4 +1,4 @@
-// Stand-alone driver of the CPU-emulated kernels, for sanitizer runs (ASan / TSan need an instrumented main):
+// Stand-alone driver of the CPU-emulated kernels, for sanitizer runs (AddressSanitizer needs an instrumented main):
 //   emu_main <n> <sigma> <seed> [key_words]
 // Sorts a random text through the emulated library and compares with the CPU oracle. Test infrastructure only.
 #include "../../include/cascade_hip.h"
