@@ -1130,6 +1130,8 @@ __global__ __launch_bounds__(BLOCK) void place_presorted_kernel(PresortedArgs a)
     u32 g[ITEMS], gs[ITEMS], src[ITEMS], sec[ITEMS];
     u32 big = 0, heads = 0; // one bit per item
     u32 lh = 0;             // last run head among this thread's places, as place + 1
+    u32 cur_gs = 0, cur_ge = 0;
+    bool cur_mirrored = false;
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         const u64 p = base + k;
@@ -1141,8 +1143,15 @@ __global__ __launch_bounds__(BLOCK) void place_presorted_kernel(PresortedArgs a)
             atomicExch(a.err, DEV_ERR_SMALLSORT_TABLES);
             continue;
         }
-        gs[k] = a.gstart[g[k]];
-        const u32 ge = a.gstart[g[k] + 1];
+        // neighbouring places mostly lie in one group: its tables are looked up once per thread, not once per place
+        // (four dependent loads each time)
+        const bool same_group = k > 0 && (big & (1u << (k - 1))) && g[k - 1] == g[k];
+        if (!same_group) {
+            cur_gs = a.gstart[g[k]];
+            cur_ge = a.gstart[g[k] + 1];
+        }
+        gs[k] = cur_gs;
+        const u32 ge = cur_ge;
         if (!(gs[k] <= p && p < ge && ge <= a.m)) {
             atomicExch(a.err, DEV_ERR_SMALLSORT_TABLES);
             continue;
@@ -1150,7 +1159,9 @@ __global__ __launch_bounds__(BLOCK) void place_presorted_kernel(PresortedArgs a)
         if (ge - gs[k] <= a.maxg)
             continue; // a small group: the small-group kernel has placed it
         big |= 1u << k;
-        const bool mirrored = a.not_asc[a.big_first[g[k]] / a.maxg] != 0;
+        if (!same_group)
+            cur_mirrored = a.not_asc[a.big_first[g[k]] / a.maxg] != 0;
+        const bool mirrored = cur_mirrored;
         src[k] = mirrored ? gs[k] + (ge - 1u - (u32)p) : (u32)p;
         sec[k] = a.big_sec[src[k]];
         bool head = p == gs[k];
