@@ -1130,44 +1130,54 @@ __global__ __launch_bounds__(BLOCK) void place_presorted_kernel(PresortedArgs a)
     u32 g[ITEMS], gs[ITEMS], src[ITEMS], sec[ITEMS];
     u32 big = 0, heads = 0; // one bit per item
     u32 lh = 0;             // last run head among this thread's places, as place + 1
-    u32 cur_gs = 0, cur_ge = 0;
-    bool cur_mirrored = false;
+    // The loads of a thread's places are issued in rounds (group ids, then the groups' tables, then the gathered ranks)
+    // rather than place after place: the four chains of dependent loads run side by side.
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         const u64 p = base + k;
-        g[k] = gs[k] = src[k] = sec[k] = 0;
+        gs[k] = src[k] = sec[k] = 0;
+        g[k] = p < a.m ? a.gids[p] : 0xFFFFFFFFu;
+    }
+    // neighbouring places mostly lie in one group: its tables are looked up once per thread, not once per place
+    u32 ge[ITEMS];
+    bool mirrored[ITEMS];
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const u64 p = base + k;
+        ge[k] = 0;
+        mirrored[k] = false;
         if (p >= a.m)
             continue;
-        g[k] = a.gids[p];
         if (g[k] >= a.groups) {
             atomicExch(a.err, DEV_ERR_SMALLSORT_TABLES);
             continue;
         }
-        // neighbouring places mostly lie in one group: its tables are looked up once per thread, not once per place
-        // (four dependent loads each time)
         const bool same_group = k > 0 && (big & (1u << (k - 1))) && g[k - 1] == g[k];
-        if (!same_group) {
-            cur_gs = a.gstart[g[k]];
-            cur_ge = a.gstart[g[k] + 1];
-        }
-        gs[k] = cur_gs;
-        const u32 ge = cur_ge;
-        if (!(gs[k] <= p && p < ge && ge <= a.m)) {
+        gs[k] = same_group ? gs[k - 1] : a.gstart[g[k]];
+        ge[k] = same_group ? ge[k - 1] : a.gstart[g[k] + 1];
+        if (!(gs[k] <= p && p < ge[k] && ge[k] <= a.m)) {
             atomicExch(a.err, DEV_ERR_SMALLSORT_TABLES);
             continue;
         }
-        if (ge - gs[k] <= a.maxg)
+        if (ge[k] - gs[k] <= a.maxg)
             continue; // a small group: the small-group kernel has placed it
         big |= 1u << k;
-        if (!same_group)
-            cur_mirrored = a.not_asc[a.big_first[g[k]] / a.maxg] != 0;
-        const bool mirrored = cur_mirrored;
-        src[k] = mirrored ? gs[k] + (ge - 1u - (u32)p) : (u32)p;
-        sec[k] = a.big_sec[src[k]];
+        mirrored[k] = same_group ? mirrored[k - 1] : a.not_asc[a.big_first[g[k]] / a.maxg] != 0;
+        src[k] = mirrored[k] ? gs[k] + (ge[k] - 1u - (u32)p) : (u32)p;
+    }
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k)
+        if (big & (1u << k))
+            sec[k] = a.big_sec[src[k]];
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const u64 p = base + k;
+        if (!(big & (1u << k)))
+            continue;
         bool head = p == gs[k];
         if (!head) { // the member at the place before this one, in the same order
             const u32 before = (k > 0 && (big & (1u << (k - 1))) && g[k - 1] == g[k]) ? sec[k - 1]
-                                                                                     : a.big_sec[mirrored ? src[k] + 1u : src[k] - 1u];
+                                                                                     : a.big_sec[mirrored[k] ? src[k] + 1u : src[k] - 1u];
             head = before != sec[k];
         }
         if (head) {
